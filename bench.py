@@ -1,0 +1,398 @@
+"""Benchmark of the policy-loss hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c1|c5]
+
+Prints ONE JSON line.  A "step" is one pass of the hot path (forward + backward) over one batch of
+synthetic inputs that already live in HBM.  Workloads are the BASELINE configs:
+
+  c3 (default, the headline metric): fused lm_head + logprob + entropy + GRPO loss, fwd + bwd, at
+      Llama-3.1-8B shape: hidden bf16 [32768, 4096], W bf16 [128256, 4096], 70 % response tokens.
+  c2: GRPO loss on materialised bf16 logits [64, 1024, 128256], fwd + bwd (HBM-bound).
+  c1: logprob + entropy + masked_mean on fp32 logits [4, 512, 32000], forward only.
+  c5: DPO at Llama-3.1-70B head shape: hidden [32768, 8192], W [128256, 8192], bwd to dHidden only.
+
+`roofline` describes the dominant kernel of the workload, timed with HIP events on the stream it
+runs on inside the timed region; `cpu_baseline` is the oracle's restatement of the reference's
+PyTorch path on a bounded sample of the same workload, on this machine's host cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+import types
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0
+PEAK_BF16_TFLOPS = 2500.0
+
+
+def _cfg():
+    return types.SimpleNamespace(loss_fn="dapo", clip_lower=0.2, clip_higher=0.28, beta=0.05, kl_estimator=2)
+
+
+class EventTimer:
+    """Accumulates the duration of one region per step with HIP events on the current stream."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.pairs = []
+
+    def __enter__(self):
+        self.a = self.torch.cuda.Event(enable_timing=True)
+        self.b = self.torch.cuda.Event(enable_timing=True)
+        self.a.record()
+        return self
+
+    def __exit__(self, *exc):
+        self.b.record()
+        self.pairs.append((self.a, self.b))
+
+    def mean_ms(self):
+        return sum(a.elapsed_time(b) for a, b in self.pairs) / max(1, len(self.pairs))
+
+    def reset(self):
+        self.pairs = []
+
+
+# ------------------------------------------------------------------------------------------------
+# workloads
+# ------------------------------------------------------------------------------------------------
+def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False):
+    dev = "cuda:0"
+    torch.manual_seed(0)
+    hidden = torch.randn(n_tokens, hdim, device=dev).bfloat16().requires_grad_(True)
+    weight = (torch.randn(vocab, hdim, device=dev) * w_std).bfloat16().requires_grad_(not dpo)
+    labels = torch.randint(0, vocab, (n_tokens,), device=dev)
+    cfg = _cfg()
+    if not dpo:
+        mask = torch.rand(n_tokens, device=dev) < 0.7
+        adv = torch.randn(n_tokens, device=dev)
+        with torch.no_grad():
+            lp0, _ = oi.fused_lm_head_logprobs(hidden, weight, labels, mask=mask)
+        old = lp0 + 0.05 * torch.randn(n_tokens, device=dev)
+        ref = lp0 + 0.1 * torch.randn(n_tokens, device=dev)
+        n_eff = int(mask.sum().item())
+    else:
+        # 16 sequences of 2048 tokens, prompt (128..1024 tokens) masked out with -100 labels
+        seqs, per = n_tokens // 2048, 2048
+        prompt = torch.randint(128, 1025, (seqs,), device=dev)
+        pos = torch.arange(per, device=dev).unsqueeze(0).expand(seqs, per)
+        lab2 = labels.view(seqs, per).clone()
+        lab2[pos < prompt.unsqueeze(1)] = -100
+        labels = lab2.view(1, -1)
+        cu = torch.arange(0, n_tokens + 1, per, device=dev, dtype=torch.int32)
+        shifted = oi.padding_free_collator.shift_labels(labels)
+        mask = (shifted != -100).view(-1)
+        ref_c = torch.randn(seqs // 2, device=dev) * 50 - 400
+        ref_r = torch.randn(seqs // 2, device=dev) * 50 - 400
+        n_eff = int(mask.sum().item())
+    fwd_timer = EventTimer(torch)
+
+    def step():
+        hidden.grad = None
+        weight.grad = None
+        if not dpo:
+            with fwd_timer:
+                lp, ent = oi.fused_lm_head_logprobs(hidden, weight, labels, mask=mask, return_entropy=True)
+            loss, _ = oi.grpo_utils.grpo_loss_fused(
+                lp[None], old[None], ref[None], adv[None], mask[None], cfg, entropy=ent[None]
+            )
+        else:
+            with fwd_timer:
+                lp, _ = oi.fused_lm_head_logprobs(hidden, weight, shifted.view(-1), mask=mask)
+            logps = oi.padding_free_collator.get_batch_logps(lp.view(1, -1), labels, cu)
+            bs = logps.shape[0] // 2
+            losses, _, _ = oi.dpo_utils.dpo_loss(logps[:bs], logps[bs:], ref_c, ref_r, beta=0.1)
+            loss = losses.mean()
+        loss.backward()
+        return loss
+
+    flops_fwd = 2.0 * n_eff * hdim * vocab
+    info = {
+        "tokens": n_tokens,
+        "rows_multiplied": n_eff,
+        "flops_step": (2.0 if dpo else 3.0) * flops_fwd,
+        "kernel": "lmhead_fwd_kernel (fused lm_head forward: MFMA tiles + online softmax statistics)",
+        "alg_per_launch": flops_fwd,
+        "bound": "mfma",
+        "timer": fwd_timer,
+    }
+    return step, info
+
+
+def make_c2(torch, oi, rows_b=64, t=1024, vocab=128256):
+    dev = "cuda:0"
+    torch.manual_seed(0)
+    logits = torch.empty(rows_b, t, vocab, device=dev, dtype=torch.bfloat16)
+    for b in range(rows_b):  # generated per row block to bound the fp32 temporary
+        logits[b] = (torch.randn(t, vocab, device=dev) * 3.0).bfloat16()
+    logits.requires_grad_(True)
+    labels = torch.randint(0, vocab, (rows_b, t), device=dev)
+    rewards = (torch.rand(rows_b, device=dev) < 0.3).double()
+    adv = oi.grpo_utils.group_advantages(rewards, 8).unsqueeze(1).expand(rows_b, t).contiguous()
+    mask = torch.ones(rows_b, t, dtype=torch.bool, device=dev)
+    with torch.no_grad():
+        lp0 = oi.model_utils.log_softmax_and_gather(logits, labels)
+    old = lp0 + 0.05 * torch.randn(rows_b, t, device=dev)
+    ref = lp0 + 0.1 * torch.randn(rows_b, t, device=dev)
+    cfg = _cfg()
+    fwd_timer = EventTimer(torch)
+
+    def step():
+        logits.grad = None
+        with fwd_timer:
+            lp = oi.model_utils.log_softmax_and_gather(logits, labels)
+        loss, _ = oi.grpo_utils.grpo_loss_fused(lp, old, ref, adv, mask, cfg)
+        loss.backward()
+        return loss
+
+    n = rows_b * t
+    info = {
+        "tokens": n,
+        "rows_multiplied": n,
+        "bytes_step": 3.0 * n * vocab * 2,
+        "kernel": "lsg_entropy_fwd_kernel (row-wise log-softmax gather, one read of the logits)",
+        "alg_per_launch": 1.0 * n * vocab * 2,
+        "bound": "hbm",
+        "timer": fwd_timer,
+    }
+    return step, info
+
+
+def make_c1(torch, oi):
+    dev = "cuda:0"
+    torch.manual_seed(0)
+    logits = (torch.randn(4, 512, 32000) * 2.0).to(dev)
+    ids = torch.randint(0, 32000, (4, 512)).to(dev)
+    length = torch.randint(64, 513, (4,))
+    mask = (torch.arange(512).unsqueeze(0) >= (512 - length).unsqueeze(1)).to(dev)
+    timer = EventTimer(torch)
+
+    def step():
+        with timer:
+            lp, ent = oi.model_utils.logprob_and_entropy(logits, ids)
+        return oi.rl_utils.masked_mean(lp, mask) + oi.rl_utils.masked_mean(ent, mask)
+
+    n = 2048
+    info = {
+        "tokens": n,
+        "rows_multiplied": n,
+        "bytes_step": 1.0 * n * 32000 * 4,
+        "kernel": "lsg_entropy_fwd_kernel (fp32 rows, logprob + entropy in one pass)",
+        "alg_per_launch": 1.0 * n * 32000 * 4,
+        "bound": "hbm",
+        "timer": timer,
+    }
+    return step, info
+
+
+# ------------------------------------------------------------------------------------------------
+# CPU baseline: the oracle's restatement of the reference path on a bounded sample
+# ------------------------------------------------------------------------------------------------
+def cpu_baseline(torch, workload):
+    from oracle import grpo as o_grpo
+    from oracle import logprob as o_lp
+    from oracle import reductions as o_red
+
+    threads = torch.get_num_threads()
+    cfg = _cfg()
+    torch.manual_seed(0)
+    if workload in ("c3", "c5"):
+        hdim = 4096 if workload == "c3" else 8192
+        vocab, n = 128256, 256
+        hidden = torch.randn(n, hdim).bfloat16().requires_grad_(True)
+        weight = (torch.randn(vocab, hdim) * 0.02).bfloat16().requires_grad_(workload == "c3")
+        labels = torch.randint(0, vocab, (n,))
+        mask = torch.rand(n) < 0.7
+        adv, noise = torch.randn(n), torch.randn(n)
+
+        def run():
+            hidden.grad = None
+            weight.grad = None
+            # reference order: bf16 lm_head GEMM, fp32 upcast, log_softmax + gather, entropy (no grad)
+            z = torch.nn.functional.linear(hidden, weight)
+            lp = o_lp.log_softmax_and_gather(z, labels, torch.float32)
+            with torch.no_grad():
+                o_lp.entropy_from_logits(z, torch.float32)
+            old, ref = lp.detach() + 0.05 * noise, lp.detach() + 0.1 * noise
+            loss, *_ = o_grpo.grpo_token_loss(lp[None], old[None], ref[None], adv[None], mask[None], cfg)
+            loss.backward()
+
+        sample = f"{n} of 32768 token rows at full H={hdim}, V={vocab}; fwd+bwd; bf16 GEMM + fp32 log_softmax"
+    elif workload == "c2":
+        n, vocab = 512, 128256
+        logits = (torch.randn(n, vocab) * 3.0).bfloat16().requires_grad_(True)
+        labels = torch.randint(0, vocab, (n,))
+        adv, noise = torch.randn(n), torch.randn(n)
+        mask = torch.ones(n, dtype=torch.bool)
+
+        def run():
+            logits.grad = None
+            lp = o_lp.log_softmax_and_gather(logits, labels, None).float()  # bf16 log_softmax as the reference
+            old, ref = lp.detach() + 0.05 * noise, lp.detach() + 0.1 * noise
+            loss, *_ = o_grpo.grpo_token_loss(lp[None], old[None], ref[None], adv[None], mask[None], cfg)
+            loss.backward()
+
+        sample = f"{n} of 65536 rows of bf16 logits at V={vocab}; fwd+bwd"
+    else:
+        n = 2048
+        logits = torch.randn(4, 512, 32000) * 2.0
+        ids = torch.randint(0, 32000, (4, 512))
+        mask = torch.ones(4, 512)
+
+        def run():
+            lp = o_lp.log_softmax_and_gather(logits, ids, None)
+            ent = o_lp.entropy_from_logits(logits, None)
+            o_red.masked_mean(lp, mask) + o_red.masked_mean(ent, mask)
+
+        sample = "the full config-1 batch (2048 rows, V=32000, fp32)"
+    run()  # warm-up
+    times = []
+    t_end = time.time() + 20.0
+    while len(times) < 3 or (time.time() < t_end and len(times) < 5):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": n / med,
+        "unit": "tokens/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": sample + f"; median of {len(times)} runs, {med:.3f} s each, torch CPU threads={threads}",
+    }
+
+
+def library_gemm_tflops(torch, n, hdim, vocab):
+    """bf16 GEMM ceiling of the vendor library at the forward's shape (reported next to the peak)."""
+    a = torch.randn(min(n, 8192), hdim, device="cuda:0").bfloat16()
+    w = (torch.randn(vocab, hdim, device="cuda:0") * 0.02).bfloat16()
+    out = torch.empty(a.shape[0], vocab, device="cuda:0", dtype=torch.bfloat16)
+    for _ in range(2):
+        torch.matmul(a, w.t(), out=out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    reps = 5
+    for _ in range(reps):
+        torch.matmul(a, w.t(), out=out)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / reps
+    return 2.0 * a.shape[0] * hdim * vocab / dt / 1e12
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-library-gemm", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures the one-GPU hot path only: run it with --gpus 1 (no multi-GPU figure exists).")
+        sys.exit(2)
+
+    import torch
+
+    import open_instruct_amd as oi
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the package has no CPU path).")
+        sys.exit(2)
+    oi._lib.load()
+
+    if args.workload == "c3":
+        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02)
+        name = "c3: fused lm_head+logprob+entropy+GRPO loss fwd+bwd, hidden bf16 [32768,4096], W bf16 [128256,4096], 70% response tokens (rows compacted)"
+        dtype = "bf16"
+    elif args.workload == "c5":
+        step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True)
+        name = "c5: fused lm_head+per-sequence logprob sums+sigmoid DPO loss, hidden bf16 [32768,8192], W bf16 [128256,8192], bwd to dHidden only"
+        dtype = "bf16"
+    elif args.workload == "c2":
+        step, info = make_c2(torch, oi)
+        name = "c2: GRPO loss on materialised bf16 logits [64,1024,128256], fwd+bwd"
+        dtype = "bf16"
+    else:
+        step, info = make_c1(torch, oi)
+        name = "c1: logprob+entropy+masked_mean on fp32 logits [4,512,32000], forward"
+        dtype = "f32"
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    info["timer"].reset()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = info["tokens"] / (elapsed / args.steps)
+
+    kernel_ms = info["timer"].mean_ms()
+    if info["bound"] == "mfma":
+        achieved = info["alg_per_launch"] / (kernel_ms * 1e-3) / 1e12
+        peak, unit = PEAK_BF16_TFLOPS, "TFLOP/s"
+    else:
+        achieved = info["alg_per_launch"] / (kernel_ms * 1e-3) / 1e9
+        peak, unit = PEAK_HBM_GBS, "GB/s"
+    roofline = {
+        "bound": info["bound"],
+        "achieved": achieved,
+        "peak": peak,
+        "unit": unit,
+        "frac": achieved / peak,
+        "traffic": None,
+        "kernel": info["kernel"],
+        "kernel_ms": kernel_ms,
+        "algorithmic_per_launch": info["alg_per_launch"],
+    }
+    if "flops_step" in info:
+        roofline["whole_step_tflops"] = info["flops_step"] / (ms_per_step * 1e-3) / 1e12
+        roofline["whole_step_frac"] = roofline["whole_step_tflops"] / PEAK_BF16_TFLOPS
+        if not args.no_library_gemm:
+            hdim = 8192 if args.workload == "c5" else 4096
+            roofline["library_bf16_gemm_tflops"] = library_gemm_tflops(torch, 32768, hdim, 128256)
+    if "bytes_step" in info:
+        roofline["whole_step_gbs"] = info["bytes_step"] / (ms_per_step * 1e-3) / 1e9
+        roofline["whole_step_frac"] = roofline["whole_step_gbs"] / PEAK_HBM_GBS
+
+    line = {
+        "metric": "tokens/s fused lm_head+logprob+GRPO loss fwd+bwd, V=128k; % MFMA/HBM peak",
+        "value": value,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype,
+        "data": "synthetic",
+        "config": {
+            "workload": name,
+            "tokens_per_step": info["tokens"],
+            "rows_multiplied": info["rows_multiplied"],
+            "loss_value": float(loss.item()) if math.isfinite(float(loss.item())) else None,
+        },
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(torch, args.workload)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,246 @@
+/*
+ * C-ABI of the MI355X (gfx950) policy-loss kernels.
+ *
+ * The reference (allenai/open-instruct) has no native interface for this path: its boundary is
+ * plain Python functions on torch tensors.  Each entry point below names the reference function
+ * whose arithmetic it carries; the Python package binds them with ctypes and exposes the
+ * reference's own names and signatures on top.
+ *
+ * Conventions
+ *  - Every pointer is DEVICE memory owned by the caller.  The library never allocates, frees or
+ *    keeps a pointer after the call returns.  Scratch memory is passed in as `workspace` and sized
+ *    by the matching oi_*_workspace_bytes().
+ *  - Work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the null stream) and the
+ *    call returns without waiting for it.
+ *  - Return value: 0 on success, a negative OI_E* code for a rejected argument (nothing was
+ *    launched), a positive value = the hipError_t of a failed launch.
+ *  - The library keeps no mutable global state; calls are re-entrant.
+ *  - Row-major everywhere; strides are in ELEMENTS, not bytes.
+ *  - Token ids / labels are int64, sequence boundaries int32, masks one byte per token (0 / 1).
+ */
+#ifndef OI_KERNELS_H
+#define OI_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OI_OK 0
+#define OI_EINVAL (-1)     /* a size or scalar argument is out of range            */
+#define OI_ENULL (-2)      /* a required pointer is NULL                            */
+#define OI_EALIGN (-3)     /* pointer/stride alignment the kernel needs is not met  */
+#define OI_EDTYPE (-4)     /* unknown or unsupported dtype tag                      */
+#define OI_EWORKSPACE (-5) /* workspace_bytes is smaller than the op needs          */
+
+#define OI_DTYPE_F32 0
+#define OI_DTYPE_BF16 1
+#define OI_DTYPE_F16 2
+
+#define OI_LOSS_DAPO 0
+#define OI_LOSS_CISPO 1
+
+/* Library ABI version (major * 1000 + minor). */
+int oi_version(void);
+/* Human-readable text for a negative OI_E* code (static storage). */
+const char* oi_error_string(int code);
+
+/* ------------------------------------------------------------------------------------------
+ * Row-wise log-softmax gather + entropy over materialised logits.
+ *
+ * Carries open_instruct/model_utils.py:587-600 (log_softmax_and_gather),
+ * open_instruct/model_utils.py:326-333 (entropy_from_logits) and, with the label clamp done by
+ * the caller, open_instruct/padding_free_collator.py:10-16 (calculate_per_token_logps).  The
+ * division by temperature of open_instruct/grpo_utils.py:560 is folded in as `inv_temperature`.
+ *
+ * Rows are addressed as row = o * n_inner + i  ->  logits + o * stride_outer + i * stride_inner,
+ * which covers the reference's non-contiguous `logits[:, :-1]` view (n_outer = B, n_inner = T-1,
+ * stride_outer = T*V, stride_inner = V).  The vocabulary dim has stride 1.
+ *
+ *   logprob[row] = z[index[row]] * inv_T - logsumexp(z * inv_T)
+ *   entropy[row] = logsumexp(z * inv_T) - sum_j softmax(z * inv_T)_j * z_j * inv_T   (optional)
+ *   lse[row]     = logsumexp(z * inv_T)                                              (optional)
+ *
+ * All three outputs are fp32, contiguous, n_outer * n_inner long.  index values outside [0, V)
+ * are clamped into range (never a fault).  One pass over the logits.
+ * ------------------------------------------------------------------------------------------ */
+int oi_lsg_entropy_fwd(const void* logits, int dtype, int64_t n_outer, int64_t n_inner, int64_t stride_outer,
+                       int64_t stride_inner, int64_t vocab, const int64_t* index, float inv_temperature,
+                       float* logprob, float* entropy, float* lse, void* stream);
+
+/*
+ * Backward of the gather-logprob above (autograd supplies it in the reference; formula
+ * d z_j = g * inv_T * (1[j == index] - softmax_j)).  Reads logits + lse, writes dlogits in the
+ * logits' dtype with its own outer/inner strides.  Rows whose grad_logprob is exactly 0 are
+ * written as zeros without reading their logits.  `dlogits` may alias `logits` (in-place) when
+ * the strides are equal.
+ */
+int oi_lsg_bwd(const void* logits, int dtype, int64_t n_outer, int64_t n_inner, int64_t stride_outer,
+               int64_t stride_inner, int64_t vocab, const int64_t* index, const float* lse,
+               const float* grad_logprob, float inv_temperature, void* dlogits, int64_t out_stride_outer,
+               int64_t out_stride_inner, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Per-token GRPO loss terms.  Carries open_instruct/grpo_utils.py:504-538 (compute_grpo_loss)
+ * with open_instruct/model_utils.py:793-818 (estimate_kl) for the selected estimator.
+ * All tensors fp32, contiguous, n elements.  ref_logprobs may be NULL (kl = 0).
+ * ratio_lo / ratio_hi are the clamp bounds themselves, i.e. 1 - clip_lower and 1 + clip_higher
+ * evaluated by the caller in double and rounded once to fp32, as torch does for a Python scalar.
+ * ------------------------------------------------------------------------------------------ */
+int oi_grpo_terms_fwd(const float* new_logprobs, const float* ratio, const float* advantages,
+                      const float* ref_logprobs, const float* rho_weights, int64_t n, int loss_fn, float ratio_lo,
+                      float ratio_hi, int kl_estimator, float* pg_loss, float* clipfrac, float* kl, void* stream);
+
+/* Backward of oi_grpo_terms_fwd towards new_logprobs and ratio (either output may be NULL).
+ * grad_pg / grad_kl are the upstream gradients of pg_loss / kl (either may be NULL = zeros). */
+int oi_grpo_terms_bwd(const float* new_logprobs, const float* ratio, const float* advantages,
+                      const float* ref_logprobs, const float* rho_weights, const float* grad_pg,
+                      const float* grad_kl, int64_t n, int loss_fn, float ratio_lo, float ratio_hi,
+                      int kl_estimator, float* d_new_logprobs, float* d_ratio, void* stream);
+
+/*
+ * Fused scalar GRPO loss over a [rows, cols] micro-batch.  Carries the loss assembly of
+ * open_instruct/grpo_fast.py:702-724 / open_instruct/olmo_core_train_modules.py:547-568:
+ *   ratio = exp(new - old); (pg, clipfrac, kl) as above;
+ *   loss  = masked_mean(pg + beta * kl, mask, axis, denominator) * scale
+ * together with the no-grad statistics of open_instruct/grpo_utils.py:699-729 in the same pass.
+ *
+ * axis_mode 0: masked_mean(axis=None) - one denominator (`denominator` if > 0, else mask.sum()).
+ * axis_mode 1: masked_mean(axis=1)    - per-row means, then the mean over rows.
+ * old_logprobs / ref_logprobs / rho_weights / entropy may be NULL (old NULL => ratio == 1 with
+ * gradient, as when old = new.detach(); ref NULL => kl = 0; rho NULL => 1).
+ *
+ * out_stats (fp32[OI_GRPO_NUM_STATS]): [0] loss, [1] masked mean pg, [2..5] masked mean of KL
+ * estimators 0..3, [6] masked mean clipfrac, [7] masked mean ratio, [8] masked mean entropy,
+ * [9] mask.sum().  row_denoms (fp32[rows]) receives the reciprocal denominator applied to each
+ * row's tokens, which oi_grpo_fused_bwd consumes.
+ */
+#define OI_GRPO_NUM_STATS 10
+size_t oi_grpo_fused_workspace_bytes(int64_t rows, int64_t cols);
+int oi_grpo_fused_fwd(const float* new_logprobs, const float* old_logprobs, const float* ref_logprobs,
+                      const float* advantages, const uint8_t* mask, const float* rho_weights, const float* entropy,
+                      int64_t rows, int64_t cols, int loss_fn, float ratio_lo, float ratio_hi, int kl_estimator,
+                      float beta, int axis_mode, float denominator, float scale, float* out_stats,
+                      float* row_denoms, void* workspace, size_t workspace_bytes, void* stream);
+/* d loss / d new_logprobs (fp32 [rows, cols]); grad_loss is a DEVICE scalar (upstream gradient). */
+int oi_grpo_fused_bwd(const float* new_logprobs, const float* old_logprobs, const float* ref_logprobs,
+                      const float* advantages, const uint8_t* mask, const float* rho_weights, int64_t rows,
+                      int64_t cols, int loss_fn, float ratio_lo, float ratio_hi, int kl_estimator, float beta,
+                      float scale, const float* row_denoms, const float* grad_loss, float* d_new_logprobs,
+                      void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Small per-token helpers of the GRPO step (fp32, contiguous).
+ * oi_estimate_kl_*: open_instruct/model_utils.py:793-818 - out is [4, n]: d, d^2/2,
+ *   expm1(-d)+d, ratio*d.  The backward takes grad_out [4, n]; d_diff / d_ratio may be NULL.
+ * oi_mask_logprobs_*: open_instruct/grpo_utils.py:340-344 - positions off the mask and NaNs
+ *   become `fill` (INVALID_LOGPROB = 1.0 in the reference, open_instruct/utils.py:83).
+ * oi_rho_correction: open_instruct/grpo_utils.py:372-463 - per token rho = exp(clamp(old - vllm,
+ *   +-10)) on the mask (1 elsewhere), optional per-row geometric mean / TV-divergence drop rule,
+ *   drop outside (mask_lower, mask_upper), clamp to [clamp_lower, clamp_upper] (a bound of 0
+ *   disables it); six fp32 [rows, cols] outputs: rho, weights, dropped, dropped-low,
+ *   dropped-high, clamped-flag.
+ * ------------------------------------------------------------------------------------------ */
+int oi_estimate_kl_fwd(const float* ref_logprobs_diff, const float* ratio, int64_t n, float* out, void* stream);
+int oi_estimate_kl_bwd(const float* ref_logprobs_diff, const float* ratio, const float* grad_out, int64_t n,
+                       float* d_diff, float* d_ratio, void* stream);
+int oi_mask_logprobs_fwd(const float* logprobs, const uint8_t* mask, int64_t n, float fill, float* out,
+                         void* stream);
+int oi_mask_logprobs_bwd(const float* logprobs, const uint8_t* mask, const float* grad_out, int64_t n,
+                         float* d_logprobs, void* stream);
+int oi_rho_correction(const float* old_logprobs, const float* vllm_logprobs, const uint8_t* mask,
+                      const float* advantages, int64_t rows, int64_t cols, int sequence_level, int tv_divergence,
+                      float mask_lower, float mask_upper, float clamp_lower, float clamp_upper, float* rho,
+                      float* weights, float* drop_any, float* drop_low, float* drop_high, float* clipped,
+                      void* stream);
+
+/* Group-normalised advantages.  Carries open_instruct/data_loader.py:1472-1484: population std,
+ * mode 0 "standard" (s - mean) / (std + 1e-8), mode 1 "centered" s - mean.  Computed in fp64 like
+ * the reference's numpy, stored as fp32.  scores: fp64 [n_groups * group_size]. */
+int oi_group_advantages(const double* scores, int64_t n_groups, int64_t group_size, int mode, float* advantages,
+                        void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Masked mean.  Carries open_instruct/rl_utils.py:426-448 for fp32 values [extra, rows, cols]
+ * and a byte or fp32 mask [rows, cols] (mask_is_float selects).  axis_mode as above;
+ * out: fp32 [extra].  row_denoms (fp32 [rows], may be NULL) as above.
+ * ------------------------------------------------------------------------------------------ */
+size_t oi_masked_mean_workspace_bytes(int64_t extra, int64_t rows, int64_t cols);
+int oi_masked_mean_fwd(const float* values, const void* mask, int mask_is_float, int64_t extra, int64_t rows,
+                       int64_t cols, int axis_mode, float denominator, float* out, float* row_denoms,
+                       void* workspace, size_t workspace_bytes, void* stream);
+/* d values[e, r, c] = grad_out[e] * mask[r, c] * row_denoms[r]. */
+int oi_masked_mean_bwd(const float* grad_out, const void* mask, int mask_is_float, const float* row_denoms,
+                       int64_t extra, int64_t rows, int64_t cols, float* d_values, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Per-sequence log-probability sums.
+ * Packed rows (cu_seq_lens != NULL): carries open_instruct/padding_free_collator.py:202-229 -
+ * per_token_logps / labels are one packed row of `total` positions, cu_seq_lens int32 [n_seqs+1];
+ * position t < total-1 is kept when labels[t+1] != -100 and belongs to the segment given by the
+ * boundaries shifted left by one (leading 0 kept, tail clamped into the last segment).
+ * Padded rows (cu_seq_lens == NULL): carries open_instruct/dpo_utils.py:689-712 - n_seqs rows of
+ * `total` positions each.  average != 0 divides by max(count, 1).
+ * out: fp32 [n_seqs]; counts: fp32 [n_seqs] (kept positions, may be NULL).  Deterministic.
+ * ------------------------------------------------------------------------------------------ */
+int oi_seq_logp_fwd(const float* per_token_logps, const int64_t* labels, const int32_t* cu_seq_lens, int64_t n_seqs,
+                    int64_t total, int average, float* out, float* counts, void* stream);
+/* d per_token_logps (same shape as the input; the dropped last position(s) get 0).  `counts` is
+ * the forward's output and is required when average != 0. */
+int oi_seq_logp_bwd(const float* grad_out, const int64_t* labels, const int32_t* cu_seq_lens, const float* counts,
+                    int64_t n_seqs, int64_t total, int average, float* d_per_token_logps, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Sigmoid preference loss per pair.  Carries open_instruct/dpo_utils.py:523-563 (dpo_loss) and,
+ * with ref pointers NULL and `margin` = gamma/beta, open_instruct/dpo_utils.py:617-642
+ * (simpo_loss):   x = (pc - pr) - (rc - rr) - margin
+ *                 loss = -(1 - ls) * logsigmoid(beta x) - ls * logsigmoid(-beta x)
+ * `weights` (may be NULL) multiplies the loss per pair (open_instruct/dpo_utils.py:566-613, wpo).
+ * rewards: beta * (p - ref) (ref treated as 0 when NULL); either may be NULL.
+ * ------------------------------------------------------------------------------------------ */
+int oi_dpo_sigmoid_fwd(const float* policy_chosen, const float* policy_rejected, const float* ref_chosen,
+                       const float* ref_rejected, const float* weights, int64_t n_pairs, float beta,
+                       float label_smoothing, float margin, float* losses, float* chosen_rewards,
+                       float* rejected_rewards, void* stream);
+int oi_dpo_sigmoid_bwd(const float* policy_chosen, const float* policy_rejected, const float* ref_chosen,
+                       const float* ref_rejected, const float* weights, const float* grad_losses, int64_t n_pairs,
+                       float beta, float label_smoothing, float margin, float* d_policy_chosen,
+                       float* d_policy_rejected, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Fused lm_head projection + per-token logprob / entropy, logits never materialised.
+ *
+ * Replaces the pair "lm_head GEMM -> calculate_per_token_logps" of
+ * open_instruct/olmo_core_train_modules.py:71-76 (DPOLMHead.forward) and
+ * open_instruct/grpo_utils.py:558-572 (forward_for_logprobs); no single reference function
+ * computes it.  hidden: bf16 [n_tokens, hidden_dim]; weight: bf16 [vocab, hidden_dim] (both
+ * row-major, 16-byte aligned, hidden_dim a multiple of 64); labels int64 [n_tokens], negative
+ * labels are scored as token 0 (clamp(min=0) at open_instruct/padding_free_collator.py:15).
+ *
+ *   z = hidden @ weight^T (bf16 MFMA, fp32 accumulate), logprob/entropy/lse as for oi_lsg_*.
+ * ------------------------------------------------------------------------------------------ */
+size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab);
+int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
+                       int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob, float* entropy,
+                       float* lse, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Backward: recomputes the logits tile by tile,
+ *   dZ[n, v] = grad_logprob[n] * inv_T * (1[v == label_n] - exp(z[n,v] * inv_T - lse[n])),
+ *   d_hidden = dZ @ weight   (bf16 [n_tokens, hidden_dim]),
+ *   d_weight = dZ^T @ hidden (bf16 [vocab, hidden_dim]; NULL skips it).
+ * Vocabulary is processed in chunks of `oi_lmhead_bwd_vocab_chunk()` columns; only one chunk of
+ * dZ (bf16) lives in the workspace at a time.
+ */
+size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int want_d_weight);
+int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
+                       const float* grad_logprob, int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
+                       float inv_temperature, void* d_hidden, void* d_weight, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OI_KERNELS_H */

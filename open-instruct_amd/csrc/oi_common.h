@@ -1,0 +1,87 @@
+// Shared device helpers for the gfx950 policy-loss kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "oi_kernels.h"
+
+#define OI_WAVE 64
+
+#define OI_LOG2E 1.4426950408889634f
+#define OI_LN2 0.6931471805599453f
+// Finite stand-in for -inf as the starting value of a running maximum: keeps (m_old - m_new)
+// finite so that exp2 of it is 1 and not NaN when nothing has been seen yet.
+#define OI_NEG_BIG (-3.0e38f)
+
+#define OI_RETURN_IF(cond, code) \
+    do {                         \
+        if (cond) return (code); \
+    } while (0)
+
+static inline int oi_launch_status() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? OI_OK : (int)e;
+}
+
+static inline bool oi_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+typedef uint32_t oi_u32x4 __attribute__((ext_vector_type(4)));
+typedef float oi_f32x4 __attribute__((ext_vector_type(4)));
+
+// ---- bf16 / f16 <-> f32 ------------------------------------------------------------------
+__device__ __forceinline__ float oi_bf16lo_to_f32(uint32_t packed) { return __uint_as_float(packed << 16); }
+__device__ __forceinline__ float oi_bf16hi_to_f32(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
+
+// round-to-nearest-even f32 -> bf16 bits (NaN kept quiet)
+__device__ __forceinline__ uint32_t oi_f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ uint32_t oi_pack_bf16x2(float lo, float hi) {
+    return oi_f32_to_bf16_bits(lo) | (oi_f32_to_bf16_bits(hi) << 16);
+}
+
+__device__ __forceinline__ float oi_f16bits_to_f32(uint16_t h) {
+    _Float16 v;
+    __builtin_memcpy(&v, &h, 2);
+    return (float)v;
+}
+__device__ __forceinline__ uint16_t oi_f32_to_f16bits(float f) {
+    _Float16 v = (_Float16)f;
+    uint16_t h;
+    __builtin_memcpy(&h, &v, 2);
+    return h;
+}
+
+// ---- wavefront (64 lanes) reductions -------------------------------------------------------
+__device__ __forceinline__ float oi_wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, OI_WAVE);
+    return v;
+}
+__device__ __forceinline__ double oi_wave_sum(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, OI_WAVE);
+    return v;
+}
+__device__ __forceinline__ float oi_wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, OI_WAVE));
+    return v;
+}
+
+// Block-wide sum for blockDim.x a multiple of 64, up to 1024 threads; `scratch` holds >= 16
+// floats.  Every thread gets the total; summation order is fixed (deterministic).
+__device__ __forceinline__ float oi_block_sum(float v, float* scratch) {
+    v = oi_wave_sum(v);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int w = 0; w < nw; ++w) t += scratch[w];
+    return t;
+}

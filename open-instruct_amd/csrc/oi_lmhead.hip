@@ -1,0 +1,567 @@
+// Fused lm_head projection + per-token logprob / entropy for gfx950, logits never materialised.
+//
+// One bf16 MFMA main loop (C[m, n] = sum_k A[m, k] * B[n, k], both operands row-major with k
+// contiguous) serves four kernels that differ only in what they do with the fp32 tile:
+//
+//   forward   A = W [V, H],  B = hidden [N, H]   -> online (max, sum-exp, sum exp*z) per token,
+//                                                    merged over the vocabulary tiles of a split
+//   dz        A = W,         B = hidden          -> dZ = g * (onehot - softmax), bf16, written in
+//                                                    both [token, vocab] and [vocab, token] order
+//   d_hidden  A = dZ [N, Vc], B = W^T [H, V]     -> fp32 accumulate over vocabulary chunks
+//   d_weight  A = dZ^T [Vc, N], B = hidden^T     -> bf16 rows of dW for the chunk
+//
+// Tile: 256 x 256 x 64 per 512-thread workgroup, 8 waves as 4 (m) x 2 (n), each wave 64 x 128 =
+// 2 x 4 MFMA 32x32x16 accumulators.  With vocabulary as the m dim a lane's 16 accumulator
+// registers of one MFMA tile belong to ONE token (column), so the softmax statistics reduce
+// inside the lane.  LDS: two buffers of (A + B) tiles with rows padded to 72 bf16 (144 B), which
+// keeps the 16-byte fragment reads of 32 consecutive rows on distinct banks.
+#include "oi_common.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int NTHREADS = 512;
+constexpr int LDS_STRIDE = BK + 8;             // bf16 elements per padded tile row
+constexpr int TILE_ELEMS = BM * LDS_STRIDE;    // one operand tile
+constexpr int BUF_ELEMS = 2 * TILE_ELEMS;      // A + B
+constexpr int LDS_BYTES = 2 * BUF_ELEMS * 2;   // two buffers, 147456 B
+constexpr int STAGE_STRIDE = 256 + 8;          // bf16 per row of the dZ staging tile
+static_assert(256 * STAGE_STRIDE * 2 <= LDS_BYTES, "dZ staging tile must fit in the main-loop LDS");
+
+typedef f32x16 AccTile[2][4];
+
+// XCD-aware tile order.  Consecutive workgroup ids go round-robin to the 8 XCDs, each with its own
+// L2; the 32 workgroups resident on one XCD form an 8 (m) x 4 (n) super-tile so that they share
+// operand slabs in that L2, and the 8 XCDs take super-tiles that are neighbours along m.
+__device__ __forceinline__ bool tile_of_block(int64_t tiles_m, int64_t tiles_n, int64_t* tm, int64_t* tn) {
+    const int64_t pid = blockIdx.x;
+    const int64_t xcd = pid & 7, local = pid >> 3;
+    const int64_t nsm = (tiles_m + 7) / 8;
+    const int64_t st = (local >> 5) * 8 + xcd, inner = local & 31;
+    *tm = (st % nsm) * 8 + (inner & 7);
+    *tn = (st / nsm) * 4 + (inner >> 3);
+    return *tm < tiles_m && *tn < tiles_n;
+}
+inline unsigned grid_for_tiles(int64_t tiles_m, int64_t tiles_n) {
+    const int64_t nst = ((tiles_m + 7) / 8) * ((tiles_n + 3) / 4);
+    return (unsigned)(((nst + 7) / 8) * 8 * 32);
+}
+
+// acc = A[m0 : m0+256, :K] * B[n0 : n0+256, :K]^T.  Rows past M / N are clamped onto the last
+// valid row (their results are discarded by the epilogues); K must be a multiple of 64.
+__device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restrict__ A, int64_t lda, int64_t m0,
+                                          int64_t M, const uint16_t* __restrict__ B, int64_t ldb, int64_t n0,
+                                          int64_t N, int64_t K, uint16_t* lds) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave & 3, wn = wave >> 2;
+
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // global -> LDS staging: 2048 16-byte chunks per operand tile, 4 per thread
+    const int lrow = tid >> 3, kc = tid & 7;
+    const uint16_t* ap[4];
+    const uint16_t* bp[4];
+    int soff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = lrow + i * 64;
+        int64_t ga = m0 + r, gb = n0 + r;
+        ga = ga < M ? ga : M - 1;
+        gb = gb < N ? gb : N - 1;
+        ap[i] = A + ga * lda + kc * 8;
+        bp[i] = B + gb * ldb + kc * 8;
+        soff[i] = r * LDS_STRIDE + kc * 8;
+    }
+    oi_u32x4 sa[4], sb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        sa[i] = *reinterpret_cast<const oi_u32x4*>(ap[i]);
+        sb[i] = *reinterpret_cast<const oi_u32x4*>(bp[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        *reinterpret_cast<oi_u32x4*>(lds + soff[i]) = sa[i];
+        *reinterpret_cast<oi_u32x4*>(lds + TILE_ELEMS + soff[i]) = sb[i];
+    }
+    __syncthreads();
+
+    const int frag_off = (lane & 31) * LDS_STRIDE + (lane >> 5) * 8;
+    const int a_off = wm * 64 * LDS_STRIDE + frag_off;
+    const int b_off = TILE_ELEMS + wn * 128 * LDS_STRIDE + frag_off;
+
+    const int64_t ktiles = K / BK;
+    for (int64_t kt = 0; kt < ktiles; ++kt) {
+        const bool more = kt + 1 < ktiles;
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                sa[i] = *reinterpret_cast<const oi_u32x4*>(ap[i] + (kt + 1) * BK);
+                sb[i] = *reinterpret_cast<const oi_u32x4*>(bp[i] + (kt + 1) * BK);
+            }
+        }
+        const uint16_t* cur = lds + (kt & 1) * BUF_ELEMS;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            bf16x8 af[2], bf[4];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                af[i] = *reinterpret_cast<const bf16x8*>(cur + a_off + i * 32 * LDS_STRIDE + ks * 16);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                bf[j] = *reinterpret_cast<const bf16x8*>(cur + b_off + j * 32 * LDS_STRIDE + ks * 16);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            uint16_t* nxt = lds + ((kt + 1) & 1) * BUF_ELEMS;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                *reinterpret_cast<oi_u32x4*>(nxt + soff[i]) = sa[i];
+                *reinterpret_cast<oi_u32x4*>(nxt + TILE_ELEMS + soff[i]) = sb[i];
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// Accumulator geometry of one wave: element (i, j, r) of lane `lane` is
+//   m (row, vocabulary in the logits kernels) = wm*64 + i*32 + (r/4)*8 + (lane/32)*4 + r%4
+//   n (column, token in the logits kernels)   = wn*128 + j*32 + lane%32
+__device__ __forceinline__ int acc_row(int wm, int i, int r, int lane) {
+    return wm * 64 + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+}
+__device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * 128 + j * 32 + (lane & 31); }
+
+// ---------------------------------------------------------------------------------------------
+// forward: per-token softmax statistics over the vocabulary tiles of one split
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(NTHREADS)
+    lmhead_fwd_kernel(const uint16_t* __restrict__ W, const uint16_t* __restrict__ hidden,
+                      const int64_t* __restrict__ labels, int64_t n_tokens, int64_t hdim, int64_t vocab, float c,
+                      int64_t n_splits, int64_t tiles_per_split, int64_t n_pad, float4* __restrict__ partial,
+                      float* __restrict__ zy) {
+    __shared__ __align__(16) uint16_t lds[LDS_BYTES / 2];
+    const int64_t token_tiles = (n_tokens + BN - 1) / BN;
+    int64_t split, tt;
+    if (!tile_of_block(n_splits, token_tiles, &split, &tt)) return;
+    const int64_t vocab_tiles = (vocab + BM - 1) / BM;
+    const int64_t vt_begin = split * tiles_per_split;
+    int64_t vt_end = vt_begin + tiles_per_split;
+    vt_end = vt_end < vocab_tiles ? vt_end : vocab_tiles;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave & 3, wn = wave >> 2;
+    const int64_t n0 = tt * BN;
+
+    float st_m[4], st_s[4], st_t[4];
+    int64_t lab[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        st_m[j] = OI_NEG_BIG;
+        st_s[j] = 0.f;
+        st_t[j] = 0.f;
+        const int64_t n = n0 + acc_col(wn, j, lane);
+        int64_t y = n < n_tokens ? labels[n] : 0;
+        lab[j] = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
+    }
+
+    for (int64_t vt = vt_begin; vt < vt_end; ++vt) {
+        AccTile acc;
+        const int64_t m0 = vt * BM;
+        gemm_tile(acc, W, hdim, m0, vocab, hidden, hdim, n0, n_tokens, hdim, lds);
+        const bool partial_tile = m0 + BM > vocab;
+        const int64_t wave_row0 = m0 + wm * 64;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            // the target logit, when its row falls into this wave's 64 rows
+            const int64_t rel = lab[j] - wave_row0;
+            if (rel >= 0 && rel < 64) {
+                const int ri = (int)rel >> 5, rr = (int)rel & 31;
+                if (((rr >> 2) & 1) == (lane >> 5)) {
+                    const int reg = (rr >> 3) * 4 + (rr & 3);
+                    float v = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            if (i == ri && r == reg) v = acc[i][j][r];
+                    const int64_t n = n0 + acc_col(wn, j, lane);
+                    if (n < n_tokens) zy[n] = v;
+                }
+            }
+            float vmax = OI_NEG_BIG;
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    if (partial_tile && m0 + acc_row(wm, i, r, lane) >= vocab) acc[i][j][r] = -INFINITY;
+                    vmax = fmaxf(vmax, acc[i][j][r] * c);
+                }
+            const float mn = fmaxf(st_m[j], vmax);
+            const float alpha = __builtin_amdgcn_exp2f(st_m[j] - mn);
+            float s = st_s[j] * alpha, t = st_t[j] * alpha;
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float z = acc[i][j][r];
+                    const float e = __builtin_amdgcn_exp2f(fmaf(z, c, -mn));
+                    s += e;
+                    t = fmaf(e, z > -INFINITY ? z : 0.f, t);
+                }
+            st_m[j] = mn;
+            st_s[j] = s;
+            st_t[j] = t;
+        }
+    }
+
+    // merge the two lane halves (same token, other rows), then the four m-waves through LDS
+    float* red = reinterpret_cast<float*>(lds);  // [4 wm][256 tokens][3]
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float om = __shfl_xor(st_m[j], 32, OI_WAVE), os = __shfl_xor(st_s[j], 32, OI_WAVE),
+                    ot = __shfl_xor(st_t[j], 32, OI_WAVE);
+        const float mn = fmaxf(st_m[j], om);
+        const float fa = __builtin_amdgcn_exp2f(st_m[j] - mn), fb = __builtin_amdgcn_exp2f(om - mn);
+        const float s = st_s[j] * fa + os * fb, t = st_t[j] * fa + ot * fb;
+        if (lane < 32) {
+            float* p = red + (wm * 256 + acc_col(wn, j, lane)) * 3;
+            p[0] = mn;
+            p[1] = s;
+            p[2] = t;
+        }
+    }
+    __syncthreads();
+    if (tid < 256) {
+        float m = red[tid * 3], s = red[tid * 3 + 1], t = red[tid * 3 + 2];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            const float* p = red + (w * 256 + tid) * 3;
+            const float mn = fmaxf(m, p[0]);
+            const float fa = __builtin_amdgcn_exp2f(m - mn), fb = __builtin_amdgcn_exp2f(p[0] - mn);
+            s = s * fa + p[1] * fb;
+            t = t * fa + p[2] * fb;
+            m = mn;
+        }
+        const int64_t n = n0 + tid;
+        if (n < n_tokens) partial[split * n_pad + n] = make_float4(m, s, t, 0.f);
+    }
+}
+
+__global__ void lmhead_fwd_combine_kernel(const float4* __restrict__ partial, const float* __restrict__ zy,
+                                          int64_t n_tokens, int64_t n_splits, int64_t n_pad, float inv_t,
+                                          float* __restrict__ logprob, float* __restrict__ entropy,
+                                          float* __restrict__ lse_out) {
+    const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= n_tokens) return;
+    float m = OI_NEG_BIG, s = 0.f, t = 0.f;
+    for (int64_t sp = 0; sp < n_splits; ++sp) {
+        const float4 p = partial[sp * n_pad + n];
+        const float mn = fmaxf(m, p.x);
+        const float fa = __builtin_amdgcn_exp2f(m - mn), fb = __builtin_amdgcn_exp2f(p.x - mn);
+        s = s * fa + p.y * fb;
+        t = t * fa + p.z * fb;
+        m = mn;
+    }
+    const float lse = (m + log2f(s)) * OI_LN2;
+    logprob[n] = zy[n] * inv_t - lse;
+    if (entropy) entropy[n] = lse - inv_t * (t / s);
+    if (lse_out) lse_out[n] = lse;
+}
+
+// ---------------------------------------------------------------------------------------------
+// backward step 1: dZ tile = g * inv_T * (onehot - softmax), bf16, both orientations
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(NTHREADS)
+    lmhead_dz_kernel(const uint16_t* __restrict__ W, const uint16_t* __restrict__ hidden,
+                     const int64_t* __restrict__ labels, const float* __restrict__ lse,
+                     const float* __restrict__ grad, int64_t n_tokens, int64_t hdim, int64_t vocab, float c,
+                     float inv_t, int64_t v_begin, int64_t chunk_cols, int64_t n_pad, uint16_t* __restrict__ dz,
+                     uint16_t* __restrict__ dzt) {
+    __shared__ __align__(16) uint16_t lds[LDS_BYTES / 2];
+    const int64_t token_tiles = n_pad / BN, vocab_tiles = chunk_cols / BM;
+    int64_t vt, tt;
+    if (!tile_of_block(vocab_tiles, token_tiles, &vt, &tt)) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave & 3, wn = wave >> 2;
+    const int64_t n0 = tt * BN, m0 = v_begin + vt * BM;
+
+    AccTile acc;
+    gemm_tile(acc, W, hdim, m0, vocab, hidden, hdim, n0, n_tokens, hdim, lds);
+
+    // stage[n][v]: rows = tokens of the tile, 256 (+8 pad) vocabulary columns
+    uint16_t* stage = lds;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int nl = acc_col(wn, j, lane);
+        const int64_t n = n0 + nl;
+        const bool live = n < n_tokens;
+        const float g = live ? grad[n] * inv_t : 0.f;
+        const float l2 = live ? lse[n] * OI_LOG2E : 0.f;
+        int64_t y = live ? labels[n] : -1;
+        if (live) y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float d[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int r = q * 4 + e;
+                    const int64_t v = m0 + acc_row(wm, i, r, lane);
+                    float val = 0.f;
+                    if (g != 0.f && v < vocab) {
+                        val = -g * __builtin_amdgcn_exp2f(fmaf(acc[i][j][r], c, -l2));
+                        if (v == y) val += g;
+                    }
+                    d[e] = val;
+                }
+                const int vl = acc_row(wm, i, q * 4, lane);
+                uint2 pk = make_uint2(oi_pack_bf16x2(d[0], d[1]), oi_pack_bf16x2(d[2], d[3]));
+                *reinterpret_cast<uint2*>(stage + nl * STAGE_STRIDE + vl) = pk;
+            }
+    }
+    __syncthreads();
+    const int64_t vcol0 = vt * BM;  // column of this tile inside the chunk
+    // [token, vocab] order: 32 16-byte pieces per token row
+#pragma unroll 4
+    for (int it = 0; it < 16; ++it) {
+        const int cidx = tid + it * NTHREADS;
+        const int row = cidx >> 5, ch = cidx & 31;
+        const oi_u32x4 v = *reinterpret_cast<const oi_u32x4*>(stage + row * STAGE_STRIDE + ch * 8);
+        *reinterpret_cast<oi_u32x4*>(dz + (n0 + row) * chunk_cols + vcol0 + ch * 8) = v;
+    }
+    // [vocab, token] order: every thread gathers 8 tokens of one vocabulary row
+    if (dzt) {
+#pragma unroll 2
+        for (int it = 0; it < 16; ++it) {
+            const int cidx = tid + it * NTHREADS;
+            const int vrow = cidx & 255, nch = cidx >> 8;
+            uint32_t w[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t lo = stage[(nch * 8 + 2 * e) * STAGE_STRIDE + vrow];
+                const uint32_t hi = stage[(nch * 8 + 2 * e + 1) * STAGE_STRIDE + vrow];
+                w[e] = lo | (hi << 16);
+            }
+            const oi_u32x4 v = {w[0], w[1], w[2], w[3]};
+            *reinterpret_cast<oi_u32x4*>(dzt + (vcol0 + vrow) * n_pad + n0 + nch * 8) = v;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// backward steps 2 and 3: plain tile products with a store epilogue
+// ---------------------------------------------------------------------------------------------
+// mode 0: out_f32  = acc          mode 1: out_f32 += acc
+// mode 2: out_bf16 = acc          mode 3: out_bf16 = out_f32 + acc   (last chunk of d_hidden)
+__global__ void __launch_bounds__(NTHREADS)
+    gemm_store_kernel(const uint16_t* __restrict__ A, int64_t lda, int64_t M, const uint16_t* __restrict__ B,
+                      int64_t ldb, int64_t N, int64_t K, int mode, float* out_f32, uint16_t* out_bf16, int64_t ldo,
+                      int64_t m_valid) {
+    __shared__ __align__(16) uint16_t lds[LDS_BYTES / 2];
+    const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    int64_t tm, tn;
+    if (!tile_of_block(tiles_m, tiles_n, &tm, &tn)) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave & 3, wn = wave >> 2;
+    const int64_t m0 = tm * BM, n0 = tn * BN;
+    AccTile acc;
+    gemm_tile(acc, A, lda, m0, M, B, ldb, n0, N, K, lds);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t col = n0 + acc_col(wn, j, lane);
+            if (col >= N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t row = m0 + acc_row(wm, i, r, lane);
+                if (row >= m_valid) continue;
+                const int64_t o = row * ldo + col;
+                float v = acc[i][j][r];
+                if (mode == 1 || mode == 3) v += out_f32[o];
+                if (mode <= 1) out_f32[o] = v;
+                else out_bf16[o] = (uint16_t)oi_f32_to_bf16_bits(v);
+            }
+        }
+}
+
+// out[c, r] = in[r, c] for bf16, rows of `out` padded with zeros up to ld_out columns
+__global__ void __launch_bounds__(256)
+    transpose_pad_kernel(const uint16_t* __restrict__ in, int64_t rows, int64_t cols, uint16_t* __restrict__ out,
+                         int64_t ld_out) {
+    __shared__ uint16_t tile[64][66];
+    const int64_t r0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int k = ty; k < 64; k += 4) {
+        const int64_t r = r0 + k, cc = c0 + tx;
+        tile[k][tx] = (r < rows && cc < cols) ? in[r * cols + cc] : (uint16_t)0;
+    }
+    __syncthreads();
+    for (int k = ty; k < 64; k += 4) {
+        const int64_t cc = c0 + k, r = r0 + tx;
+        if (cc < cols && r < ld_out) out[cc * ld_out + r] = tile[tx][k];
+    }
+}
+
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+constexpr int64_t BWD_VOCAB_CHUNK = 16384;
+
+struct FwdPlan {
+    int64_t token_tiles, vocab_tiles, n_splits, tiles_per_split, n_pad;
+};
+FwdPlan plan_fwd(int64_t n_tokens, int64_t vocab) {
+    FwdPlan p;
+    p.token_tiles = (n_tokens + BN - 1) / BN;
+    p.vocab_tiles = (vocab + BM - 1) / BM;
+    p.n_pad = p.token_tiles * BN;
+    // enough workgroups for ~4 rounds over 256 CUs, but at least 8 vocabulary tiles per split
+    int64_t want = (1024 + p.token_tiles - 1) / p.token_tiles;
+    int64_t max_splits = (p.vocab_tiles + 7) / 8;
+    if (max_splits < 1) max_splits = 1;
+    int64_t s = want < max_splits ? want : max_splits;
+    if (s < 1) s = 1;
+    p.tiles_per_split = (p.vocab_tiles + s - 1) / s;
+    p.n_splits = (p.vocab_tiles + p.tiles_per_split - 1) / p.tiles_per_split;
+    return p;
+}
+
+struct BwdPlan {
+    int64_t n_pad, v_pad, chunk;
+    size_t off_wt, off_ht, off_dz, off_dzt, off_dh32, total;
+};
+BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab, int want_dw) {
+    BwdPlan p;
+    p.n_pad = round_up(n_tokens, 256);
+    p.v_pad = round_up(vocab, 256);
+    p.chunk = p.v_pad < BWD_VOCAB_CHUNK ? p.v_pad : BWD_VOCAB_CHUNK;
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        size_t o = off;
+        off += (bytes + 255) / 256 * 256;
+        return o;
+    };
+    p.off_wt = take((size_t)hdim * p.v_pad * 2);
+    p.off_dz = take((size_t)p.n_pad * p.chunk * 2);
+    p.off_dh32 = take((size_t)n_tokens * hdim * 4);
+    p.off_ht = want_dw ? take((size_t)hdim * p.n_pad * 2) : 0;
+    p.off_dzt = want_dw ? take((size_t)p.chunk * p.n_pad * 2) : 0;
+    p.total = off;
+    return p;
+}
+
+int check_lmhead(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens, int64_t hdim,
+                 int64_t vocab, float inv_t) {
+    OI_RETURN_IF(n_tokens < 0 || hdim <= 0 || vocab <= 0, OI_EINVAL);
+    OI_RETURN_IF(hdim % BK != 0, OI_EINVAL);
+    OI_RETURN_IF(!(inv_t > 0.f) || !(inv_t < 3.0e38f), OI_EINVAL);
+    OI_RETURN_IF(n_tokens > (int64_t)1 << 30 || vocab > (int64_t)1 << 30, OI_EINVAL);
+    if (n_tokens == 0) return OI_OK;
+    OI_RETURN_IF(!hidden || !weight || !labels, OI_ENULL);
+    OI_RETURN_IF(!oi_aligned(hidden, 16) || !oi_aligned(weight, 16), OI_EALIGN);
+    return OI_OK;
+}
+
+}  // namespace
+
+extern "C" size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab) {
+    (void)hidden_dim;
+    if (n_tokens <= 0 || vocab <= 0) return 0;
+    const FwdPlan p = plan_fwd(n_tokens, vocab);
+    return (size_t)p.n_splits * p.n_pad * sizeof(float4) + (size_t)p.n_pad * sizeof(float);
+}
+
+extern "C" int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
+                                  int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob,
+                                  float* entropy, float* lse, void* workspace, size_t workspace_bytes, void* stream) {
+    const int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
+    if (rc != OI_OK) return rc;
+    if (n_tokens == 0) return OI_OK;
+    OI_RETURN_IF(!logprob || !workspace, OI_ENULL);
+    OI_RETURN_IF(!oi_aligned(workspace, 16), OI_EALIGN);
+    OI_RETURN_IF(workspace_bytes < oi_lmhead_fwd_workspace_bytes(n_tokens, hidden_dim, vocab), OI_EWORKSPACE);
+    const FwdPlan p = plan_fwd(n_tokens, vocab);
+    float4* partial = static_cast<float4*>(workspace);
+    float* zy = reinterpret_cast<float*>(partial + p.n_splits * p.n_pad);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const float c = inv_temperature * OI_LOG2E;
+    hipLaunchKernelGGL(lmhead_fwd_kernel, dim3(grid_for_tiles(p.n_splits, p.token_tiles)), dim3(NTHREADS), 0, s,
+                       static_cast<const uint16_t*>(weight), static_cast<const uint16_t*>(hidden), labels, n_tokens,
+                       hidden_dim, vocab, c, p.n_splits, p.tiles_per_split, p.n_pad, partial, zy);
+    hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
+                       zy, n_tokens, p.n_splits, p.n_pad, inv_temperature, logprob, entropy, lse);
+    return oi_launch_status();
+}
+
+extern "C" size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
+                                                int want_d_weight) {
+    if (n_tokens <= 0 || hidden_dim <= 0 || vocab <= 0) return 0;
+    return plan_bwd(n_tokens, hidden_dim, vocab, want_d_weight).total;
+}
+
+extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
+                                  const float* grad_logprob, int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
+                                  float inv_temperature, void* d_hidden, void* d_weight, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+    const int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
+    if (rc != OI_OK) return rc;
+    if (n_tokens == 0) return OI_OK;
+    OI_RETURN_IF(!lse || !grad_logprob || !d_hidden || !workspace, OI_ENULL);
+    OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 2) || !oi_aligned(d_weight, 2), OI_EALIGN);
+    const int want_dw = d_weight != nullptr;
+    const BwdPlan p = plan_bwd(n_tokens, hidden_dim, vocab, want_dw);
+    OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    char* ws = static_cast<char*>(workspace);
+    uint16_t* wt = reinterpret_cast<uint16_t*>(ws + p.off_wt);
+    uint16_t* dz = reinterpret_cast<uint16_t*>(ws + p.off_dz);
+    float* dh32 = reinterpret_cast<float*>(ws + p.off_dh32);
+    uint16_t* ht = want_dw ? reinterpret_cast<uint16_t*>(ws + p.off_ht) : nullptr;
+    uint16_t* dzt = want_dw ? reinterpret_cast<uint16_t*>(ws + p.off_dzt) : nullptr;
+    const uint16_t* Wp = static_cast<const uint16_t*>(weight);
+    const uint16_t* Hp = static_cast<const uint16_t*>(hidden);
+    const float c = inv_temperature * OI_LOG2E;
+
+    // W^T [H, v_pad] and hidden^T [H, n_pad], zero padded (the pads are multiplied by zero dZ
+    // entries and must not hold NaN/Inf bit patterns)
+    hipLaunchKernelGGL(transpose_pad_kernel, dim3((unsigned)(p.v_pad / 64), (unsigned)(hidden_dim / 64)), dim3(256), 0,
+                       s, Wp, vocab, hidden_dim, wt, p.v_pad);
+    if (want_dw)
+        hipLaunchKernelGGL(transpose_pad_kernel, dim3((unsigned)(p.n_pad / 64), (unsigned)(hidden_dim / 64)), dim3(256),
+                           0, s, Hp, n_tokens, hidden_dim, ht, p.n_pad);
+
+    const int64_t n_chunks = (p.v_pad + p.chunk - 1) / p.chunk;
+    for (int64_t ci = 0; ci < n_chunks; ++ci) {
+        const int64_t v_begin = ci * p.chunk;
+        const int64_t cols = (p.v_pad - v_begin) < p.chunk ? (p.v_pad - v_begin) : p.chunk;  // multiple of 256
+        hipLaunchKernelGGL(lmhead_dz_kernel, dim3(grid_for_tiles(cols / BM, p.n_pad / BN)), dim3(NTHREADS), 0,
+                           s, Wp, Hp, labels, lse, grad_logprob, n_tokens, hidden_dim, vocab, c, inv_temperature,
+                           v_begin, cols, p.n_pad, dz, dzt);
+        // d_hidden[n, h] (+)= sum_v dZ[n, v] * W^T[h, v_begin + v]
+        const bool first = ci == 0, last = ci == n_chunks - 1;
+        const int mode = last ? (first ? 2 : 3) : (first ? 0 : 1);
+        hipLaunchKernelGGL(gemm_store_kernel, dim3(grid_for_tiles(p.n_pad / BM, (hidden_dim + BN - 1) / BN)),
+                           dim3(NTHREADS), 0, s, dz, cols, p.n_pad, wt + v_begin, p.v_pad, hidden_dim, cols,
+                           mode, dh32, static_cast<uint16_t*>(d_hidden), hidden_dim, n_tokens);
+        if (want_dw) {
+            // d_weight[v_begin + m, h] = sum_n dZ^T[m, n] * hidden^T[h, n]
+            const int64_t valid = vocab - v_begin < cols ? vocab - v_begin : cols;
+            hipLaunchKernelGGL(gemm_store_kernel, dim3(grid_for_tiles(cols / BM, (hidden_dim + BN - 1) / BN)),
+                               dim3(NTHREADS), 0, s, dzt, p.n_pad, cols, ht, p.n_pad, hidden_dim, p.n_pad, 2,
+                               static_cast<float*>(nullptr), static_cast<uint16_t*>(d_weight) + v_begin * hidden_dim,
+                               hidden_dim, valid);
+        }
+    }
+    return oi_launch_status();
+}

@@ -1,0 +1,379 @@
+// Row-wise log-softmax gather / entropy over materialised logits, forward and backward.
+//
+// One workgroup streams one row of `vocab` logits exactly once with 16-byte non-temporal loads.
+// Every lane keeps an online (max, sum-exp, sum exp*z) triple in the log2 domain, rescaled once
+// per 16-byte vector rather than per element; lanes are merged by wave shuffles and the four
+// waves through LDS.  The kernel is HBM-bound: 2 (bf16) or 4 (fp32) bytes per logit, nothing
+// else of size [rows, vocab] is read or written by the forward.
+#include "oi_common.h"
+
+namespace {
+
+struct F32Row {
+    typedef float elem_t;
+    static constexpr int VEC = 4;
+    static __device__ __forceinline__ void load_vec(const elem_t* p, float (&z)[VEC]) {
+        oi_f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const oi_f32x4*>(p));
+        z[0] = v.x; z[1] = v.y; z[2] = v.z; z[3] = v.w;
+    }
+    static __device__ __forceinline__ float load_one(const elem_t* p) { return *p; }
+    static __device__ __forceinline__ void store_vec(elem_t* p, const float (&z)[VEC]) {
+        oi_f32x4 v = {z[0], z[1], z[2], z[3]};
+        __builtin_nontemporal_store(v, reinterpret_cast<oi_f32x4*>(p));
+    }
+    static __device__ __forceinline__ void store_one(elem_t* p, float z) { *p = z; }
+};
+
+struct BF16Row {
+    typedef uint16_t elem_t;
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ void load_vec(const elem_t* p, float (&z)[VEC]) {
+        oi_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const oi_u32x4*>(p));
+        z[0] = oi_bf16lo_to_f32(v.x); z[1] = oi_bf16hi_to_f32(v.x);
+        z[2] = oi_bf16lo_to_f32(v.y); z[3] = oi_bf16hi_to_f32(v.y);
+        z[4] = oi_bf16lo_to_f32(v.z); z[5] = oi_bf16hi_to_f32(v.z);
+        z[6] = oi_bf16lo_to_f32(v.w); z[7] = oi_bf16hi_to_f32(v.w);
+    }
+    static __device__ __forceinline__ float load_one(const elem_t* p) { return __uint_as_float((uint32_t)(*p) << 16); }
+    static __device__ __forceinline__ void store_vec(elem_t* p, const float (&z)[VEC]) {
+        oi_u32x4 v = {oi_pack_bf16x2(z[0], z[1]), oi_pack_bf16x2(z[2], z[3]), oi_pack_bf16x2(z[4], z[5]),
+                      oi_pack_bf16x2(z[6], z[7])};
+        __builtin_nontemporal_store(v, reinterpret_cast<oi_u32x4*>(p));
+    }
+    static __device__ __forceinline__ void store_one(elem_t* p, float z) { *p = (uint16_t)oi_f32_to_bf16_bits(z); }
+};
+
+struct F16Row {
+    typedef uint16_t elem_t;
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ void load_vec(const elem_t* p, float (&z)[VEC]) {
+        oi_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const oi_u32x4*>(p));
+        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            z[2 * i] = oi_f16bits_to_f32((uint16_t)(w[i] & 0xffffu));
+            z[2 * i + 1] = oi_f16bits_to_f32((uint16_t)(w[i] >> 16));
+        }
+    }
+    static __device__ __forceinline__ float load_one(const elem_t* p) { return oi_f16bits_to_f32(*p); }
+    static __device__ __forceinline__ void store_vec(elem_t* p, const float (&z)[VEC]) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            w[i] = (uint32_t)oi_f32_to_f16bits(z[2 * i]) | ((uint32_t)oi_f32_to_f16bits(z[2 * i + 1]) << 16);
+        oi_u32x4 v = {w[0], w[1], w[2], w[3]};
+        __builtin_nontemporal_store(v, reinterpret_cast<oi_u32x4*>(p));
+    }
+    static __device__ __forceinline__ void store_one(elem_t* p, float z) { *p = oi_f32_to_f16bits(z); }
+};
+
+// Online softmax statistics of the scaled logits x = z * c (c = log2(e) / T), log2 domain:
+//   m = running max of x,  s = sum 2^(x - m),  t = sum 2^(x - m) * z   (t only when ENT).
+struct RowStat {
+    float m, s, t;
+};
+
+template <int VEC, bool ENT>
+__device__ __forceinline__ void stat_update(RowStat& st, const float (&z)[VEC], float c) {
+    float x[VEC];
+    float vmax = OI_NEG_BIG;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        x[j] = z[j] * c;
+        vmax = fmaxf(vmax, x[j]);
+    }
+    const float mn = fmaxf(st.m, vmax);
+    const float alpha = __builtin_amdgcn_exp2f(st.m - mn);
+    float s = st.s * alpha, t = st.t * alpha;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        const float e = __builtin_amdgcn_exp2f(x[j] - mn);
+        s += e;
+        if (ENT) t = fmaf(e, z[j], t);
+    }
+    st.m = mn;
+    st.s = s;
+    st.t = t;
+}
+
+template <bool ENT>
+__device__ __forceinline__ void stat_update1(RowStat& st, float z, float c) {
+    const float x = z * c;
+    const float mn = fmaxf(st.m, x);
+    const float alpha = __builtin_amdgcn_exp2f(st.m - mn);
+    const float e = __builtin_amdgcn_exp2f(x - mn);
+    st.s = st.s * alpha + e;
+    if (ENT) st.t = fmaf(e, z, st.t * alpha);
+    st.m = mn;
+}
+
+__device__ __forceinline__ RowStat stat_merge(const RowStat& a, const RowStat& b) {
+    RowStat r;
+    r.m = fmaxf(a.m, b.m);
+    const float fa = __builtin_amdgcn_exp2f(a.m - r.m), fb = __builtin_amdgcn_exp2f(b.m - r.m);
+    r.s = a.s * fa + b.s * fb;
+    r.t = a.t * fa + b.t * fb;
+    return r;
+}
+
+__device__ __forceinline__ int64_t row_offset(int64_t row, int64_t n_inner, int64_t stride_outer, int64_t stride_inner) {
+    const int64_t o = row / n_inner, i = row - o * n_inner;
+    return o * stride_outer + i * stride_inner;
+}
+
+constexpr int FWD_UNROLL = 4;
+
+template <typename R, bool VECTORISED, bool ENT>
+__global__ void __launch_bounds__(256) lsg_entropy_fwd_kernel(const typename R::elem_t* __restrict__ logits,
+                                                              int64_t n_inner, int64_t stride_outer,
+                                                              int64_t stride_inner, int64_t vocab,
+                                                              const int64_t* __restrict__ index, float inv_t,
+                                                              float* __restrict__ logprob, float* __restrict__ entropy,
+                                                              float* __restrict__ lse_out) {
+    constexpr int VEC = R::VEC;
+    const int64_t row = blockIdx.x;
+    const typename R::elem_t* p = logits + row_offset(row, n_inner, stride_outer, stride_inner);
+    const float c = inv_t * OI_LOG2E;
+    const int tid = threadIdx.x, nthr = blockDim.x;
+
+    RowStat st = {OI_NEG_BIG, 0.f, 0.f};
+    int64_t done = 0;
+    if (VECTORISED) {
+        const int64_t nvec = vocab / VEC;
+        int64_t i = tid;
+        // full groups of FWD_UNROLL vectors per lane: all loads are issued before the first use
+        for (; i + (int64_t)(FWD_UNROLL - 1) * nthr < nvec; i += (int64_t)FWD_UNROLL * nthr) {
+            float z[FWD_UNROLL][VEC];
+#pragma unroll
+            for (int u = 0; u < FWD_UNROLL; ++u) R::load_vec(p + (i + (int64_t)u * nthr) * VEC, z[u]);
+#pragma unroll
+            for (int u = 0; u < FWD_UNROLL; ++u) stat_update<VEC, ENT>(st, z[u], c);
+        }
+        for (; i < nvec; i += nthr) {
+            float z[VEC];
+            R::load_vec(p + i * VEC, z);
+            stat_update<VEC, ENT>(st, z, c);
+        }
+        done = nvec * VEC;
+    }
+    for (int64_t j = done + tid; j < vocab; j += nthr) stat_update1<ENT>(st, R::load_one(p + j), c);
+
+    // lanes -> wave
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        RowStat o;
+        o.m = __shfl_xor(st.m, off, OI_WAVE);
+        o.s = __shfl_xor(st.s, off, OI_WAVE);
+        o.t = ENT ? __shfl_xor(st.t, off, OI_WAVE) : 0.f;
+        st = stat_merge(st, o);
+    }
+    // waves -> block
+    __shared__ float sm[3][4];
+    const int wave = tid >> 6, lane = tid & 63, nw = nthr >> 6;
+    if (lane == 0) {
+        sm[0][wave] = st.m;
+        sm[1][wave] = st.s;
+        sm[2][wave] = st.t;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        RowStat tot = {sm[0][0], sm[1][0], sm[2][0]};
+        for (int w = 1; w < nw; ++w) {
+            RowStat o = {sm[0][w], sm[1][w], sm[2][w]};
+            tot = stat_merge(tot, o);
+        }
+        const float lse = (tot.m + log2f(tot.s)) * OI_LN2;
+        int64_t y = index[row];
+        y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
+        const float zy = R::load_one(p + y);
+        logprob[row] = zy * inv_t - lse;
+        if (ENT) entropy[row] = lse - inv_t * (tot.t / tot.s);
+        if (lse_out) lse_out[row] = lse;
+    }
+}
+
+template <typename R, bool VECTORISED>
+__global__ void __launch_bounds__(256) lsg_bwd_kernel(const typename R::elem_t* logits, int64_t n_inner,
+                                                      int64_t stride_outer, int64_t stride_inner, int64_t vocab,
+                                                      const int64_t* __restrict__ index,
+                                                      const float* __restrict__ lse,
+                                                      const float* __restrict__ grad_logprob, float inv_t,
+                                                      typename R::elem_t* dlogits, int64_t out_stride_outer,
+                                                      int64_t out_stride_inner) {
+    constexpr int VEC = R::VEC;
+    const int64_t row = blockIdx.x;
+    const typename R::elem_t* p = logits + row_offset(row, n_inner, stride_outer, stride_inner);
+    typename R::elem_t* q = dlogits + row_offset(row, n_inner, out_stride_outer, out_stride_inner);
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    const float g = grad_logprob[row] * inv_t;
+    const int64_t nvec = VECTORISED ? vocab / VEC : 0;
+
+    if (g == 0.f) {  // masked-out token: the gradient row is zero, the logits are not needed
+        float zero[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) zero[j] = 0.f;
+        for (int64_t i = tid; i < nvec; i += nthr) R::store_vec(q + i * VEC, zero);
+        for (int64_t j = nvec * VEC + tid; j < vocab; j += nthr) R::store_one(q + j, 0.f);
+        return;
+    }
+
+    const float c = inv_t * OI_LOG2E;
+    const float l2 = lse[row] * OI_LOG2E;
+    int64_t y = index[row];
+    y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
+    const float ng = -g;
+
+    int64_t i = tid;
+    constexpr int U = 2;
+    for (; i + (int64_t)(U - 1) * nthr < nvec; i += (int64_t)U * nthr) {
+        float z[U][VEC];
+#pragma unroll
+        for (int u = 0; u < U; ++u) R::load_vec(p + (i + (int64_t)u * nthr) * VEC, z[u]);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t base = (i + (int64_t)u * nthr) * VEC;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) z[u][j] = ng * __builtin_amdgcn_exp2f(fmaf(z[u][j], c, -l2));
+            if (y >= base && y < base + VEC) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    if (base + j == y) z[u][j] += g;
+            }
+            R::store_vec(q + base, z[u]);
+        }
+    }
+    for (; i < nvec; i += nthr) {
+        float z[VEC];
+        const int64_t base = i * VEC;
+        R::load_vec(p + base, z);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            z[j] = ng * __builtin_amdgcn_exp2f(fmaf(z[j], c, -l2));
+            if (base + j == y) z[j] += g;
+        }
+        R::store_vec(q + base, z);
+    }
+    for (int64_t j = nvec * VEC + tid; j < vocab; j += nthr) {
+        float d = ng * __builtin_amdgcn_exp2f(fmaf(R::load_one(p + j), c, -l2));
+        if (j == y) d += g;
+        R::store_one(q + j, d);
+    }
+}
+
+inline int block_for_vocab(int64_t vocab, int vec) {
+    // one 16-byte vector per lane per trip; short rows do not need four waves
+    const int64_t vecs = vocab / vec;
+    if (vecs >= 1024) return 256;
+    if (vecs >= 256) return 128;
+    return 64;
+}
+
+template <typename R>
+int launch_fwd(const void* logits, int64_t rows, int64_t n_inner, int64_t so, int64_t si, int64_t vocab,
+               const int64_t* index, float inv_t, float* logprob, float* entropy, float* lse, hipStream_t stream) {
+    typedef typename R::elem_t E;
+    const bool vec = oi_aligned(logits, 16) && (so % R::VEC == 0) && (si % R::VEC == 0);
+    const dim3 grid((unsigned)rows), block(block_for_vocab(vocab, R::VEC));
+    const E* p = static_cast<const E*>(logits);
+#define OI_FWD(V_, E_)                                                                                              \
+    hipLaunchKernelGGL((lsg_entropy_fwd_kernel<R, V_, E_>), grid, block, 0, stream, p, n_inner, so, si, vocab, index, \
+                       inv_t, logprob, entropy, lse)
+    if (vec) {
+        if (entropy) OI_FWD(true, true); else OI_FWD(true, false);
+    } else {
+        if (entropy) OI_FWD(false, true); else OI_FWD(false, false);
+    }
+#undef OI_FWD
+    return oi_launch_status();
+}
+
+template <typename R>
+int launch_bwd(const void* logits, int64_t rows, int64_t n_inner, int64_t so, int64_t si, int64_t vocab,
+               const int64_t* index, const float* lse, const float* grad, float inv_t, void* dlogits, int64_t oso,
+               int64_t osi, hipStream_t stream) {
+    typedef typename R::elem_t E;
+    const bool vec = oi_aligned(logits, 16) && oi_aligned(dlogits, 16) && (so % R::VEC == 0) && (si % R::VEC == 0) &&
+                     (oso % R::VEC == 0) && (osi % R::VEC == 0);
+    const dim3 grid((unsigned)rows), block(block_for_vocab(vocab, R::VEC));
+    const E* p = static_cast<const E*>(logits);
+    E* q = static_cast<E*>(dlogits);
+    if (vec)
+        hipLaunchKernelGGL((lsg_bwd_kernel<R, true>), grid, block, 0, stream, p, n_inner, so, si, vocab, index, lse,
+                           grad, inv_t, q, oso, osi);
+    else
+        hipLaunchKernelGGL((lsg_bwd_kernel<R, false>), grid, block, 0, stream, p, n_inner, so, si, vocab, index, lse,
+                           grad, inv_t, q, oso, osi);
+    return oi_launch_status();
+}
+
+int check_rows(const void* logits, int64_t n_outer, int64_t n_inner, int64_t so, int64_t si, int64_t vocab,
+               const int64_t* index, float inv_t, int64_t* rows) {
+    OI_RETURN_IF(n_outer < 0 || n_inner < 0 || vocab <= 0, OI_EINVAL);
+    OI_RETURN_IF(!(inv_t > 0.f) || !(inv_t < 3.0e38f), OI_EINVAL);
+    *rows = n_outer * n_inner;
+    OI_RETURN_IF(*rows > 0x7fffffffLL, OI_EINVAL);
+    if (*rows == 0) return OI_OK;
+    OI_RETURN_IF(!logits || !index, OI_ENULL);
+    OI_RETURN_IF(si < vocab && n_inner > 1, OI_EINVAL);
+    OI_RETURN_IF(so < 0 || si < 0, OI_EINVAL);
+    return OI_OK;
+}
+
+}  // namespace
+
+extern "C" int oi_lsg_entropy_fwd(const void* logits, int dtype, int64_t n_outer, int64_t n_inner,
+                                  int64_t stride_outer, int64_t stride_inner, int64_t vocab, const int64_t* index,
+                                  float inv_temperature, float* logprob, float* entropy, float* lse, void* stream) {
+    int64_t rows = 0;
+    const int rc = check_rows(logits, n_outer, n_inner, stride_outer, stride_inner, vocab, index, inv_temperature, &rows);
+    if (rc != OI_OK) return rc;
+    OI_RETURN_IF(dtype != OI_DTYPE_F32 && dtype != OI_DTYPE_BF16 && dtype != OI_DTYPE_F16, OI_EDTYPE);
+    if (rows == 0) return OI_OK;
+    OI_RETURN_IF(!logprob, OI_ENULL);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case OI_DTYPE_F32:
+            OI_RETURN_IF(!oi_aligned(logits, 4), OI_EALIGN);
+            return launch_fwd<F32Row>(logits, rows, n_inner, stride_outer, stride_inner, vocab, index, inv_temperature,
+                                      logprob, entropy, lse, s);
+        case OI_DTYPE_BF16:
+            OI_RETURN_IF(!oi_aligned(logits, 2), OI_EALIGN);
+            return launch_fwd<BF16Row>(logits, rows, n_inner, stride_outer, stride_inner, vocab, index,
+                                       inv_temperature, logprob, entropy, lse, s);
+        default:
+            OI_RETURN_IF(!oi_aligned(logits, 2), OI_EALIGN);
+            return launch_fwd<F16Row>(logits, rows, n_inner, stride_outer, stride_inner, vocab, index, inv_temperature,
+                                      logprob, entropy, lse, s);
+    }
+}
+
+extern "C" int oi_lsg_bwd(const void* logits, int dtype, int64_t n_outer, int64_t n_inner, int64_t stride_outer,
+                          int64_t stride_inner, int64_t vocab, const int64_t* index, const float* lse,
+                          const float* grad_logprob, float inv_temperature, void* dlogits, int64_t out_stride_outer,
+                          int64_t out_stride_inner, void* stream) {
+    int64_t rows = 0;
+    const int rc = check_rows(logits, n_outer, n_inner, stride_outer, stride_inner, vocab, index, inv_temperature, &rows);
+    if (rc != OI_OK) return rc;
+    OI_RETURN_IF(dtype != OI_DTYPE_F32 && dtype != OI_DTYPE_BF16 && dtype != OI_DTYPE_F16, OI_EDTYPE);
+    if (rows == 0) return OI_OK;
+    OI_RETURN_IF(!lse || !grad_logprob || !dlogits, OI_ENULL);
+    OI_RETURN_IF(out_stride_outer < 0 || out_stride_inner < 0, OI_EINVAL);
+    OI_RETURN_IF(out_stride_inner < vocab && n_inner > 1, OI_EINVAL);
+    // in-place use is only defined when every row maps onto itself
+    OI_RETURN_IF(dlogits == logits && (out_stride_outer != stride_outer || out_stride_inner != stride_inner),
+                 OI_EINVAL);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t esz = dtype == OI_DTYPE_F32 ? 4 : 2;
+    OI_RETURN_IF(!oi_aligned(logits, esz) || !oi_aligned(dlogits, esz), OI_EALIGN);
+    switch (dtype) {
+        case OI_DTYPE_F32:
+            return launch_bwd<F32Row>(logits, rows, n_inner, stride_outer, stride_inner, vocab, index, lse,
+                                      grad_logprob, inv_temperature, dlogits, out_stride_outer, out_stride_inner, s);
+        case OI_DTYPE_BF16:
+            return launch_bwd<BF16Row>(logits, rows, n_inner, stride_outer, stride_inner, vocab, index, lse,
+                                       grad_logprob, inv_temperature, dlogits, out_stride_outer, out_stride_inner, s);
+        default:
+            return launch_bwd<F16Row>(logits, rows, n_inner, stride_outer, stride_inner, vocab, index, lse,
+                                      grad_logprob, inv_temperature, dlogits, out_stride_outer, out_stride_inner, s);
+    }
+}

@@ -1,0 +1,210 @@
+"""DPO-family sequence losses on the GPU.
+
+Names and signatures follow open_instruct/dpo_utils.py in the reference (``dpo_loss`` :523-563,
+``wpo_loss`` :566-613, ``simpo_loss`` :617-642, ``compute_loss`` :645-686, ``_get_batch_logps``
+:689-712, ``concatenated_inputs`` :734-763, ``concatenated_forward`` :826-878).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib, padding_free_collator
+from .padding_free_collator import get_batch_logps_padded
+
+
+class _SigmoidPairLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, pc, pr, rc, rr, weights, beta, label_smoothing, margin):
+        dev = _lib.require_gpu(pc, pr, rc, rr, weights)
+        shape = pc.shape
+        pc_c, pr_c = _lib.f32c(pc).reshape(-1), _lib.f32c(pr).reshape(-1)
+        rc_c = _lib.f32c(rc).reshape(-1) if rc is not None else None
+        rr_c = _lib.f32c(rr).reshape(-1) if rr is not None else None
+        w_c = _lib.f32c(weights).reshape(-1) if weights is not None else None
+        n = pc_c.numel()
+        out = torch.empty((3, n), dtype=torch.float32, device=dev)
+        _lib.call(
+            "oi_dpo_sigmoid_fwd", pc_c.data_ptr(), pr_c.data_ptr(), _lib.ptr(rc_c), _lib.ptr(rr_c), _lib.ptr(w_c), n,
+            beta, label_smoothing, margin, out[0].data_ptr(), out[1].data_ptr(), out[2].data_ptr(),
+            _lib.stream_of(pc_c),
+        )  # fmt: skip
+        ctx.save_for_backward(pc_c, pr_c, rc_c, rr_c, w_c)
+        ctx.meta = (beta, label_smoothing, margin, shape, pc.dtype, pr.dtype)
+        losses, cr, rj = (t.reshape(shape) for t in out.unbind(0))
+        ctx.mark_non_differentiable(cr, rj)
+        return losses, cr, rj
+
+    @staticmethod
+    def backward(ctx, g_losses, _g_cr, _g_rj):
+        pc_c, pr_c, rc_c, rr_c, w_c = ctx.saved_tensors
+        beta, ls, margin, shape, dt_c, dt_r = ctx.meta
+        g = _lib.f32c(g_losses).reshape(-1)
+        n = pc_c.numel()
+        d = torch.empty((2, n), dtype=torch.float32, device=g.device)
+        _lib.call(
+            "oi_dpo_sigmoid_bwd", pc_c.data_ptr(), pr_c.data_ptr(), _lib.ptr(rc_c), _lib.ptr(rr_c), _lib.ptr(w_c),
+            g.data_ptr(), n, beta, ls, margin, d[0].data_ptr(), d[1].data_ptr(), _lib.stream_of(g),
+        )  # fmt: skip
+        return d[0].reshape(shape).to(dt_c), d[1].reshape(shape).to(dt_r), None, None, None, None, None, None
+
+
+def dpo_loss(
+    policy_chosen_logps: torch.Tensor,
+    policy_rejected_logps: torch.Tensor,
+    reference_chosen_logps: torch.Tensor,
+    reference_rejected_logps: torch.Tensor,
+    beta: float,
+    reference_free: bool = False,
+    label_smoothing: float = 0.0,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Sigmoid DPO loss per pair and detached rewards; drop-in for open_instruct/dpo_utils.py:523-563.
+
+    ``reference_free`` drops the reference log-ratio from the loss only; the rewards still use the
+    provided reference logps, as in the reference.
+    """
+    if reference_free:
+        losses, _, _ = _SigmoidPairLoss.apply(
+            policy_chosen_logps, policy_rejected_logps, None, None, None, float(beta), float(label_smoothing), 0.0
+        )
+        with torch.no_grad():
+            _, cr, rj = _SigmoidPairLoss.apply(
+                policy_chosen_logps.detach(), policy_rejected_logps.detach(), reference_chosen_logps.detach(),
+                reference_rejected_logps.detach(), None, float(beta), float(label_smoothing), 0.0,
+            )  # fmt: skip
+        return losses, cr, rj
+    return _SigmoidPairLoss.apply(
+        policy_chosen_logps, policy_rejected_logps, reference_chosen_logps.detach(),
+        reference_rejected_logps.detach(), None, float(beta), float(label_smoothing), 0.0,
+    )  # fmt: skip
+
+
+def simpo_loss(
+    policy_chosen_logps: torch.Tensor,
+    policy_rejected_logps: torch.Tensor,
+    beta: float,
+    gamma_beta_ratio: float,
+    label_smoothing: float = 0.0,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """SimPO loss (margin ``gamma/beta``, no reference model); open_instruct/dpo_utils.py:617-642."""
+    return _SigmoidPairLoss.apply(
+        policy_chosen_logps, policy_rejected_logps, None, None, None, float(beta), float(label_smoothing),
+        float(gamma_beta_ratio),
+    )  # fmt: skip
+
+
+def wpo_loss(
+    policy_chosen_logps: torch.Tensor,
+    policy_rejected_logps: torch.Tensor,
+    reference_chosen_logps: torch.Tensor,
+    reference_rejected_logps: torch.Tensor,
+    beta: float,
+    chosen_loss_mask: torch.Tensor,
+    rejected_loss_mask: torch.Tensor,
+    label_smoothing: float = 0.0,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """WPO: the DPO pair loss times ``min(1, exp(avg_c + avg_r))``; open_instruct/dpo_utils.py:566-613.
+
+    Follows the reference literally, including that the weights are not detached: the gradient
+    flows through them as well, so the weight factor is assembled with differentiable tensor ops on
+    the ``[bs]`` vectors and multiplied onto the kernel's per-pair loss.
+    """
+    avg_c = (policy_chosen_logps * chosen_loss_mask).sum(-1) / chosen_loss_mask.sum(-1)
+    avg_r = (policy_rejected_logps * rejected_loss_mask).sum(-1) / rejected_loss_mask.sum(-1)
+    weights = torch.clamp(torch.exp(avg_c + avg_r), max=1)
+    base, cr, rj = _SigmoidPairLoss.apply(
+        policy_chosen_logps, policy_rejected_logps, reference_chosen_logps.detach(),
+        reference_rejected_logps.detach(), None, float(beta), float(label_smoothing), 0.0,
+    )  # fmt: skip
+    return base * weights, cr, rj
+
+
+def compute_loss(args, batch: dict, policy_chosen_logps, policy_rejected_logps, reference_cache=None):
+    """Dispatch on ``args.loss_type``; open_instruct/dpo_utils.py:645-686.
+
+    ``reference_cache[batch["index"]]`` must return a mapping with ``chosen_logps`` /
+    ``rejected_logps`` (the reference's ``TensorCache``, open_instruct/model_utils.py:92-115).
+    """
+    loss_type = str(getattr(args.loss_type, "value", args.loss_type))
+    if loss_type in ("dpo", "dpo_norm"):
+        assert reference_cache is not None
+        ref = reference_cache[batch["index"]]
+        return dpo_loss(
+            policy_chosen_logps, policy_rejected_logps, ref["chosen_logps"], ref["rejected_logps"], beta=args.beta,
+            label_smoothing=args.label_smoothing,
+        )  # fmt: skip
+    if loss_type == "simpo":
+        return simpo_loss(
+            policy_chosen_logps, policy_rejected_logps, beta=args.beta, gamma_beta_ratio=args.gamma_beta_ratio,
+            label_smoothing=args.label_smoothing,
+        )  # fmt: skip
+    if loss_type == "wpo":
+        assert reference_cache is not None
+        ref = reference_cache[batch["index"]]
+        return wpo_loss(
+            policy_chosen_logps, policy_rejected_logps, ref["chosen_logps"], ref["rejected_logps"], beta=args.beta,
+            label_smoothing=args.label_smoothing, chosen_loss_mask=batch["chosen_labels"] != -100,
+            rejected_loss_mask=batch["rejected_labels"] != -100,
+        )  # fmt: skip
+    raise ValueError(f"Unknown loss type: {args.loss_type}")
+
+
+def _get_batch_logps(
+    per_token_logps: torch.Tensor, labels: torch.Tensor, average_log_prob: bool = False
+) -> torch.Tensor:
+    """Per-row sum or mean of kept per-token logps; drop-in for open_instruct/dpo_utils.py:689-712."""
+    return get_batch_logps_padded(per_token_logps, labels, average_log_prob)
+
+
+def _pad_to(t: torch.Tensor, length: int, value: int) -> torch.Tensor:
+    if t.shape[1] == length:
+        return t
+    pad = torch.full((t.shape[0], length - t.shape[1]), value, dtype=t.dtype, device=t.device)
+    return torch.cat([t, pad], dim=1)
+
+
+def concatenated_inputs(batch: dict) -> dict:
+    """Chosen and rejected stacked along the batch dim, padded to a common length.
+
+    Integer plumbing of open_instruct/dpo_utils.py:734-763: ``labels`` pad with -100, everything
+    else with 0.
+    """
+    keys = [k for k in batch if k.startswith("chosen_") and isinstance(batch[k], torch.Tensor)]
+    max_len = max(batch["chosen_input_ids"].shape[1], batch["rejected_input_ids"].shape[1])
+    out = {}
+    for k in keys:
+        name = k[len("chosen_") :]
+        pad = -100 if "labels" in name else 0
+        out[f"concatenated_{name}"] = torch.cat(
+            [_pad_to(batch[k], max_len, pad), _pad_to(batch[f"rejected_{name}"], max_len, pad)], dim=0
+        )
+    return out
+
+
+def concatenated_forward(model, batch: dict, average_log_prob: bool = False, packing: bool = False):
+    """One model forward over chosen+rejected, then per-sequence logps; open_instruct/dpo_utils.py:826-878.
+
+    Returns ``(chosen_logps, rejected_logps, aux_loss)`` with ``aux_loss`` None (router losses are
+    outside this package).
+    """
+    if packing:
+        concat, bs = padding_free_collator.concatenated_inputs(batch)
+    else:
+        concat = concatenated_inputs(batch)
+        bs = batch["chosen_input_ids"].shape[0]
+    inputs = {
+        k.replace("concatenated_", ""): v
+        for k, v in concat.items()
+        if k.startswith("concatenated_") and not k.endswith("labels")
+    }
+    output = model(**inputs)
+    logits = getattr(output, "logits", output)
+    labels = concat["concatenated_labels"]
+    per_token = padding_free_collator.calculate_per_token_logps(logits, labels)
+    if packing:
+        logps = padding_free_collator.get_batch_logps(
+            per_token, labels, concat["concatenated_cu_seq_lens_k"], average_log_prob
+        )
+    else:
+        logps = _get_batch_logps(per_token, labels, average_log_prob)
+    return logps[:bs], logps[bs:], None

@@ -1,0 +1,510 @@
+"""GRPO logprob forward and loss functions on the GPU.
+
+Names, signatures and argument meaning follow open_instruct/grpo_utils.py in the reference
+(``mask_logprobs`` :340-344, ``compute_rho_correction`` :410-463, ``resolve_old_logprob`` :475-501,
+``compute_grpo_loss`` :504-538, ``forward_for_logprobs`` :541-574, ``compute_logprobs`` :577-648,
+``calculate_token_counts`` :651-671, loss-stat helpers :674-742).  ``config`` is duck-typed as in
+the reference: only attributes are read.
+
+``grpo_loss_fused`` and ``group_advantages`` have no single counterpart in the reference; they
+carry the loss assembly of open_instruct/grpo_fast.py:702-724 and the advantage formula of
+open_instruct/data_loader.py:1472-1484 in one or two kernel launches each.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+from . import _lib, model_utils
+from .rl_utils import masked_mean
+
+INVALID_LOGPROB = 1.0  # open_instruct/utils.py:83
+
+
+# ----------------------------------------------------------------------------------------------
+# mask_logprobs
+# ----------------------------------------------------------------------------------------------
+class _MaskLogprobs(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logprobs, mask):
+        _lib.require_gpu(logprobs, mask)
+        lp, m = _lib.f32c(logprobs), _lib.mask_u8(mask)
+        out = torch.empty_like(lp)
+        _lib.call(
+            "oi_mask_logprobs_fwd", lp.data_ptr(), m.data_ptr(), lp.numel(), INVALID_LOGPROB, out.data_ptr(),
+            _lib.stream_of(lp),
+        )  # fmt: skip
+        ctx.save_for_backward(lp, m)
+        ctx.in_dtype = logprobs.dtype
+        return out.to(logprobs.dtype)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        lp, m = ctx.saved_tensors
+        g = _lib.f32c(grad_out)
+        d = torch.empty_like(lp)
+        _lib.call(
+            "oi_mask_logprobs_bwd", lp.data_ptr(), m.data_ptr(), g.data_ptr(), lp.numel(), d.data_ptr(),
+            _lib.stream_of(lp),
+        )  # fmt: skip
+        return d.to(ctx.in_dtype), None
+
+
+def mask_logprobs(vllm_logprobs: torch.Tensor, response_mask: torch.Tensor) -> torch.Tensor:
+    """Set non-response positions and NaNs to ``INVALID_LOGPROB`` (+1.0); open_instruct/grpo_utils.py:340-344."""
+    if tuple(vllm_logprobs.shape) != tuple(response_mask.shape):
+        response_mask = response_mask.expand_as(vllm_logprobs)
+    return _MaskLogprobs.apply(vllm_logprobs, response_mask)
+
+
+# ----------------------------------------------------------------------------------------------
+# rho correction
+# ----------------------------------------------------------------------------------------------
+@dataclass
+class RhoCorrection:
+    """Same fields as the reference's dataclass (open_instruct/grpo_utils.py:393-407)."""
+
+    weights: torch.Tensor
+    metrics: dict[str, torch.Tensor]
+    histogram_metrics: dict[str, torch.Tensor] = field(default_factory=dict)
+
+
+def compute_rho_correction(
+    old_logprob: torch.Tensor,
+    vllm_logprobs: torch.Tensor,
+    response_mask: torch.Tensor,
+    advantages: torch.Tensor,
+    config,
+) -> RhoCorrection:
+    """Train/infer mismatch weights rho = pi_train_old / pi_infer_old; open_instruct/grpo_utils.py:410-463.
+
+    Stop-gradient by construction (the reference's inputs carry no grad either).
+    """
+    dev = _lib.require_gpu(old_logprob, vllm_logprobs, response_mask, advantages)
+    with torch.no_grad():
+        old, vl, adv = _lib.f32c(old_logprob.detach()), _lib.f32c(vllm_logprobs.detach()), _lib.f32c(advantages)
+        m = _lib.mask_u8(response_mask)
+        shape = tuple(old.shape)
+        cols = shape[-1] if shape else 1
+        rows = old.numel() // max(cols, 1)
+        bufs = torch.empty((6,) + shape, dtype=torch.float32, device=dev)
+        use = bool(config.use_rho_correction)
+        _lib.call(
+            "oi_rho_correction", old.data_ptr(), vl.data_ptr(), m.data_ptr(), adv.data_ptr(), rows, cols,
+            int(bool(config.rho_mask_sequence_level)) if use else 0,
+            int(bool(config.rho_mask_tv_divergence)) if use else 0,
+            float(config.rho_mask_lower_bound) if use else 0.0, float(config.rho_mask_upper_bound) if use else 0.0,
+            float(config.rho_clamp_lower_bound) if use else 0.0, float(config.rho_clamp_upper_bound) if use else 0.0,
+            *[bufs[k].data_ptr() for k in range(6)], _lib.stream_of(old),
+        )  # fmt: skip
+        rho, weights, drop_any, drop_low, drop_high, clipped = bufs.unbind(0)
+        hist = {"val/rho_hist": rho[response_mask.bool()].detach().float()}
+        if not use:
+            return RhoCorrection(weights=torch.ones_like(rho), metrics={}, histogram_metrics=hist)
+        metrics = {
+            "val/rho_drop_frac": drop_any,
+            "val/rho_drop_low_frac": drop_low,
+            "val/rho_drop_high_frac": drop_high,
+            "val/rho_weight": weights,
+            "val/rho_clipfrac": clipped,
+        }
+        return RhoCorrection(weights=weights, metrics=metrics, histogram_metrics=hist)
+
+
+def accumulate_rho_histograms(acc: dict[str, list[torch.Tensor]], correction: RhoCorrection) -> None:
+    for key, values in correction.histogram_metrics.items():
+        acc.setdefault(key, []).append(values.detach().cpu())
+
+
+def finalize_rho_histograms(acc: dict[str, list[torch.Tensor]]) -> dict:
+    return {key: torch.cat(chunks).numpy() for key, chunks in acc.items()}
+
+
+def resolve_old_logprob(
+    old_logprobs_cache: list,
+    sample_idx: int,
+    epoch_idx: int,
+    num_mini_batches: int,
+    use_vllm_logprobs: bool,
+    vllm_logprobs: torch.Tensor,
+    new_logprobs: torch.Tensor,
+) -> torch.Tensor:
+    """Pick the baseline logprobs of a sample; host-side bookkeeping only (open_instruct/grpo_utils.py:475-501)."""
+    if num_mini_batches > 1:
+        result = old_logprobs_cache[sample_idx]
+    else:
+        with torch.no_grad():
+            if epoch_idx == 0:
+                old_logprobs_cache[sample_idx] = vllm_logprobs if use_vllm_logprobs else new_logprobs.detach()
+            result = old_logprobs_cache[sample_idx]
+    assert result is not None
+    return result
+
+
+# ----------------------------------------------------------------------------------------------
+# compute_grpo_loss
+# ----------------------------------------------------------------------------------------------
+def _loss_fn_tag(config) -> int:
+    name = str(getattr(config.loss_fn, "value", config.loss_fn))
+    if name not in _lib.LOSS_FN_TAGS:
+        raise ValueError(f"Invalid loss function: {config.loss_fn}")
+    return _lib.LOSS_FN_TAGS[name]
+
+
+def _clip_bounds(config) -> tuple[float, float]:
+    # evaluated in double and rounded to fp32 once at the C boundary, like a Python scalar in torch.clamp
+    return 1.0 - float(config.clip_lower), 1.0 + float(config.clip_higher)
+
+
+class _GrpoTerms(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, new_logprobs, ratio, advantages, ref_logprobs, rho_weights, loss_fn, lo, hi, kl_estimator):
+        dev = _lib.require_gpu(new_logprobs, ratio, advantages, ref_logprobs, rho_weights)
+        shape = torch.broadcast_shapes(new_logprobs.shape, ratio.shape, advantages.shape, rho_weights.shape)
+        nl = _lib.f32c(new_logprobs.expand(shape))
+        rt = _lib.f32c(ratio.expand(shape))
+        adv = _lib.f32c(advantages.expand(shape))
+        w = _lib.f32c(rho_weights.expand(shape))
+        ref = _lib.f32c(ref_logprobs.expand(shape)) if ref_logprobs is not None else None
+        out = torch.empty((3,) + tuple(shape), dtype=torch.float32, device=dev)
+        n = nl.numel()
+        _lib.call(
+            "oi_grpo_terms_fwd", nl.data_ptr(), rt.data_ptr(), adv.data_ptr(), _lib.ptr(ref), w.data_ptr(), n, loss_fn,
+            lo, hi, kl_estimator, out[0].data_ptr(), out[1].data_ptr(), out[2].data_ptr(), _lib.stream_of(nl),
+        )  # fmt: skip
+        ctx.save_for_backward(nl, rt, adv, ref, w)
+        ctx.cfg = (loss_fn, lo, hi, kl_estimator)
+        ctx.in_shapes = (new_logprobs.shape, ratio.shape)
+        pg, clipfrac, kl = out.unbind(0)
+        ctx.mark_non_differentiable(clipfrac)
+        return pg, clipfrac, kl
+
+    @staticmethod
+    def backward(ctx, g_pg, _g_clip, g_kl):
+        nl, rt, adv, ref, w = ctx.saved_tensors
+        loss_fn, lo, hi, kl_estimator = ctx.cfg
+        need_new, need_ratio = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        g_pg = _lib.f32c(g_pg) if g_pg is not None else None
+        g_kl = _lib.f32c(g_kl) if g_kl is not None else None
+        d_new = torch.empty_like(nl) if need_new else None
+        d_ratio = torch.empty_like(rt) if need_ratio else None
+        _lib.call(
+            "oi_grpo_terms_bwd", nl.data_ptr(), rt.data_ptr(), adv.data_ptr(), _lib.ptr(ref), w.data_ptr(),
+            _lib.ptr(g_pg), _lib.ptr(g_kl), nl.numel(), loss_fn, lo, hi, kl_estimator, _lib.ptr(d_new),
+            _lib.ptr(d_ratio), _lib.stream_of(nl),
+        )  # fmt: skip
+        if d_new is not None and d_new.shape != ctx.in_shapes[0]:
+            d_new = d_new.sum_to_size(ctx.in_shapes[0])
+        if d_ratio is not None and d_ratio.shape != ctx.in_shapes[1]:
+            d_ratio = d_ratio.sum_to_size(ctx.in_shapes[1])
+        return d_new, d_ratio, None, None, None, None, None, None, None
+
+
+def compute_grpo_loss(
+    new_logprobs: torch.Tensor,
+    ratio: torch.Tensor,
+    advantages: torch.Tensor,
+    ref_logprobs: torch.Tensor | None,
+    config,
+    rho_weights: torch.Tensor,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Per-token ``(pg_loss, clipfrac, kl)``; drop-in for open_instruct/grpo_utils.py:504-538.
+
+    DAPO gradients flow to ``ratio``; CISPO uses the detached ratio and sends its gradient to
+    ``new_logprobs``; the KL term flows to ``new_logprobs`` (and to ``ratio`` for estimator 3).
+    """
+    tag = _loss_fn_tag(config)
+    lo, hi = _clip_bounds(config)
+    return _GrpoTerms.apply(
+        new_logprobs, ratio, advantages, ref_logprobs, rho_weights, tag, lo, hi, int(config.kl_estimator)
+    )
+
+
+# ----------------------------------------------------------------------------------------------
+# fused scalar loss (+ statistics) of one micro-batch
+# ----------------------------------------------------------------------------------------------
+GRPO_STAT_NAMES = (
+    "loss/total_avg",
+    "loss/policy_avg",
+    "objective/kl0_avg",
+    "objective/kl1_avg",
+    "objective/kl2_avg",
+    "objective/kl3_avg",
+    "policy/clipfrac_avg",
+    "val/ratio",
+    "policy/entropy_avg",
+    "num_response_tokens",
+)
+
+
+class _GrpoFused(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, new_logprobs, old, ref, adv, mask, rho, entropy, cfg):
+        dev = _lib.require_gpu(new_logprobs, old, ref, adv, mask, rho, entropy)
+        loss_fn, lo, hi, kl_estimator, beta, axis_mode, denominator, scale = cfg
+        nl = _lib.f32c(new_logprobs)
+        if nl.ndim != 2:
+            raise ValueError("grpo_loss_fused expects [rows, cols] tensors")
+        rows, cols = nl.shape
+        sides = [None if t is None else _lib.f32c(t.expand(rows, cols)) for t in (old, ref, adv, rho, entropy)]
+        old_c, ref_c, adv_c, rho_c, ent_c = sides
+        m = _lib.mask_u8(mask.expand(rows, cols))
+        stats = torch.empty(len(GRPO_STAT_NAMES), dtype=torch.float32, device=dev)
+        row_denoms = torch.empty(rows, dtype=torch.float32, device=dev)
+        ws_bytes = _lib.load().oi_grpo_fused_workspace_bytes(rows, cols)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        _lib.call(
+            "oi_grpo_fused_fwd", nl.data_ptr(), _lib.ptr(old_c), _lib.ptr(ref_c), adv_c.data_ptr(), m.data_ptr(),
+            _lib.ptr(rho_c), _lib.ptr(ent_c), rows, cols, loss_fn, lo, hi, kl_estimator, beta, axis_mode, denominator,
+            scale, stats.data_ptr(), row_denoms.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(nl),
+        )  # fmt: skip
+        ctx.save_for_backward(nl, old_c, ref_c, adv_c, m, rho_c, row_denoms)
+        ctx.cfg = cfg
+        ctx.in_dtype = new_logprobs.dtype
+        loss = stats[0]
+        ctx.mark_non_differentiable(stats)
+        return loss.clone(), stats
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_stats):
+        nl, old_c, ref_c, adv_c, m, rho_c, row_denoms = ctx.saved_tensors
+        loss_fn, lo, hi, kl_estimator, beta, _axis_mode, _denominator, scale = ctx.cfg
+        g = _lib.f32c(g_loss).reshape(1)
+        d_new = torch.empty_like(nl)
+        rows, cols = nl.shape
+        _lib.call(
+            "oi_grpo_fused_bwd", nl.data_ptr(), _lib.ptr(old_c), _lib.ptr(ref_c), adv_c.data_ptr(), m.data_ptr(),
+            _lib.ptr(rho_c), rows, cols, loss_fn, lo, hi, kl_estimator, beta, scale, row_denoms.data_ptr(),
+            g.data_ptr(), d_new.data_ptr(), _lib.stream_of(nl),
+        )  # fmt: skip
+        return d_new.to(ctx.in_dtype), None, None, None, None, None, None, None
+
+
+def grpo_loss_fused(
+    new_logprobs: torch.Tensor,
+    old_logprobs: torch.Tensor | None,
+    ref_logprobs: torch.Tensor | None,
+    advantages: torch.Tensor,
+    response_mask: torch.Tensor,
+    config,
+    rho_weights: torch.Tensor | None = None,
+    entropy: torch.Tensor | None = None,
+    loss_denominator: float | None = None,
+    axis: int | None = None,
+    dp_scale: float = 1.0,
+) -> tuple[torch.Tensor, dict[str, torch.Tensor]]:
+    """Scalar GRPO loss of a ``[B, T]`` micro-batch and its statistics in two launches.
+
+    Equivalent to the reference sequence ``ratio = exp(new - old)`` → ``compute_grpo_loss`` →
+    ``masked_mean(pg + beta * kl, mask, axis, loss_denominator) * dp_scale``
+    (open_instruct/grpo_fast.py:702-724) plus the masked means that
+    ``populate_sample_loss_stats`` records (open_instruct/grpo_utils.py:699-729).
+    ``old_logprobs=None`` means ``old = new.detach()`` (ratio 1 with a live gradient).
+    Differentiable with respect to ``new_logprobs`` only; ``old``/``ref``/``advantages``/``rho`` are
+    constants, as in the reference.  Returns ``(loss, stats)`` with ``stats`` keyed by
+    ``GRPO_STAT_NAMES`` (0-dim views of one device vector, no host sync).
+    """
+    if axis not in (None, 1, -1):
+        raise ValueError("axis must be None or the token axis (1)")
+    if loss_denominator is not None and float(loss_denominator) <= 0.0:
+        raise ValueError("loss_denominator must be positive when given")
+    lo, hi = _clip_bounds(config)
+    cfg = (
+        _loss_fn_tag(config), lo, hi, int(config.kl_estimator), float(config.beta), 0 if axis is None else 1,
+        0.0 if loss_denominator is None else float(loss_denominator), float(dp_scale),
+    )  # fmt: skip
+    detach = lambda t: None if t is None else t.detach()  # noqa: E731
+    loss, stats = _GrpoFused.apply(
+        new_logprobs, detach(old_logprobs), detach(ref_logprobs), advantages.detach(), response_mask,
+        detach(rho_weights), detach(entropy), cfg,
+    )  # fmt: skip
+    return loss, {name: stats[i] for i, name in enumerate(GRPO_STAT_NAMES)}
+
+
+def group_advantages(scores: torch.Tensor, group_size: int, normalization: str = "standard") -> torch.Tensor:
+    """Group-normalised advantages; open_instruct/data_loader.py:1472-1484 on the device.
+
+    ``scores`` holds ``n_groups * group_size`` rewards, groups contiguous.  fp64 arithmetic with a
+    population std and ``+1e-8`` like the reference's numpy code, fp32 result.
+    """
+    dev = _lib.require_gpu(scores)
+    if normalization not in ("standard", "centered"):
+        raise ValueError(f"Invalid advantage normalization type: {normalization}")
+    s = scores.reshape(-1).to(torch.float64).contiguous()
+    if group_size <= 0 or s.numel() % group_size:
+        raise ValueError(f"{s.numel()} scores do not split into groups of {group_size}")
+    out = torch.empty(s.numel(), dtype=torch.float32, device=dev)
+    _lib.call(
+        "oi_group_advantages", s.data_ptr(), s.numel() // group_size, group_size,
+        0 if normalization == "standard" else 1, out.data_ptr(), _lib.stream_of(s),
+    )  # fmt: skip
+    return out
+
+
+# ----------------------------------------------------------------------------------------------
+# model forward -> logprobs
+# ----------------------------------------------------------------------------------------------
+def forward_for_logprobs(
+    model: torch.nn.Module,
+    query_responses: torch.Tensor,
+    attention_mask: torch.Tensor | None,
+    position_ids: torch.Tensor,
+    pad_token_id: int,
+    temperature: float,
+    return_entropy: bool = False,
+    pass_olmo_core_doc_lens: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """Model forward, then logprob (and entropy) of each next token; open_instruct/grpo_utils.py:541-574.
+
+    Differences from the reference that do not change results: the temperature is applied inside
+    the kernel instead of through a scaled copy of the logits, the ``[:, :-1]`` slice is an
+    argument of the kernel instead of a view, and entropy comes out of the same pass over the
+    logits as the logprob.  ``pass_olmo_core_doc_lens`` needs ``doc_lens`` derived from the
+    attention mask, which lives in the model-plumbing layer outside this package: pass a model
+    whose forward accepts ``attention_mask`` instead.
+    """
+    if pass_olmo_core_doc_lens:
+        raise NotImplementedError("doc_lens plumbing for olmo-core models is outside this package")
+    output = model(input_ids=query_responses, attention_mask=attention_mask, position_ids=position_ids)
+    logits = getattr(output, "logits", output)
+    labels = query_responses[:, 1:].clone().to(logits.device)
+    labels[labels == pad_token_id] = 0
+    logprob, entropy = model_utils.logprob_and_entropy(
+        logits, labels, temperature=temperature, drop_last=True, want_entropy=return_entropy
+    )
+    return logprob, entropy
+
+
+def compute_logprobs(
+    model: torch.nn.Module,
+    data_BT,
+    pad_token_id: int,
+    temperature: float,
+    use_grad: bool = False,
+    batch_size: int | None = None,
+    pass_olmo_core_doc_lens: bool = False,
+) -> list[torch.Tensor]:
+    """Masked logprobs of every sample in a collated batch; open_instruct/grpo_utils.py:577-648.
+
+    Samples of one shape are concatenated along the batch dim for a single forward, others are
+    run one by one; off-response positions hold ``INVALID_LOGPROB``.
+    """
+    out: list[torch.Tensor] = []
+    n = len(data_BT.query_responses)
+    step = 1 if batch_size is None else batch_size
+    with torch.enable_grad() if use_grad else torch.no_grad():
+        for start in range(0, n, step):
+            idx = list(range(start, min(start + step, n)))
+            same_shape = len({tuple(data_BT.query_responses[i].shape) for i in idx}) == 1
+            groups = [idx] if same_shape else [[i] for i in idx]
+            for grp in groups:
+                qr = torch.cat([data_BT.query_responses[i] for i in grp], dim=0)
+                pos = torch.cat([data_BT.position_ids[i] for i in grp], dim=0)
+                att = (
+                    torch.cat([data_BT.attention_masks[i] for i in grp], dim=0) if pass_olmo_core_doc_lens else None
+                )
+                lp, _ = forward_for_logprobs(
+                    model, qr, att, pos, pad_token_id, temperature, False,
+                    pass_olmo_core_doc_lens=pass_olmo_core_doc_lens,
+                )  # fmt: skip
+                sizes = [data_BT.query_responses[i].shape[0] for i in grp]
+                for i, part in zip(grp, torch.split(lp, sizes, dim=0)):
+                    out.append(mask_logprobs(part, data_BT.response_masks[i][:, 1:]))
+    return out
+
+
+def calculate_token_counts(
+    accumulation_steps: int, data_BT, device: torch.device, process_group=None
+) -> dict[int, float]:
+    """Response-token count per accumulation group; open_instruct/grpo_utils.py:651-671.
+
+    The reference all-reduces the counts over the data-parallel group; this build is single-GPU,
+    so the sum over ranks is the local value (a ``process_group`` is used when one is initialised).
+    """
+    counts: dict[int, float] = {}
+    local = [mask[:, 1:].sum().float() for mask in data_BT.response_masks]
+    if not local:
+        return counts
+    t = torch.stack(local).to(device)
+    if torch.distributed.is_available() and torch.distributed.is_initialized():
+        torch.distributed.all_reduce(t, op=torch.distributed.ReduceOp.SUM, group=process_group)
+    for i, c in enumerate(t.tolist()):
+        key = int((i // accumulation_steps) * accumulation_steps)
+        counts[key] = counts.get(key, 0.0) + c
+    return counts
+
+
+# ----------------------------------------------------------------------------------------------
+# loss statistics (open_instruct/grpo_utils.py:674-742)
+# ----------------------------------------------------------------------------------------------
+_SCALAR_LOSS_STAT_KEYS = [
+    "loss/kl_avg",
+    "loss/policy_avg",
+    "loss/total_avg",
+    "objective/kl0_avg",
+    "objective/kl1_avg",
+    "objective/kl2_avg",
+    "objective/kl3_avg",
+    "policy/clipfrac_avg",
+    "val/ratio",
+    "val/rho_clipfrac",
+    "val/rho_weight",
+    "val/rho_drop_frac",
+    "val/rho_drop_low_frac",
+    "val/rho_drop_high_frac",
+]
+
+
+def create_loss_stats(num_samples: int, device: torch.device, record_entropy: bool = False) -> dict[str, torch.Tensor]:
+    stats = {key: torch.zeros(num_samples, device=device) for key in _SCALAR_LOSS_STAT_KEYS}
+    if record_entropy:
+        stats["policy/entropy_avg"] = torch.zeros(num_samples, device=device)
+    return stats
+
+
+def populate_sample_loss_stats(
+    loss_stats_B: dict[str, torch.Tensor],
+    sample_idx: int,
+    pg_loss: torch.Tensor,
+    clipfrac: torch.Tensor,
+    ratio: torch.Tensor,
+    loss: torch.Tensor,
+    response_mask: torch.Tensor,
+    new_logprobs: torch.Tensor,
+    ref_logprobs: torch.Tensor | None,
+    entropy: torch.Tensor | None,
+    config,
+    rho_metrics: dict[str, torch.Tensor] | None = None,
+) -> None:
+    """Record the masked means of one sample; open_instruct/grpo_utils.py:699-729."""
+    with torch.no_grad():
+        if config.load_ref_policy and ref_logprobs is not None:
+            diff = (new_logprobs - ref_logprobs).clamp(-40.0, 40.0)
+            kl_values = masked_mean(model_utils.estimate_kl(diff, ratio), response_mask).float()
+            for j in range(4):
+                loss_stats_B[f"objective/kl{j}_avg"][sample_idx] = kl_values[j]
+            loss_stats_B["loss/kl_avg"][sample_idx] = kl_values[config.kl_estimator] * config.beta
+        if rho_metrics is not None:
+            for key, value in rho_metrics.items():
+                loss_stats_B[key][sample_idx] = masked_mean(value, response_mask)
+        loss_stats_B["policy/clipfrac_avg"][sample_idx] = masked_mean(clipfrac, response_mask)
+        loss_stats_B["loss/policy_avg"][sample_idx] = masked_mean(pg_loss, response_mask)
+        loss_stats_B["loss/total_avg"][sample_idx] = loss
+        loss_stats_B["val/ratio"][sample_idx] = masked_mean(ratio, response_mask)
+        if entropy is not None:
+            loss_stats_B["policy/entropy_avg"][sample_idx] = masked_mean(entropy, response_mask).float()
+
+
+def compute_metrics_from_loss_stats(
+    loss_stats_B: dict[str, torch.Tensor], token_counts: torch.Tensor
+) -> dict[str, float]:
+    """Token-weighted averages over samples + ratio variance; open_instruct/grpo_utils.py:732-742."""
+    total = token_counts.sum()
+    weights = token_counts / total if total > 0 else torch.zeros_like(token_counts)
+    metrics: dict[str, float] = {}
+    for key, value in loss_stats_B.items():
+        metrics[key] = (value * weights).sum().item()
+    metrics["val/ratio_var"] = (weights * (loss_stats_B["val/ratio"] - metrics["val/ratio"]) ** 2).sum().item()
+    return metrics

@@ -1,0 +1,105 @@
+"""Fused lm_head projection + per-token logprob / entropy (no ``[tokens, vocab]`` logits tensor).
+
+There is no single counterpart in the reference: this replaces the pair "lm_head GEMM, then
+``calculate_per_token_logps`` / ``log_softmax_and_gather`` (+ ``entropy_from_logits``)" at
+open_instruct/olmo_core_train_modules.py:71-76 and open_instruct/grpo_utils.py:558-572.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+
+class _FusedLMHead(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, hidden, weight, labels, inv_temperature, want_entropy):
+        dev = _lib.require_gpu(hidden, weight, labels)
+        if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+            raise ValueError("fused lm_head expects bf16 hidden states and weight")
+        if hidden.ndim != 2 or weight.ndim != 2 or hidden.shape[1] != weight.shape[1]:
+            raise ValueError(f"shape mismatch: hidden {tuple(hidden.shape)} weight {tuple(weight.shape)}")
+        n, h = hidden.shape
+        v = weight.shape[0]
+        if h % 64:
+            raise ValueError("hidden size must be a multiple of 64")
+        hid, w = hidden.contiguous(), weight.contiguous()
+        lab = labels.reshape(-1).to(torch.int64).contiguous()
+        if lab.numel() != n:
+            raise ValueError(f"{lab.numel()} labels for {n} hidden rows")
+        logprob = torch.empty(n, dtype=torch.float32, device=dev)
+        entropy = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
+        lse = torch.empty(n, dtype=torch.float32, device=dev)
+        if n > 0:
+            ws_bytes = _lib.load().oi_lmhead_fwd_workspace_bytes(n, h, v)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            _lib.call(
+                "oi_lmhead_logp_fwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), n, h, v, inv_temperature,
+                logprob.data_ptr(), _lib.ptr(entropy), lse.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
+            )  # fmt: skip
+        ctx.save_for_backward(hid, w, lab, lse)
+        ctx.inv_temperature = inv_temperature
+        if want_entropy:
+            ctx.mark_non_differentiable(entropy)
+        return logprob, entropy
+
+    @staticmethod
+    def backward(ctx, grad_logprob, _grad_entropy):
+        hid, w, lab, lse = ctx.saved_tensors
+        n, h = hid.shape
+        v = w.shape[0]
+        need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        if grad_logprob is None or not (need_h or need_w):
+            return None, None, None, None, None
+        g = _lib.f32c(grad_logprob)
+        d_hidden = torch.empty_like(hid)
+        d_weight = torch.empty_like(w) if need_w else None
+        if n > 0:
+            ws_bytes = _lib.load().oi_lmhead_bwd_workspace_bytes(n, h, v, int(need_w))
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=hid.device)
+            _lib.call(
+                "oi_lmhead_logp_bwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), lse.data_ptr(), g.data_ptr(), n, h,
+                v, ctx.inv_temperature, d_hidden.data_ptr(), _lib.ptr(d_weight), ws.data_ptr(), ws_bytes,
+                _lib.stream_of(hid),
+            )  # fmt: skip
+        elif d_weight is not None:
+            d_weight.zero_()
+        return (d_hidden if need_h else None), d_weight, None, None, None
+
+
+def fused_lm_head_logprobs(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    temperature: float = 1.0,
+    mask: torch.Tensor | None = None,
+    return_entropy: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """``log_softmax(hidden @ weight.T / temperature)[labels]`` (+ entropy) per token, fp32.
+
+    ``hidden`` is ``[N, H]`` bf16 (or any leading shape ``[..., H]``), ``weight`` ``[V, H]`` bf16,
+    ``labels`` int64 with the leading shape of ``hidden``; negative labels are scored as token 0
+    (the reference's ``clamp(min=0)``, open_instruct/padding_free_collator.py:15).  ``mask`` (bool,
+    same leading shape) selects the rows that are computed at all: masked-out rows cost nothing,
+    return 0 and receive a zero gradient.  Differentiable with respect to ``hidden`` and
+    ``weight``; the entropy carries no gradient, as in the reference.
+    """
+    lead = hidden.shape[:-1]
+    hid2 = hidden.reshape(-1, hidden.shape[-1])
+    lab1 = labels.reshape(-1)
+    inv_t = 1.0 / float(temperature)
+    if not float(temperature) > 0.0:
+        raise ValueError(f"temperature must be positive, got {temperature}")
+    if mask is None:
+        lp, ent = _FusedLMHead.apply(hid2, weight, lab1, inv_t, return_entropy)
+        return lp.reshape(lead), (ent.reshape(lead) if ent is not None else None)
+    keep = mask.reshape(-1).bool()
+    idx = torch.nonzero(keep, as_tuple=False).squeeze(1)
+    lp_c, ent_c = _FusedLMHead.apply(hid2.index_select(0, idx), weight, lab1.index_select(0, idx), inv_t, return_entropy)
+    lp = torch.zeros(hid2.shape[0], dtype=torch.float32, device=hidden.device).index_copy(0, idx, lp_c)
+    ent = None
+    if ent_c is not None:
+        ent = torch.zeros(hid2.shape[0], dtype=torch.float32, device=hidden.device).index_copy(0, idx, ent_c)
+        ent = ent.reshape(lead)
+    return lp.reshape(lead), ent

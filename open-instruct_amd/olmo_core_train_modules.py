@@ -1,0 +1,66 @@
+"""DPO LM head that returns per-token log-probabilities, backed by the fused lm_head kernel.
+
+Mirrors ``DPOLMHead`` of the reference (open_instruct/olmo_core_train_modules.py:39-85), which
+subclasses ``olmo_core.nn.lm_head.LMHead``.  olmo-core is a third-party package outside this
+build, so this class is a plain ``torch.nn.Module`` with the attributes the reference's forward
+touches (``norm``, ``w_out``) and the same ``forward`` keyword signature and return fields.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Literal
+
+import torch
+
+from . import lm_head, padding_free_collator
+
+
+@dataclass
+class LMOutputWithLoss:
+    """Same fields as ``olmo_core.nn.lm_head.LMOutputWithLoss``."""
+
+    logits: torch.Tensor | None
+    loss: torch.Tensor
+    ce_loss: torch.Tensor
+    z_loss: torch.Tensor | None
+
+
+class DPOLMHead(torch.nn.Module):
+    """``norm(x) -> w_out -> per-token logps`` in one fused call.
+
+    ``output.loss[b, i] = log p(labels[b, i+1] | x[b, i])`` with the label shift done internally,
+    as ``calculate_per_token_logps`` does (open_instruct/padding_free_collator.py:10-16).  The
+    ``[B, T, V]`` logits are never formed when labels are given.
+    """
+
+    def __init__(self, d_model: int, vocab_size: int, bias: bool = False, norm: torch.nn.Module | None = None,
+                 dtype: torch.dtype = torch.bfloat16, device=None):  # fmt: skip
+        super().__init__()
+        if bias:
+            raise NotImplementedError("the fused lm_head path is bias-free, like the reference's lm heads")
+        self.norm = norm
+        self.w_out = torch.nn.Linear(d_model, vocab_size, bias=False, dtype=dtype, device=device)
+        self.tp_enabled = False
+
+    def forward(
+        self,
+        x: torch.Tensor,
+        *,
+        labels: torch.Tensor | None = None,
+        ignore_index: int = -100,
+        loss_reduction: Literal["mean", "sum", "none"] = "mean",
+        z_loss_multiplier: float | None = None,
+        loss_div_factor: torch.Tensor | float | None = None,
+        return_logits: bool | None = None,
+        logits_to_keep: int | torch.Tensor = 0,
+    ) -> torch.Tensor | LMOutputWithLoss:
+        h = self.norm(x) if self.norm is not None else x
+        if labels is None:
+            # no labels: the parent class returns plain logits (library GEMM; not the fused path)
+            return self.w_out(h)
+        shifted = padding_free_collator.shift_labels(labels)
+        per_token_logps, _ = lm_head.fused_lm_head_logprobs(h, self.w_out.weight, shifted)
+        return LMOutputWithLoss(
+            logits=None, loss=per_token_logps, ce_loss=per_token_logps.detach().clone(), z_loss=None
+        )

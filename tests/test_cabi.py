@@ -1,0 +1,91 @@
+"""The C-ABI library: exported symbols, header/binding agreement, argument validation.
+
+Runs without a GPU: nothing here launches a kernel (rejected calls return before any HIP call).
+"""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import open_instruct_amd
+from open_instruct_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "oi_kernels.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    decls = {}
+    for m in re.finditer(r"\b(?:int|size_t|const char\*)\s+(oi_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+        args = m.group(2).strip()
+        n = 0 if args in ("", "void") else len([a for a in args.split(",") if a.strip()])
+        decls[m.group(1)] = n
+    return decls
+
+
+def test_library_is_built_and_loads():
+    assert os.path.exists(_lib.LIB_PATH), "build with: python -m open_instruct_amd.build"
+    lib = _lib.load()
+    assert lib.oi_version() == 1000
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    decls = _declared()
+    assert len(decls) >= 25
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name, nargs in decls.items():
+        assert hasattr(lib, name), f"{name} declared in oi_kernels.h but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature"
+        assert len(_lib.SIGNATURES[name][1]) == nargs, f"{name}: header has {nargs} args"
+    assert set(_lib.SIGNATURES) == set(decls)
+
+
+def test_error_strings():
+    lib = _lib.load()
+    assert b"NULL" in lib.oi_error_string(-2)
+    assert lib.oi_error_string(0) == b"ok"
+
+
+def test_rejected_arguments_return_codes_without_launching():
+    lib = _lib.load()
+    # vocab <= 0
+    assert lib.oi_lsg_entropy_fwd(None, 0, 1, 1, 0, 0, 0, None, 1.0, None, None, None, None) == -1
+    # null logits with rows > 0
+    assert lib.oi_lsg_entropy_fwd(None, 0, 1, 4, 0, 8, 8, None, 1.0, None, None, None, None) == -2
+    # bad temperature
+    assert lib.oi_lsg_entropy_fwd(None, 0, 1, 4, 0, 8, 8, None, 0.0, None, None, None, None) == -1
+    # empty problem is fine
+    assert lib.oi_lsg_entropy_fwd(None, 0, 0, 4, 0, 8, 8, None, 1.0, None, None, None, None) == 0
+    # hidden size not a multiple of 64
+    assert lib.oi_lmhead_logp_fwd(None, None, None, 4, 100, 32, 1.0, None, None, None, None, 0, None) == -1
+    # unknown loss function / estimator
+    assert lib.oi_grpo_terms_fwd(None, None, None, None, None, 4, 7, 0.8, 1.2, 2, None, None, None, None) == -1
+    assert lib.oi_grpo_terms_fwd(None, None, None, None, None, 4, 0, 0.8, 1.2, 9, None, None, None, None) == -1
+    assert lib.oi_grpo_terms_fwd(None, None, None, None, None, 4, 0, 0.8, 1.2, 2, None, None, None, None) == -2
+    assert lib.oi_group_advantages(None, 2, 0, 0, None, None) == -1
+    assert lib.oi_seq_logp_fwd(None, None, None, 2, 0, 0, None, None, None) == -1
+    assert lib.oi_masked_mean_workspace_bytes(4, 2, 3) == (4 + 1) * 2 * 1 * 4
+    assert lib.oi_lmhead_fwd_workspace_bytes(0, 64, 10) == 0
+    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1) > lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 0)
+
+
+def test_cpu_tensors_are_refused_loudly():
+    logits = torch.randn(2, 8)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        open_instruct_amd.model_utils.log_softmax_and_gather(logits, torch.zeros(2, dtype=torch.long))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        open_instruct_amd.rl_utils.masked_mean(torch.ones(2, 3), torch.ones(2, 3))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        open_instruct_amd.dpo_utils.dpo_loss(torch.zeros(2), torch.zeros(2), torch.zeros(2), torch.zeros(2), 0.1)
+
+
+def test_missing_library_is_an_error(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/liboi_kernels.so")
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.load()

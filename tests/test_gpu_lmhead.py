@@ -1,0 +1,141 @@
+"""GPU parity: fused lm_head + logprob/entropy (bf16 MFMA, logits never materialised), forward and
+backward, against the CPU oracle (fp32 F.linear on the upcast bf16 inputs + logsumexp).
+
+Tolerance 2e-3 abs for logprob / entropy / gradients (bf16 inputs, fp32 accumulation).
+"""
+
+import math
+
+import pytest
+import torch
+
+from open_instruct_amd import lm_head
+from open_instruct_amd.olmo_core_train_modules import DPOLMHead
+from oracle import lm_head as o_lm
+from oracle import logprob as o_logprob
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 2e-3
+
+
+def _case(n, h, v, seed, w_scale=None):
+    g = torch.Generator().manual_seed(seed)
+    hidden = torch.randn(n, h, generator=g).bfloat16()
+    weight = (torch.randn(v, h, generator=g) * (w_scale or 1.0 / math.sqrt(h))).bfloat16()
+    labels = torch.randint(0, v, (n,), generator=g)
+    return hidden, weight, labels
+
+
+@pytest.mark.parametrize(
+    "n,h,v",
+    [
+        (256, 64, 256),  # exactly one tile
+        (300, 128, 1000),  # ragged tokens and vocabulary
+        (1, 64, 50),  # single row, tiny vocabulary
+        (700, 256, 5000),  # several token tiles, partial last vocabulary tile
+        (513, 192, 20000),  # several splits of the vocabulary
+    ],
+)
+@pytest.mark.parametrize("temperature", [1.0, 0.7])
+def test_forward_matches_oracle(n, h, v, temperature):
+    print(f"case N={n} H={h} V={v} T={temperature}", flush=True)
+    hidden, weight, labels = _case(n, h, v, seed=0, w_scale=3.0 / math.sqrt(h))
+    labels[0] = v - 1
+    if n > 2:
+        labels[1], labels[2] = 0, -100
+    exp_lp, exp_ent = o_lm.lm_head_logprobs(hidden, weight, labels, temperature, True)
+    lp, ent = lm_head.fused_lm_head_logprobs(hidden.to(DEV), weight.to(DEV), labels.to(DEV), temperature, return_entropy=True)
+    assert lp.dtype == torch.float32 and lp.shape == (n,)
+    assert (lp.cpu() - exp_lp).abs().max().item() <= TOL
+    assert (ent.cpu() - exp_ent).abs().max().item() <= TOL
+    lp2, none = lm_head.fused_lm_head_logprobs(hidden.to(DEV), weight.to(DEV), labels.to(DEV), temperature)
+    assert none is None and torch.equal(lp2, lp)  # deterministic, run to run
+
+
+@pytest.mark.parametrize("n,h,v", [(256, 64, 256), (300, 128, 1000), (700, 256, 5000), (260, 64, 17000)])
+@pytest.mark.parametrize("want_dw", [True, False])
+def test_backward_matches_oracle(n, h, v, want_dw):
+    print(f"case N={n} H={h} V={v} dW={want_dw}", flush=True)
+    hidden, weight, labels = _case(n, h, v, seed=1, w_scale=3.0 / math.sqrt(h))
+    g = torch.Generator().manual_seed(2)
+    upstream = torch.randn(n, generator=g)
+    upstream[::3] = 0.0  # masked-out tokens
+    rh = hidden.float().requires_grad_(True)
+    rw = weight.float().requires_grad_(True)
+    lp, _ = o_lm.lm_head_logprobs(rh, rw, labels, 0.9)
+    lp.backward(upstream)
+    dh = hidden.to(DEV).requires_grad_(True)
+    dw = weight.to(DEV).requires_grad_(want_dw)
+    out, _ = lm_head.fused_lm_head_logprobs(dh, dw, labels.to(DEV), 0.9)
+    out.backward(upstream.to(DEV))
+    assert dh.grad.dtype == torch.bfloat16 and dh.grad.shape == hidden.shape
+    # bf16 outputs: allow one bf16 rounding of the largest entry on top of the absolute tolerance
+    tol_h = TOL + rh.grad.abs().max().item() * 2**-7
+    assert (dh.grad.float().cpu() - rh.grad).abs().max().item() <= tol_h
+    assert (dh.grad[::3] == 0).all()
+    if want_dw:
+        tol_w = TOL + rw.grad.abs().max().item() * 2**-7
+        err = (dw.grad.float().cpu() - rw.grad).abs().max().item()
+        assert err <= tol_w, (err, tol_w)
+        # relative check on the aggregate, so a dropped chunk or a transposed operand cannot hide
+        rel = (dw.grad.float().cpu() - rw.grad).norm() / rw.grad.norm()
+        assert rel.item() <= 2e-2, rel.item()
+    else:
+        assert dw.grad is None
+    rel = (dh.grad.float().cpu() - rh.grad).norm() / rh.grad.norm()
+    assert rel.item() <= 2e-2, rel.item()
+
+
+def test_mask_compaction_and_leading_shape():
+    hidden, weight, labels = _case(6 * 50, 64, 700, seed=3)
+    hidden3, labels2 = hidden.reshape(6, 50, 64), labels.reshape(6, 50)
+    g = torch.Generator().manual_seed(4)
+    mask = torch.rand(6, 50, generator=g) > 0.3
+    exp_lp, exp_ent = o_lm.lm_head_logprobs(hidden, weight, labels, 1.0, True)
+    dh = hidden3.to(DEV).requires_grad_(True)
+    lp, ent = lm_head.fused_lm_head_logprobs(dh, weight.to(DEV), labels2.to(DEV), mask=mask.to(DEV), return_entropy=True)
+    assert lp.shape == (6, 50) and ent.shape == (6, 50)
+    assert ((lp.cpu() - exp_lp.reshape(6, 50)) * mask).abs().max().item() <= TOL
+    assert ((ent.cpu() - exp_ent.reshape(6, 50)) * mask).abs().max().item() <= TOL
+    assert (lp.cpu()[~mask] == 0).all()
+    lp.sum().backward()
+    assert (dh.grad.cpu()[~mask] == 0).all() and dh.grad.cpu()[mask].abs().sum() > 0
+
+
+def test_dpo_lm_head_matches_calculate_per_token_logps():
+    """open_instruct/test_padding_free_collator.py:366-399 with the fused head."""
+    torch.manual_seed(42)
+    d_model, vocab, seq, batch = 64, 320, 10, 2
+    head = DPOLMHead(d_model=d_model, vocab_size=vocab, bias=False).to(DEV)
+    x = torch.randn(batch, seq, d_model, device=DEV).bfloat16()
+    labels = torch.randint(0, vocab, (batch, seq), device=DEV)
+    labels[0, -2:] = -100
+    output = head(x, labels=labels)
+    with torch.no_grad():
+        raw = head.w_out(x)
+    expected = o_logprob.calculate_per_token_logps(
+        torch.nn.functional.linear(x.float().cpu(), head.w_out.weight.detach().float().cpu()), labels.cpu()
+    )
+    assert output.logits is None and output.z_loss is None
+    assert output.loss.shape == (batch, seq) and output.loss.requires_grad and not output.ce_loss.requires_grad
+    assert (output.loss.detach().cpu() - expected).abs().max().item() <= TOL
+    logits = head(x[:1], labels=None)
+    assert isinstance(logits, torch.Tensor) and logits.shape == (1, seq, vocab) and torch.equal(logits, raw[:1])
+
+
+def test_fused_equals_materialised_path_on_device():
+    """A mid-sized shape where the CPU oracle would be slow: the fused kernel must agree with the
+    row-wise kernel run on logits materialised by a library GEMM in fp32."""
+    from open_instruct_amd import model_utils
+
+    n, h, v = 2048, 1024, 32000
+    torch.manual_seed(0)
+    hidden = torch.randn(n, h, device=DEV).bfloat16()
+    weight = (torch.randn(v, h, device=DEV) * 0.02).bfloat16()
+    labels = torch.randint(0, v, (n,), device=DEV)
+    logits = hidden.float() @ weight.float().t()
+    exp_lp, exp_ent = model_utils.logprob_and_entropy(logits, labels)
+    lp, ent = lm_head.fused_lm_head_logprobs(hidden, weight, labels, return_entropy=True)
+    assert (lp - exp_lp).abs().max().item() <= TOL
+    assert (ent - exp_ent).abs().max().item() <= TOL

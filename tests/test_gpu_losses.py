@@ -1,0 +1,418 @@
+"""GPU parity: GRPO / DPO loss kernels and masked reductions against the CPU oracle and the
+reference's known-answer vectors (tests/golden/reference_known_answers.json)."""
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_grpo_config
+from open_instruct_amd import dpo_utils, grpo_utils, model_utils, padding_free_collator, rl_utils
+from oracle import dpo as o_dpo
+from oracle import grpo as o_grpo
+from oracle import logprob as o_logprob
+from oracle import reductions as o_red
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 1e-5
+
+
+def _close(a, b, tol=TOL):
+    a, b = a.detach().float().cpu(), b.detach().float().cpu()
+    assert a.shape == b.shape, (a.shape, b.shape)
+    scale = max(1.0, b.abs().max().item()) if b.numel() else 1.0
+    err = (a - b).abs().max().item() if b.numel() else 0.0
+    assert err <= tol * scale, err
+
+
+# ------------------------------------------------------------------ masked_mean
+def test_masked_mean_reference_known_answers(golden):
+    for case in golden["masked_mean"]:
+        out = rl_utils.masked_mean(torch.tensor(case["values"], device=DEV), torch.tensor(case["mask"], device=DEV), axis=case["axis"])
+        exp = torch.tensor(case["expected"])
+        assert out.shape == exp.shape, case["source"]
+        assert torch.allclose(out.cpu(), exp, rtol=1e-6, atol=0), case["source"]
+
+
+@pytest.mark.parametrize("axis", [None, 1, 0, -1])
+@pytest.mark.parametrize("denominator", [None, 37.5])
+@pytest.mark.parametrize("bool_mask", [True, False])
+def test_masked_mean_random_and_gradient(axis, denominator, bool_mask):
+    g = torch.Generator().manual_seed(0)
+    values = torch.randn(4, 6, 2500, generator=g)
+    mask = torch.rand(6, 2500, generator=g) > 0.4
+    mask[2] = False  # an empty row
+    m = mask if bool_mask else mask.float()
+    ref_v = values.clone().requires_grad_(True)
+    ref = o_red.masked_mean(ref_v, m, axis, denominator)
+    upstream = torch.randn(4, generator=g)
+    ref.backward(upstream)
+    dv = values.to(DEV).requires_grad_(True)
+    out = rl_utils.masked_mean(dv, m.to(DEV), axis, denominator)
+    out.backward(upstream.to(DEV))
+    _close(out, ref)
+    assert (dv.grad.cpu() - ref_v.grad).abs().max().item() <= 1e-7 + 1e-5 * ref_v.grad.abs().max().item()
+
+
+def test_masked_mean_scalar_cases():
+    v = torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]], device=DEV)
+    m = torch.tensor([[True, True, False], [True, False, False]], device=DEV)
+    assert rl_utils.masked_mean(v, m, None, 10.0).item() == pytest.approx(0.7)
+    assert rl_utils.masked_mean(v, m, None, 0.0).item() == 0.0
+    assert rl_utils.masked_mean(v, torch.zeros_like(m)).item() == 0.0
+
+
+# ------------------------------------------------------------------ compute_grpo_loss
+def test_grpo_known_answers_on_device(golden):
+    case = golden["dapo_clipping"]
+    cfg = make_grpo_config(clip_lower=case["clip_lower"], clip_higher=case["clip_higher"])
+    ratio = torch.tensor(case["ratio"], device=DEV)
+    pg, clipfrac, kl = grpo_utils.compute_grpo_loss(
+        torch.randn(1, 3, device=DEV), ratio, torch.tensor(case["advantages"], device=DEV), None, cfg, torch.ones_like(ratio)
+    )
+    assert torch.allclose(pg.cpu(), torch.tensor(case["expected_pg_loss"]))
+    assert torch.equal(clipfrac.cpu(), torch.tensor(case["expected_clipfrac"]))
+    assert torch.equal(kl.cpu(), torch.zeros(1, 3))
+    case = golden["dapo_negative_advantages"]
+    cfg = make_grpo_config(clip_lower=case["clip_lower"], clip_higher=case["clip_higher"])
+    ratio = torch.tensor(case["ratio"], device=DEV)
+    pg, _, _ = grpo_utils.compute_grpo_loss(
+        torch.zeros_like(ratio), ratio, torch.full_like(ratio, case["advantage"]), None, cfg, torch.ones_like(ratio)
+    )
+    assert torch.allclose(pg.cpu(), torch.tensor(case["expected_pg_loss"]))
+    case = golden["cispo"]
+    cfg = make_grpo_config(loss_fn="cispo", clip_higher=case["clip_higher"])
+    ratio = torch.tensor(case["ratio"], device=DEV, requires_grad=True)
+    new = torch.randn(1, 3, device=DEV, requires_grad=True)
+    pg, clipfrac, _ = grpo_utils.compute_grpo_loss(new, ratio, torch.tensor(case["advantages"], device=DEV), None, cfg, torch.ones(1, 3, device=DEV))
+    pg.sum().backward()
+    assert new.grad is not None and (ratio.grad is None or (ratio.grad == 0).all())
+    assert torch.equal(clipfrac.cpu(), torch.tensor(case["expected_clipfrac"]))
+
+
+def _grpo_inputs(seed, shape=(5, 300), edge=False):
+    g = torch.Generator().manual_seed(seed)
+    new = -torch.rand(shape, generator=g) * 5
+    old = new + 0.3 * torch.randn(shape, generator=g)
+    ref = new + 0.5 * torch.randn(shape, generator=g)
+    adv = torch.randn(shape, generator=g)
+    adv[0, :10] = 0.0
+    mask = torch.rand(shape, generator=g) > 0.3
+    rho = torch.rand(shape, generator=g) * 2
+    rho[1, :20] = 0.0
+    if edge:
+        ref[2, :5] = new[2, :5] - 100.0  # outside the +-40 clamp
+        old[3, :5] = new[3, :5]  # ratio exactly 1
+    return new, old, ref, adv, mask, rho
+
+
+@pytest.mark.parametrize("loss_fn", ["dapo", "cispo"])
+@pytest.mark.parametrize("kl_estimator", [0, 1, 2, 3])
+@pytest.mark.parametrize("with_ref", [True, False])
+def test_compute_grpo_loss_parity_and_gradients(loss_fn, kl_estimator, with_ref):
+    new, old, ref, adv, _, rho = _grpo_inputs(1, edge=True)
+    cfg = make_grpo_config(loss_fn=loss_fn, clip_higher=0.28, kl_estimator=kl_estimator)
+    g = torch.Generator().manual_seed(2)
+    up_pg, up_kl = torch.randn(new.shape, generator=g), torch.randn(new.shape, generator=g)
+
+    def run(mod, dev):
+        n = new.to(dev).requires_grad_(True)
+        ratio = torch.exp(n - old.to(dev))
+        ratio.retain_grad()
+        pg, cf, kl = mod.compute_grpo_loss(n, ratio, adv.to(dev), ref.to(dev) if with_ref else None, cfg, rho.to(dev))
+        (pg * up_pg.to(dev) + kl * up_kl.to(dev)).sum().backward()
+        return pg, cf, kl, n.grad
+
+    e_pg, e_cf, e_kl, e_grad = run(o_grpo, "cpu")
+    pg, cf, kl, grad = run(grpo_utils, DEV)
+    _close(pg, e_pg)
+    assert torch.equal(cf.cpu(), e_cf)
+    _close(kl, e_kl, 2e-5)
+    _close(grad, e_grad, 2e-5)
+    assert pg.requires_grad and not cf.requires_grad
+
+
+def test_rho_correction_known_answers_on_device(golden):
+    case = golden["rho_mask"]
+    cfg = make_grpo_config(use_rho_correction=True, rho_mask_lower_bound=case["mask_lower"], rho_mask_upper_bound=case["mask_upper"])
+    old = torch.log(torch.tensor(case["rho"])).to(DEV)
+    zeros, ones = torch.zeros_like(old), torch.ones_like(old)
+    c = grpo_utils.compute_rho_correction(old, zeros, torch.tensor(case["response_mask"], device=DEV), ones, cfg)
+    assert torch.allclose(c.weights.cpu(), torch.tensor(case["expected_weights"]))
+    assert torch.equal(c.metrics["val/rho_drop_low_frac"].cpu(), torch.tensor(case["expected_drop_low"]))
+    assert torch.equal(c.metrics["val/rho_drop_high_frac"].cpu(), torch.tensor(case["expected_drop_high"]))
+    c = grpo_utils.compute_rho_correction(old, zeros, torch.tensor(case["response_mask_with_pad"], device=DEV), ones, cfg)
+    assert torch.allclose(c.weights.cpu(), torch.tensor(case["expected_weights_with_pad"]))
+    assert torch.equal(c.metrics["val/rho_drop_low_frac"].cpu(), torch.tensor(case["expected_drop_low_with_pad"]))
+    for key, extra in (("rho_mask_sequence_level", {"rho_mask_sequence_level": True}), ("rho_mask_tv_divergence", {"rho_mask_tv_divergence": True})):
+        case = golden[key]
+        cfg = make_grpo_config(use_rho_correction=True, rho_mask_lower_bound=case["mask_lower"], rho_mask_upper_bound=case["mask_upper"], **extra)
+        old = torch.log(torch.tensor(case["rho"])).to(DEV)
+        c = grpo_utils.compute_rho_correction(old, torch.zeros_like(old), torch.ones_like(old, dtype=torch.bool), torch.ones_like(old), cfg)
+        assert torch.allclose(c.weights.cpu(), torch.tensor(case["expected_weights"])), key
+        assert torch.equal(c.metrics["val/rho_drop_high_frac"].cpu(), torch.tensor(case["expected_drop_high"])), key
+
+
+@pytest.mark.parametrize("seq_level,tv", [(False, False), (True, False), (False, True)])
+def test_rho_correction_random_parity(seq_level, tv):
+    new, old, _, adv, mask, _ = _grpo_inputs(3, shape=(7, 700))
+    vl = old + 0.4 * torch.randn(old.shape, generator=torch.Generator().manual_seed(4))
+    vl[~mask] = float("nan")  # vLLM logprobs are NaN on query tokens
+    cfg = make_grpo_config(
+        use_rho_correction=True, rho_mask_sequence_level=seq_level, rho_mask_tv_divergence=tv, rho_mask_lower_bound=0.6,
+        rho_mask_upper_bound=1.6 if not tv else 0.3, rho_clamp_lower_bound=0.7, rho_clamp_upper_bound=1.4,
+    )  # fmt: skip
+    exp = o_grpo.compute_rho_correction(old, vl, mask, adv, cfg)
+    got = grpo_utils.compute_rho_correction(old.to(DEV), vl.to(DEV), mask.to(DEV), adv.to(DEV), cfg)
+    _close(got.weights, exp.weights)
+    for k in exp.metrics:
+        _close(got.metrics[k], exp.metrics[k])
+    _close(got.histogram_metrics["val/rho_hist"], exp.histogram_metrics["val/rho_hist"])
+    off = grpo_utils.compute_rho_correction(old.to(DEV), vl.to(DEV), mask.to(DEV), adv.to(DEV), make_grpo_config())
+    assert (off.weights == 1).all() and off.metrics == {}
+
+
+def test_mask_logprobs_and_estimate_kl():
+    lp = torch.tensor([[0.5, float("nan"), -3.0, -1.0]], device=DEV, requires_grad=True)
+    mask = torch.tensor([[True, True, False, True]], device=DEV)
+    out = grpo_utils.mask_logprobs(lp, mask)
+    assert out.tolist() == [[0.5, 1.0, 1.0, -1.0]]
+    out.sum().backward()
+    assert lp.grad.tolist() == [[1.0, 0.0, 0.0, 1.0]]
+    assert (grpo_utils.mask_logprobs(lp.detach(), torch.zeros_like(mask)) == grpo_utils.INVALID_LOGPROB).all()
+    g = torch.Generator().manual_seed(5)
+    d = (torch.randn(3, 50, generator=g) * 3).clamp(-40, 40)
+    ratio = torch.randn(3, 50, generator=g).exp()
+    up = torch.randn(4, 3, 50, generator=g)
+    rd, rr = d.clone().requires_grad_(True), ratio.clone().requires_grad_(True)
+    exp = o_logprob.estimate_kl(rd, rr)
+    exp.backward(up)
+    gd, gr = d.to(DEV).requires_grad_(True), ratio.to(DEV).requires_grad_(True)
+    got = model_utils.estimate_kl(gd, gr)
+    got.backward(up.to(DEV))
+    assert got.shape == (4, 3, 50)
+    _close(got, exp)
+    _close(gd.grad, rd.grad)
+    _close(gr.grad, rr.grad)
+
+
+# ------------------------------------------------------------------ fused scalar loss
+@pytest.mark.parametrize("loss_fn", ["dapo", "cispo"])
+@pytest.mark.parametrize("axis,denominator", [(None, None), (None, 1234.0), (1, None)])
+@pytest.mark.parametrize("with_old", [True, False])
+def test_grpo_loss_fused_parity(loss_fn, axis, denominator, with_old):
+    new, old, ref, adv, mask, rho = _grpo_inputs(6, shape=(9, 2100), edge=True)
+    mask[4] = False  # a row without response tokens
+    ent = torch.rand(new.shape, generator=torch.Generator().manual_seed(7)) * 3
+    cfg = make_grpo_config(loss_fn=loss_fn, clip_higher=0.28, beta=0.05)
+    rn = new.clone().requires_grad_(True)
+    o_old = old if with_old else rn.detach()
+    e_loss, e_pg, e_cf, _, e_ratio = o_grpo.grpo_token_loss(rn, o_old, ref, adv, mask, cfg, rho, denominator, axis, dp_scale=2.0)
+    e_loss.backward()
+    dn = new.to(DEV).requires_grad_(True)
+    loss, stats = grpo_utils.grpo_loss_fused(
+        dn, old.to(DEV) if with_old else None, ref.to(DEV), adv.to(DEV), mask.to(DEV), cfg, rho.to(DEV), ent.to(DEV),
+        loss_denominator=denominator, axis=axis, dp_scale=2.0,
+    )  # fmt: skip
+    loss.backward()
+    _close(loss, e_loss, 2e-5)
+    assert (dn.grad.cpu() - rn.grad).abs().max().item() <= 2e-5 * max(1e-6, rn.grad.abs().max().item()) + 1e-9
+    # statistics recorded by populate_sample_loss_stats in the reference
+    d = (rn.detach() - ref).clamp(-40, 40)
+    kl4 = o_red.masked_mean(o_logprob.estimate_kl(d, e_ratio.detach()), mask)
+    for j in range(4):
+        _close(stats[f"objective/kl{j}_avg"], kl4[j], 2e-5)
+    _close(stats["loss/policy_avg"], o_red.masked_mean(e_pg.detach(), mask), 2e-5)
+    _close(stats["policy/clipfrac_avg"], o_red.masked_mean(e_cf, mask), 2e-5)
+    _close(stats["val/ratio"], o_red.masked_mean(e_ratio.detach(), mask), 2e-5)
+    _close(stats["policy/entropy_avg"], o_red.masked_mean(ent, mask), 2e-5)
+    assert stats["num_response_tokens"].item() == float(mask.sum())
+    assert stats["loss/total_avg"].item() == loss.item()
+
+
+def test_grpo_loss_fused_empty_mask_is_zero():
+    new, old, ref, adv, mask, _ = _grpo_inputs(8, shape=(2, 50))
+    cfg = make_grpo_config()
+    dn = new.to(DEV).requires_grad_(True)
+    loss, stats = grpo_utils.grpo_loss_fused(dn, old.to(DEV), ref.to(DEV), adv.to(DEV), torch.zeros_like(mask).to(DEV), cfg)
+    loss.backward()
+    assert loss.item() == 0.0 and (dn.grad == 0).all() and stats["num_response_tokens"].item() == 0.0
+
+
+def test_group_advantages_on_device():
+    rng = np.random.default_rng(0)
+    scores = (rng.random(64) < 0.3).astype(np.float64)
+    scores[8:16] = 1.0
+    for mode in ("standard", "centered"):
+        exp = o_grpo.group_advantages(scores, 8, mode).astype(np.float32)
+        got = grpo_utils.group_advantages(torch.tensor(scores, device=DEV), 8, mode).cpu().numpy()
+        assert np.array_equal(got, exp), mode  # Bernoulli rewards: sums are exact, so fp32 results are bit-equal
+    assert (got[8:16] == 0).all()
+    cont = rng.normal(size=48)
+    got = grpo_utils.group_advantages(torch.tensor(cont, device=DEV), 16).cpu().numpy()
+    assert np.abs(got - o_grpo.group_advantages(cont, 16)).max() <= 1e-6
+
+
+# ------------------------------------------------------------------ per-sequence logps and DPO
+def test_get_batch_logps_padded_known_answers(golden):
+    for case in golden["get_batch_logps_padded_average"]:
+        out = dpo_utils._get_batch_logps(
+            torch.tensor(case["per_token_logps"], device=DEV), torch.tensor(case["labels"], device=DEV), average_log_prob=True
+        )
+        assert torch.equal(out.cpu(), torch.tensor(case["expected"])), case["source"]
+
+
+@pytest.mark.parametrize("average", [False, True])
+def test_seq_logps_packed_and_padded_parity(average):
+    g = torch.Generator().manual_seed(9)
+    lens = [700, 1, 1300, 64, 5, 2048]
+    rows, labs = [], []
+    for n in lens:
+        rows.append(-torch.rand(n, generator=g) * 4)
+        lab = torch.randint(0, 1000, (n,), generator=g)
+        lab[: max(1, n // 3)] = -100
+        labs.append(lab)
+    labs[3][:] = -100  # a fully masked sequence
+    per_token = torch.cat(rows).unsqueeze(0)
+    labels = torch.cat(labs).unsqueeze(0)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    up = torch.randn(len(lens), generator=g)
+    rp = per_token.clone().requires_grad_(True)
+    exp = o_red.get_batch_logps_packed(rp, labels, cu, average)
+    exp.backward(up)
+    dp = per_token.to(DEV).requires_grad_(True)
+    got = padding_free_collator.get_batch_logps(dp, labels.to(DEV), cu.to(DEV), average)
+    got.backward(up.to(DEV))
+    _close(got, exp, 2e-6)
+    assert not torch.isnan(got).any()
+    assert torch.equal(dp.grad.cpu(), rp.grad)  # each position gets its sequence's upstream value (or 0): bit-exact
+    # padded layout
+    tmax = max(lens)
+    pt = torch.zeros(len(lens), tmax)
+    lb = torch.full((len(lens), tmax), -100)
+    for i, n in enumerate(lens):
+        pt[i, :n], lb[i, :n] = rows[i], labs[i]
+    rp2 = pt.clone().requires_grad_(True)
+    exp2 = o_red.get_batch_logps_padded(rp2, lb, average)
+    exp2.backward(up)
+    dp2 = pt.to(DEV).requires_grad_(True)
+    got2 = dpo_utils._get_batch_logps(dp2, lb.to(DEV), average)
+    got2.backward(up.to(DEV))
+    _close(got2, exp2, 2e-6)
+    assert torch.equal(dp2.grad.cpu(), rp2.grad)
+    _close(got2, got, 2e-6)  # packed == padded
+
+
+def test_packed_all_masked_segment(golden):
+    case = golden["packed_cu_seq_lens"]
+    g = torch.Generator().manual_seed(10)
+    logits = torch.randn(1, case["seq_len"], 100, generator=g)
+    labels = torch.ones(1, case["seq_len"], dtype=torch.long)
+    lo, hi = case["masked_label_range"]
+    labels[0, lo:hi] = -100
+    cu = torch.tensor(case["cu_seq_lens"])
+    per_token = padding_free_collator.calculate_per_token_logps(logits.to(DEV), labels.to(DEV))
+    out = padding_free_collator.get_batch_logps(per_token, labels.to(DEV), cu.to(DEV), average_log_prob=True)
+    exp = o_red.get_batch_logps_packed(o_logprob.calculate_per_token_logps(logits, labels), labels, cu, True)
+    assert out.shape[0] == case["expected_num_outputs"] and not torch.isnan(out).any()
+    _close(out, exp)
+
+
+@pytest.mark.parametrize("label_smoothing", [0.0, 0.1])
+@pytest.mark.parametrize("reference_free", [False, True])
+def test_dpo_loss_parity_and_gradients(label_smoothing, reference_free, golden):
+    g = torch.Generator().manual_seed(11)
+    pc, pr = torch.randn(8, generator=g) * 30 - 400, torch.randn(8, generator=g) * 30 - 400
+    rc, rr = torch.randn(8, generator=g) * 50 - 400, torch.randn(8, generator=g) * 50 - 400
+    up = torch.randn(8, generator=g)
+
+    def run(mod, dev):
+        a, b = pc.to(dev).requires_grad_(True), pr.to(dev).requires_grad_(True)
+        losses, cr, rj = mod.dpo_loss(a, b, rc.to(dev), rr.to(dev), 0.1, reference_free, label_smoothing)
+        losses.backward(up.to(dev))
+        return losses, cr, rj, a.grad, b.grad
+
+    e = run(o_dpo, "cpu")
+    o = run(dpo_utils, DEV)
+    for got, exp in zip(o, e):
+        _close(got, exp, 2e-6)
+    assert not o[1].requires_grad and not o[2].requires_grad
+    case = golden["dpo_loss_zero_margin"]
+    losses, _, _ = dpo_utils.dpo_loss(*(torch.tensor(case[k], device=DEV) for k in ("policy_chosen", "policy_rejected", "ref_chosen", "ref_rejected")), beta=case["beta"])
+    assert torch.allclose(losses.cpu(), torch.tensor(case["expected_losses"]), atol=1e-7)
+
+
+def test_simpo_wpo_and_compute_loss_dispatch():
+    g = torch.Generator().manual_seed(12)
+    pc, pr = -torch.rand(1, generator=g) * 2, -torch.rand(1, generator=g) * 2
+    rc, rr = -torch.rand(1, generator=g) * 2, -torch.rand(1, generator=g) * 2
+    exp = o_dpo.simpo_loss(pc, pr, 2.0, 0.5, 0.1)
+    got = dpo_utils.simpo_loss(pc.to(DEV), pr.to(DEV), 2.0, 0.5, 0.1)
+    for a, b in zip(got, exp):
+        _close(a, b, 2e-6)
+    mask = torch.tensor([[True, False, True, True]])
+    a = pc.clone().requires_grad_(True)
+    exp = o_dpo.wpo_loss(a, pr, rc, rr, 0.3, mask, mask)
+    exp[0].sum().backward()
+    b = pc.to(DEV).requires_grad_(True)
+    got = dpo_utils.wpo_loss(b, pr.to(DEV), rc.to(DEV), rr.to(DEV), 0.3, mask.to(DEV), mask.to(DEV))
+    got[0].sum().backward()
+    _close(got[0], exp[0], 2e-6)
+    _close(b.grad, a.grad, 2e-6)
+
+    class Args:
+        loss_type, beta, label_smoothing, gamma_beta_ratio = "dpo_norm", 0.1, 0.0, 0.3
+
+    class Cache:
+        def __getitem__(self, index):
+            return {"chosen_logps": rc.to(DEV)[index], "rejected_logps": rr.to(DEV)[index]}
+
+    out = dpo_utils.compute_loss(Args, {"index": torch.tensor([0], device=DEV)}, pc.to(DEV), pr.to(DEV), Cache())
+    _close(out[0], o_dpo.dpo_loss(pc, pr, rc, rr, 0.1)[0], 2e-6)
+    Args.loss_type = "bogus"
+    with pytest.raises(ValueError):
+        dpo_utils.compute_loss(Args, {}, pc.to(DEV), pr.to(DEV), None)
+
+
+def test_forward_for_logprobs_and_compute_logprobs_with_mock_model():
+    """Mirrors open_instruct/test_olmo_core_train_modules.py:49-131 with a stub model returning fixed logits."""
+    from open_instruct_amd.data_types import CollatedBatchData
+
+    g = torch.Generator().manual_seed(13)
+    b, t, v = 2, 5, 10
+    logits = torch.randn(b, t, v, generator=g)
+
+    class Model(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.z = torch.nn.Parameter(logits.to(DEV))
+
+        def forward(self, input_ids, attention_mask=None, position_ids=None):
+            return self.z[: input_ids.shape[0]]
+
+    model = Model()
+    qr = torch.randint(1, v, (b, t), generator=g)
+    pos = torch.arange(t).unsqueeze(0).expand(b, -1)
+    lp1, ent1 = grpo_utils.forward_for_logprobs(model, qr.to(DEV), None, pos.to(DEV), 0, 1.0, return_entropy=True)
+    lp2, _ = grpo_utils.forward_for_logprobs(model, qr.to(DEV), None, pos.to(DEV), 0, 0.5)
+    e_lp, e_ent = o_grpo.forward_for_logprobs(logits, qr, 0, 1.0, True)
+    assert lp1.shape == (b, t - 1) and ent1.shape == (b, t - 1)
+    assert (lp1 <= 0).all() and (ent1 >= 0).all() and lp1.requires_grad and not ent1.requires_grad
+    assert not torch.allclose(lp1, lp2)
+    _close(lp1, e_lp)
+    _close(ent1, e_ent)
+    mask = torch.ones(b, t, dtype=torch.bool)
+    mask[:, :2] = False
+    data = CollatedBatchData(
+        query_responses=[qr.to(DEV), qr.to(DEV)], attention_masks=[torch.ones(b, t, dtype=torch.long, device=DEV)] * 2,
+        position_ids=[pos.to(DEV)] * 2, advantages=[torch.randn(b, t, device=DEV)] * 2,
+        response_masks=[mask.to(DEV), torch.zeros_like(mask).to(DEV)], vllm_logprobs=[torch.randn(b, t - 1, device=DEV)] * 2,
+    )  # fmt: skip
+    model1 = Model()
+    out = grpo_utils.compute_logprobs(model1, data, pad_token_id=0, temperature=1.0, use_grad=True)
+    assert len(out) == 2 and out[0].shape == (b, t - 1) and out[0].requires_grad
+    assert (out[0] <= grpo_utils.INVALID_LOGPROB).all()
+    assert (out[1] == grpo_utils.INVALID_LOGPROB).all()  # all-masked sample
+    assert (out[0][:, 0] == grpo_utils.INVALID_LOGPROB).all()
+    counts = grpo_utils.calculate_token_counts(1, data, torch.device(DEV))
+    assert counts == {0: float(mask[:, 1:].sum()), 1: 0.0}

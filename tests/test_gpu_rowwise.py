@@ -1,0 +1,206 @@
+"""GPU parity: row-wise logprob / entropy kernels (through the Python surface and the raw C-ABI)
+against the CPU oracle on the same seeded inputs.
+
+Tolerances (stated by the north star): 1e-5 abs for fp32 logits, 2e-3 abs for bf16/fp16 logits,
+both against the fp32-accumulate oracle.  Index handling is bit-exact by construction (checked
+through values that would differ by O(1) on any mis-indexing).
+"""
+
+import math
+
+import pytest
+import torch
+
+from open_instruct_amd import _lib, model_utils, padding_free_collator
+from oracle import logprob as o_logprob
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _tol(dtype):
+    return 1e-5 if dtype == torch.float32 else 2e-3
+
+
+def _case(shape, vocab, dtype, scale, seed):
+    g = torch.Generator().manual_seed(seed)
+    logits = (torch.randn(*shape, vocab, generator=g) * scale).to(dtype)
+    index = torch.randint(0, vocab, shape, generator=g)
+    return logits, index
+
+
+@pytest.mark.parametrize(
+    "shape,vocab,dtype,scale",
+    [
+        ((4, 512), 32000, torch.float32, 2.0),  # BASELINE config 1
+        ((3, 7), 10, torch.float32, 1.0),
+        ((5,), 1000, torch.float32, 3.0),
+        ((2, 33), 151936, torch.float32, 1.0),  # vocabulary of the reference's own test
+        ((2, 64), 128256, torch.bfloat16, 3.0),  # BASELINE config 2 rows
+        ((6, 5), 4099, torch.bfloat16, 3.0),  # odd vocab: rows not 16-byte aligned
+        ((2, 9), 50257, torch.float16, 2.0),
+        ((1, 1), 3, torch.float32, 1.0),
+    ],
+)
+@pytest.mark.parametrize("temperature", [1.0, 0.7])
+def test_logprob_and_entropy_forward(shape, vocab, dtype, scale, temperature):
+    logits, index = _case(shape, vocab, dtype, scale, seed=0)
+    print(f"case shape={shape} V={vocab} dtype={dtype} T={temperature}", flush=True)
+    exp_lp = o_logprob.log_softmax_and_gather(logits, index, torch.float32, temperature)
+    exp_ent = o_logprob.entropy_from_logits(logits, torch.float32, temperature)
+    lg, ix = logits.to(DEV), index.to(DEV)
+    lp = model_utils.log_softmax_and_gather(lg, ix, temperature=temperature)
+    ent = model_utils.entropy_from_logits(lg, temperature=temperature)
+    both_lp, both_ent = model_utils.logprob_and_entropy(lg, ix, temperature=temperature)
+    assert lp.dtype == torch.float32 and lp.shape == index.shape
+    tol = _tol(dtype)
+    assert (lp.cpu() - exp_lp).abs().max().item() <= tol
+    assert (ent.cpu() - exp_ent).abs().max().item() <= tol
+    assert torch.equal(both_lp, lp) and torch.equal(both_ent, ent)  # one pass == two passes, bitwise
+    assert (lp <= 0).all() and torch.isfinite(lp).all() and (ent >= -tol).all()
+
+
+def test_sliced_non_contiguous_view_like_reference_test():
+    # open_instruct/test_model_utils.py:49-64 at the reference's vocabulary size
+    g = torch.Generator().manual_seed(1)
+    full = torch.randn(2, 41, 151936, generator=g)
+    index = torch.randint(0, 151936, (2, 41), generator=g)[:, 1:].clone()
+    view = full.to(DEV)[:, :-1, :]
+    assert not view.is_contiguous()
+    out = model_utils.log_softmax_and_gather(view, index.to(DEV))
+    exp = o_logprob.log_softmax_and_gather(full[:, :-1], index)
+    assert out.shape == (2, 40) and (out <= 0).all() and torch.isfinite(out).all()
+    assert (out.cpu() - exp).abs().max().item() <= 1e-5
+    # drop_last=True on the full tensor is the same computation
+    lp2, _ = model_utils.logprob_and_entropy(full.to(DEV), index.to(DEV), drop_last=True, want_entropy=False)
+    assert torch.equal(lp2, out)
+
+
+def test_out_dtype_and_index_edge_values():
+    logits, index = _case((4,), 257, torch.bfloat16, 2.0, seed=2)
+    index[0], index[1] = 0, 256  # first and last vocabulary entry
+    out = model_utils.log_softmax_and_gather(logits.to(DEV), index.to(DEV), out_dtype=torch.bfloat16)
+    assert out.dtype == torch.bfloat16
+    exp = o_logprob.log_softmax_and_gather(logits, index)
+    assert (out.float().cpu() - exp).abs().max().item() <= 0.05  # one bf16 rounding of values around -6
+    # out-of-range ids are clamped into the vocabulary instead of faulting
+    bad = torch.tensor([-5, 300, 1, 2])
+    got = model_utils.log_softmax_and_gather(logits.to(DEV), bad.to(DEV))
+    ref = o_logprob.log_softmax_and_gather(logits, torch.tensor([0, 256, 1, 2]))
+    assert (got.cpu() - ref).abs().max().item() <= 2e-3
+
+
+def test_closed_forms_on_device():
+    v = 4096
+    uniform = torch.full((3, v), 0.25, device=DEV)
+    assert (model_utils.entropy_from_logits(uniform).cpu() - math.log(v)).abs().max().item() <= 1e-5
+    lp = model_utils.log_softmax_and_gather(uniform, torch.tensor([0, 7, v - 1], device=DEV))
+    assert (lp.cpu() + math.log(v)).abs().max().item() <= 1e-5
+    peaked = torch.zeros(1, v, device=DEV)
+    peaked[0, 17] = 80.0
+    assert abs(model_utils.entropy_from_logits(peaked).item()) <= 1e-5
+    assert abs(model_utils.log_softmax_and_gather(peaked, torch.tensor([17], device=DEV)).item()) <= 1e-5
+    # huge logits do not overflow
+    big = torch.randn(2, v, device=DEV) * 3 + 3.0e4
+    assert torch.isfinite(model_utils.log_softmax_and_gather(big, torch.zeros(2, dtype=torch.long, device=DEV))).all()
+
+
+@pytest.mark.parametrize(
+    "shape,vocab,dtype",
+    [((3, 17), 32000, torch.float32), ((2, 9), 128256, torch.bfloat16), ((5,), 4099, torch.bfloat16), ((2, 3), 10, torch.float32)],
+)
+@pytest.mark.parametrize("temperature", [1.0, 0.7])
+def test_backward_matches_oracle_autograd(shape, vocab, dtype, temperature):
+    logits, index = _case(shape, vocab, dtype, 3.0, seed=3)
+    g = torch.Generator().manual_seed(4)
+    upstream = torch.randn(shape, generator=g)
+    upstream.view(-1)[0] = 0.0  # a masked-out token: its gradient row must be exactly zero
+    ref_in = logits.float().requires_grad_(True)
+    o_logprob.log_softmax_and_gather(ref_in, index, None, temperature).backward(upstream)
+    lg = logits.to(DEV).requires_grad_(True)
+    model_utils.log_softmax_and_gather(lg, index.to(DEV), temperature=temperature).backward(upstream.to(DEV))
+    assert lg.grad.dtype == dtype and lg.grad.shape == logits.shape
+    err = (lg.grad.float().cpu() - ref_in.grad).abs().max().item()
+    assert err <= _tol(dtype), err
+    assert (lg.grad.reshape(-1, vocab)[0] == 0).all()
+    # every gradient row sums to ~0 (sum_j (onehot_j - p_j) = 0)
+    rows = lg.grad.float().reshape(-1, vocab).sum(-1).cpu()
+    bound = 1e-4 if dtype == torch.float32 else 0.05
+    assert rows.abs().max().item() <= bound * max(1.0, upstream.abs().max().item())
+
+
+def test_backward_through_sliced_view_and_drop_last():
+    g = torch.Generator().manual_seed(5)
+    full = torch.randn(2, 6, 515, generator=g)
+    index = torch.randint(0, 515, (2, 5), generator=g)
+    upstream = torch.randn(2, 5, generator=g)
+    ref_in = full.clone().requires_grad_(True)
+    o_logprob.log_softmax_and_gather(ref_in[:, :-1], index, None, 0.9).backward(upstream)
+    a = full.to(DEV).requires_grad_(True)
+    model_utils.log_softmax_and_gather(a[:, :-1], index.to(DEV), temperature=0.9).backward(upstream.to(DEV))
+    b = full.to(DEV).requires_grad_(True)
+    lp, ent = model_utils.logprob_and_entropy(b, index.to(DEV), temperature=0.9, drop_last=True)
+    assert not ent.requires_grad
+    lp.backward(upstream.to(DEV))
+    for grad in (a.grad, b.grad):
+        assert (grad.cpu() - ref_in.grad).abs().max().item() <= 1e-5
+        assert (grad[:, -1] == 0).all()
+
+
+def test_calculate_per_token_logps_matches_oracle():
+    g = torch.Generator().manual_seed(6)
+    logits = (torch.randn(2, 40, 2048, generator=g) * 2).bfloat16()
+    labels = torch.randint(0, 2048, (2, 40), generator=g)
+    labels[0, :7] = -100
+    labels[1, 30:] = -100
+    out = padding_free_collator.calculate_per_token_logps(logits.to(DEV), labels.to(DEV))
+    exp = o_logprob.calculate_per_token_logps(logits, labels)
+    assert out.dtype == torch.float32 and out.shape == (2, 40)
+    assert (out.cpu() - exp).abs().max().item() <= 2e-3
+
+
+def test_raw_c_abi_call():
+    """The same kernel through ctypes only: plain pointers and sizes, no torch types in the call."""
+    lib = _lib.load()
+    logits, index = _case((8,), 777, torch.float32, 2.0, seed=7)
+    lg, ix = logits.to(DEV), index.to(DEV)
+    lp = torch.empty(8, device=DEV)
+    ent = torch.empty(8, device=DEV)
+    lse = torch.empty(8, device=DEV)
+    rc = lib.oi_lsg_entropy_fwd(lg.data_ptr(), 0, 1, 8, 0, 777, 777, ix.data_ptr(), 1.0, lp.data_ptr(), ent.data_ptr(),
+                                lse.data_ptr(), torch.cuda.current_stream().cuda_stream)  # fmt: skip
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert (lp.cpu() - o_logprob.log_softmax_and_gather(logits, index)).abs().max().item() <= 1e-5
+    assert (lse.cpu() - torch.logsumexp(logits, -1)).abs().max().item() <= 1e-5
+    dl = torch.empty_like(lg)
+    grad = torch.ones(8, device=DEV)
+    rc = lib.oi_lsg_bwd(lg.data_ptr(), 0, 1, 8, 0, 777, 777, ix.data_ptr(), lse.data_ptr(), grad.data_ptr(), 1.0,
+                        dl.data_ptr(), 0, 777, torch.cuda.current_stream().cuda_stream)  # fmt: skip
+    assert rc == 0
+    exp = torch.nn.functional.one_hot(index, 777).float() - torch.softmax(logits, -1)
+    assert (dl.cpu() - exp).abs().max().item() <= 1e-5
+    # in place: dlogits may alias logits
+    rc = lib.oi_lsg_bwd(lg.data_ptr(), 0, 1, 8, 0, 777, 777, ix.data_ptr(), lse.data_ptr(), grad.data_ptr(), 1.0,
+                        lg.data_ptr(), 0, 777, torch.cuda.current_stream().cuda_stream)  # fmt: skip
+    assert rc == 0 and torch.equal(lg, dl)
+
+
+def test_full_size_properties_bf16_rows():
+    """BASELINE config 2 row shape at a row count that keeps the test short: run-to-run bitwise
+    determinism, shift invariance and zero-sum gradient rows - none of which need the oracle."""
+    rows, vocab = 4096, 128256
+    torch.manual_seed(0)
+    logits = (torch.randn(rows, vocab, device=DEV) * 3.0).bfloat16()
+    index = torch.randint(0, vocab, (rows,), device=DEV)
+    a, ea = model_utils.logprob_and_entropy(logits, index)
+    b, eb = model_utils.logprob_and_entropy(logits, index)
+    assert torch.equal(a, b) and torch.equal(ea, eb)
+    assert (a <= 0).all() and (ea > 0).all() and (ea <= math.log(vocab) + 1e-3).all()
+    shifted = (logits.float() + 8.0).bfloat16()  # exact in bf16 only approximately; tolerance covers it
+    c, _ = model_utils.logprob_and_entropy(shifted[:64], index[:64])
+    ref = o_logprob.log_softmax_and_gather(shifted[:64].cpu(), index[:64].cpu())
+    assert (c.cpu() - ref).abs().max().item() <= 2e-3
+    lg = logits[:512].clone().requires_grad_(True)
+    model_utils.log_softmax_and_gather(lg, index[:512]).sum().backward()
+    assert lg.grad.float().sum(-1).abs().max().item() <= 0.05
