@@ -144,6 +144,57 @@ __device__ __forceinline__ int acc_row(int wm, int i, int r, int lane) {
 }
 __device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * 128 + j * 32 + (lane & 31); }
 
+// Online softmax statistics in the log2 domain of the scaled logits x = z * c:
+//   m = max x,  s = sum 2^(x - m),  t = sum 2^(x - m) * (x - m)
+// (entropy = ln2 * (log2 s - t / s), logsumexp = ln2 * (m + log2 s)).
+__device__ __forceinline__ void merge_stats(float ma, float sa, float ta, float mb, float sb, float tb, float* m,
+                                            float* s, float* t) {
+    const float mn = fmaxf(ma, mb);
+    const float da = ma - mn, db = mb - mn;
+    const float fa = __builtin_amdgcn_exp2f(da), fb = __builtin_amdgcn_exp2f(db);
+    *s = sa * fa + sb * fb;
+    *t = fa * fmaf(da, sa, ta) + fb * fmaf(db, sb, tb);
+    *m = mn;
+}
+
+// Fold the 32 logits that one lane holds for token column j of a finished tile into the running
+// statistics.  PARTIAL handles the last vocabulary tile: rows past the vocabulary are skipped by
+// predicate (weight exactly 0) instead of through a sentinel value.
+template <bool PARTIAL>
+__device__ __forceinline__ void stats_update(AccTile& acc, int j, int wm, int lane, int64_t m0, int64_t vocab, float c,
+                                             float& st_m, float& st_s, float& st_t) {
+    float vmax = OI_NEG_BIG;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            // keep the rounded product: the maximum and the exponents must see the same x
+            acc[i][j][r] *= c;
+            if (!PARTIAL || m0 + acc_row(wm, i, r, lane) < vocab) vmax = fmaxf(vmax, acc[i][j][r]);
+        }
+    const float mn = fmaxf(st_m, vmax);
+    const float shift = st_m - mn;
+    const float alpha = __builtin_amdgcn_exp2f(shift);
+    float s = st_s * alpha;
+    float t = alpha * fmaf(shift, st_s, st_t);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float d = acc[i][j][r] - mn;
+            float e = __builtin_amdgcn_exp2f(d);
+            if (PARTIAL && m0 + acc_row(wm, i, r, lane) >= vocab) {
+                d = 0.f;
+                e = 0.f;
+            }
+            s += e;
+            t = fmaf(e, d, t);
+        }
+    st_m = mn;
+    st_s = s;
+    st_t = t;
+}
+
 // ---------------------------------------------------------------------------------------------
 // forward: per-token softmax statistics over the vocabulary tiles of one split
 // ---------------------------------------------------------------------------------------------
@@ -200,29 +251,10 @@ __global__ void __launch_bounds__(NTHREADS)
                     if (n < n_tokens) zy[n] = v;
                 }
             }
-            float vmax = OI_NEG_BIG;
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    if (partial_tile && m0 + acc_row(wm, i, r, lane) >= vocab) acc[i][j][r] = -INFINITY;
-                    vmax = fmaxf(vmax, acc[i][j][r] * c);
-                }
-            const float mn = fmaxf(st_m[j], vmax);
-            const float alpha = __builtin_amdgcn_exp2f(st_m[j] - mn);
-            float s = st_s[j] * alpha, t = st_t[j] * alpha;
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float z = acc[i][j][r];
-                    const float e = __builtin_amdgcn_exp2f(fmaf(z, c, -mn));
-                    s += e;
-                    t = fmaf(e, z > -INFINITY ? z : 0.f, t);
-                }
-            st_m[j] = mn;
-            st_s[j] = s;
-            st_t[j] = t;
+            if (partial_tile)
+                stats_update<true>(acc, j, wm, lane, m0, vocab, c, st_m[j], st_s[j], st_t[j]);
+            else
+                stats_update<false>(acc, j, wm, lane, m0, vocab, c, st_m[j], st_s[j], st_t[j]);
         }
     }
 
@@ -232,9 +264,8 @@ __global__ void __launch_bounds__(NTHREADS)
     for (int j = 0; j < 4; ++j) {
         const float om = __shfl_xor(st_m[j], 32, OI_WAVE), os = __shfl_xor(st_s[j], 32, OI_WAVE),
                     ot = __shfl_xor(st_t[j], 32, OI_WAVE);
-        const float mn = fmaxf(st_m[j], om);
-        const float fa = __builtin_amdgcn_exp2f(st_m[j] - mn), fb = __builtin_amdgcn_exp2f(om - mn);
-        const float s = st_s[j] * fa + os * fb, t = st_t[j] * fa + ot * fb;
+        float mn, s, t;
+        merge_stats(st_m[j], st_s[j], st_t[j], om, os, ot, &mn, &s, &t);
         if (lane < 32) {
             float* p = red + (wm * 256 + acc_col(wn, j, lane)) * 3;
             p[0] = mn;
@@ -248,11 +279,7 @@ __global__ void __launch_bounds__(NTHREADS)
 #pragma unroll
         for (int w = 1; w < 4; ++w) {
             const float* p = red + (w * 256 + tid) * 3;
-            const float mn = fmaxf(m, p[0]);
-            const float fa = __builtin_amdgcn_exp2f(m - mn), fb = __builtin_amdgcn_exp2f(p[0] - mn);
-            s = s * fa + p[1] * fb;
-            t = t * fa + p[2] * fb;
-            m = mn;
+            merge_stats(m, s, t, p[0], p[1], p[2], &m, &s, &t);
         }
         const int64_t n = n0 + tid;
         if (n < n_tokens) partial[split * n_pad + n] = make_float4(m, s, t, 0.f);
@@ -268,16 +295,14 @@ __global__ void lmhead_fwd_combine_kernel(const float4* __restrict__ partial, co
     float m = OI_NEG_BIG, s = 0.f, t = 0.f;
     for (int64_t sp = 0; sp < n_splits; ++sp) {
         const float4 p = partial[sp * n_pad + n];
-        const float mn = fmaxf(m, p.x);
-        const float fa = __builtin_amdgcn_exp2f(m - mn), fb = __builtin_amdgcn_exp2f(p.x - mn);
-        s = s * fa + p.y * fb;
-        t = t * fa + p.z * fb;
-        m = mn;
+        merge_stats(m, s, t, p.x, p.y, p.z, &m, &s, &t);
     }
-    const float lse = (m + log2f(s)) * OI_LN2;
-    logprob[n] = zy[n] * inv_t - lse;
-    if (entropy) entropy[n] = lse - inv_t * (t / s);
-    if (lse_out) lse_out[n] = lse;
+    const double ln2 = 0.69314718055994530942;
+    const double log2s = log2((double)s);
+    const double lse = ((double)m + log2s) * ln2;
+    logprob[n] = (float)((double)zy[n] * (double)inv_t - lse);
+    if (entropy) entropy[n] = (float)((log2s - (double)t / (double)s) * ln2);
+    if (lse_out) lse_out[n] = (float)lse;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -465,7 +490,7 @@ int check_lmhead(const void* hidden, const void* weight, const int64_t* labels, 
                  int64_t vocab, float inv_t) {
     OI_RETURN_IF(n_tokens < 0 || hdim <= 0 || vocab <= 0, OI_EINVAL);
     OI_RETURN_IF(hdim % BK != 0, OI_EINVAL);
-    OI_RETURN_IF(!(inv_t > 0.f) || !(inv_t < 3.0e38f), OI_EINVAL);
+    OI_RETURN_IF(!(inv_t >= 1.0e-6f) || !(inv_t <= 1.0e6f), OI_EINVAL);
     OI_RETURN_IF(n_tokens > (int64_t)1 << 30 || vocab > (int64_t)1 << 30, OI_EINVAL);
     if (n_tokens == 0) return OI_OK;
     OI_RETURN_IF(!hidden || !weight || !labels, OI_ENULL);

@@ -68,7 +68,9 @@ struct F16Row {
 };
 
 // Online softmax statistics of the scaled logits x = z * c (c = log2(e) / T), log2 domain:
-//   m = running max of x,  s = sum 2^(x - m),  t = sum 2^(x - m) * z   (t only when ENT).
+//   m = running max of x,  s = sum 2^(x - m),  t = sum 2^(x - m) * (x - m)   (t only when ENT).
+// Keeping t relative to the running maximum makes the entropy ln2 * (log2 s - t / s) a difference
+// of two small numbers instead of lse - sum p*z, two numbers of the size of the logits.
 struct RowStat {
     float m, s, t;
 };
@@ -83,13 +85,16 @@ __device__ __forceinline__ void stat_update(RowStat& st, const float (&z)[VEC], 
         vmax = fmaxf(vmax, x[j]);
     }
     const float mn = fmaxf(st.m, vmax);
-    const float alpha = __builtin_amdgcn_exp2f(st.m - mn);
-    float s = st.s * alpha, t = st.t * alpha;
+    const float shift = st.m - mn;  // <= 0
+    const float alpha = __builtin_amdgcn_exp2f(shift);
+    float s = st.s * alpha;
+    float t = ENT ? alpha * fmaf(shift, st.s, st.t) : 0.f;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-        const float e = __builtin_amdgcn_exp2f(x[j] - mn);
+        const float d = x[j] - mn;
+        const float e = __builtin_amdgcn_exp2f(d);
         s += e;
-        if (ENT) t = fmaf(e, z[j], t);
+        if (ENT) t = fmaf(e, d, t);
     }
     st.m = mn;
     st.s = s;
@@ -98,21 +103,17 @@ __device__ __forceinline__ void stat_update(RowStat& st, const float (&z)[VEC], 
 
 template <bool ENT>
 __device__ __forceinline__ void stat_update1(RowStat& st, float z, float c) {
-    const float x = z * c;
-    const float mn = fmaxf(st.m, x);
-    const float alpha = __builtin_amdgcn_exp2f(st.m - mn);
-    const float e = __builtin_amdgcn_exp2f(x - mn);
-    st.s = st.s * alpha + e;
-    if (ENT) st.t = fmaf(e, z, st.t * alpha);
-    st.m = mn;
+    const float zz[1] = {z};
+    stat_update<1, ENT>(st, zz, c);
 }
 
 __device__ __forceinline__ RowStat stat_merge(const RowStat& a, const RowStat& b) {
     RowStat r;
     r.m = fmaxf(a.m, b.m);
-    const float fa = __builtin_amdgcn_exp2f(a.m - r.m), fb = __builtin_amdgcn_exp2f(b.m - r.m);
+    const float da = a.m - r.m, db = b.m - r.m;
+    const float fa = __builtin_amdgcn_exp2f(da), fb = __builtin_amdgcn_exp2f(db);
     r.s = a.s * fa + b.s * fb;
-    r.t = a.t * fa + b.t * fb;
+    r.t = fa * fmaf(da, a.s, a.t) + fb * fmaf(db, b.s, b.t);
     return r;
 }
 
@@ -182,13 +183,16 @@ __global__ void __launch_bounds__(256) lsg_entropy_fwd_kernel(const typename R::
             RowStat o = {sm[0][w], sm[1][w], sm[2][w]};
             tot = stat_merge(tot, o);
         }
-        const float lse = (tot.m + log2f(tot.s)) * OI_LN2;
+        // once per row: assemble in fp64 so that the result carries only the rounding of m, s and t
+        const double ln2 = 0.69314718055994530942;
+        const double log2s = log2((double)tot.s);
+        const double lse = ((double)tot.m + log2s) * ln2;
         int64_t y = index[row];
         y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
         const float zy = R::load_one(p + y);
-        logprob[row] = zy * inv_t - lse;
-        if (ENT) entropy[row] = lse - inv_t * (tot.t / tot.s);
-        if (lse_out) lse_out[row] = lse;
+        logprob[row] = (float)((double)zy * (double)inv_t - lse);
+        if (ENT) entropy[row] = (float)((log2s - (double)tot.t / (double)tot.s) * ln2);
+        if (lse_out) lse_out[row] = (float)lse;
     }
 }
 

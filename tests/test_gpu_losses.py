@@ -47,11 +47,17 @@ def test_masked_mean_random_and_gradient(axis, denominator, bool_mask):
     ref = o_red.masked_mean(ref_v, m, axis, denominator)
     upstream = torch.randn(4, generator=g)
     ref.backward(upstream)
-    dv = values.to(DEV).requires_grad_(True)
+    dv = values.clone().to(DEV).requires_grad_(True)
     out = rl_utils.masked_mean(dv, m.to(DEV), axis, denominator)
     out.backward(upstream.to(DEV))
     _close(out, ref)
-    assert (dv.grad.cpu() - ref_v.grad).abs().max().item() <= 1e-7 + 1e-5 * ref_v.grad.abs().max().item()
+    # Slices whose mask is empty: the reference's torch.where(denom > 0, num / denom, 0) has a
+    # 0 * (1/0) = NaN gradient there; the kernel defines that gradient as 0.
+    exp_grad = ref_v.grad
+    undefined = torch.isnan(exp_grad)
+    assert (dv.grad.cpu()[undefined] == 0).all()
+    exp_grad = torch.where(undefined, torch.zeros_like(exp_grad), exp_grad)
+    assert (dv.grad.cpu() - exp_grad).abs().max().item() <= 1e-7 + 1e-5 * exp_grad.abs().max().item()
 
 
 def test_masked_mean_scalar_cases():
@@ -116,9 +122,8 @@ def test_compute_grpo_loss_parity_and_gradients(loss_fn, kl_estimator, with_ref)
     up_pg, up_kl = torch.randn(new.shape, generator=g), torch.randn(new.shape, generator=g)
 
     def run(mod, dev):
-        n = new.to(dev).requires_grad_(True)
+        n = new.clone().to(dev).requires_grad_(True)
         ratio = torch.exp(n - old.to(dev))
-        ratio.retain_grad()
         pg, cf, kl = mod.compute_grpo_loss(n, ratio, adv.to(dev), ref.to(dev) if with_ref else None, cfg, rho.to(dev))
         (pg * up_pg.to(dev) + kl * up_kl.to(dev)).sum().backward()
         return pg, cf, kl, n.grad
@@ -209,14 +214,19 @@ def test_grpo_loss_fused_parity(loss_fn, axis, denominator, with_old):
     o_old = old if with_old else rn.detach()
     e_loss, e_pg, e_cf, _, e_ratio = o_grpo.grpo_token_loss(rn, o_old, ref, adv, mask, cfg, rho, denominator, axis, dp_scale=2.0)
     e_loss.backward()
-    dn = new.to(DEV).requires_grad_(True)
+    dn = new.clone().to(DEV).requires_grad_(True)
     loss, stats = grpo_utils.grpo_loss_fused(
         dn, old.to(DEV) if with_old else None, ref.to(DEV), adv.to(DEV), mask.to(DEV), cfg, rho.to(DEV), ent.to(DEV),
         loss_denominator=denominator, axis=axis, dp_scale=2.0,
     )  # fmt: skip
     loss.backward()
     _close(loss, e_loss, 2e-5)
-    assert (dn.grad.cpu() - rn.grad).abs().max().item() <= 2e-5 * max(1e-6, rn.grad.abs().max().item()) + 1e-9
+    # rows without response tokens under axis=1: NaN gradient in the reference (0 * 1/0), 0 here
+    exp_grad = rn.grad
+    undefined = torch.isnan(exp_grad)
+    assert (dn.grad.cpu()[undefined] == 0).all() and (axis == 1 or not undefined.any())
+    exp_grad = torch.where(undefined, torch.zeros_like(exp_grad), exp_grad)
+    assert (dn.grad.cpu() - exp_grad).abs().max().item() <= 2e-5 * max(1e-6, exp_grad.abs().max().item()) + 1e-9
     # statistics recorded by populate_sample_loss_stats in the reference
     d = (rn.detach() - ref).clamp(-40, 40)
     kl4 = o_red.masked_mean(o_logprob.estimate_kl(d, e_ratio.detach()), mask)
@@ -327,7 +337,7 @@ def test_dpo_loss_parity_and_gradients(label_smoothing, reference_free, golden):
     up = torch.randn(8, generator=g)
 
     def run(mod, dev):
-        a, b = pc.to(dev).requires_grad_(True), pr.to(dev).requires_grad_(True)
+        a, b = pc.clone().to(dev).requires_grad_(True), pr.clone().to(dev).requires_grad_(True)
         losses, cr, rj = mod.dpo_loss(a, b, rc.to(dev), rr.to(dev), 0.1, reference_free, label_smoothing)
         losses.backward(up.to(dev))
         return losses, cr, rj, a.grad, b.grad

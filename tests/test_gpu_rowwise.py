@@ -54,8 +54,16 @@ def test_logprob_and_entropy_forward(shape, vocab, dtype, scale, temperature):
     both_lp, both_ent = model_utils.logprob_and_entropy(lg, ix, temperature=temperature)
     assert lp.dtype == torch.float32 and lp.shape == index.shape
     tol = _tol(dtype)
-    assert (lp.cpu() - exp_lp).abs().max().item() <= tol
-    assert (ent.cpu() - exp_ent).abs().max().item() <= tol
+    # The exact result on the same inputs (fp64 arithmetic): the kernel must be within tolerance of
+    # it.  The fp32 restatement of the reference is itself up to ~1.2e-5 away from the exact value
+    # when a temperature is applied (rounding of z / T before the reduction), so against it the
+    # bound is widened by that restatement's own measured deviation.
+    exact_lp = o_logprob.log_softmax_and_gather(logits, index, torch.float64, temperature)
+    exact_ent = o_logprob.entropy_from_logits(logits, torch.float64, temperature)
+    assert (lp.cpu().double() - exact_lp).abs().max().item() <= tol
+    assert (ent.cpu().double() - exact_ent).abs().max().item() <= tol
+    assert (lp.cpu() - exp_lp).abs().max().item() <= tol + (exp_lp.double() - exact_lp).abs().max().item()
+    assert (ent.cpu() - exp_ent).abs().max().item() <= tol + (exp_ent.double() - exact_ent).abs().max().item()
     assert torch.equal(both_lp, lp) and torch.equal(both_ent, ent)  # one pass == two passes, bitwise
     assert (lp <= 0).all() and torch.isfinite(lp).all() and (ent >= -tol).all()
 
@@ -113,11 +121,12 @@ def test_closed_forms_on_device():
 def test_backward_matches_oracle_autograd(shape, vocab, dtype, temperature):
     logits, index = _case(shape, vocab, dtype, 3.0, seed=3)
     g = torch.Generator().manual_seed(4)
-    upstream = torch.randn(shape, generator=g)
+    # |upstream| <= 0.5 keeps one bf16 rounding of a gradient entry (2^-9 relative) below 1e-3
+    upstream = (torch.randn(shape, generator=g) * 0.2).clamp(-0.5, 0.5)
     upstream.view(-1)[0] = 0.0  # a masked-out token: its gradient row must be exactly zero
-    ref_in = logits.float().requires_grad_(True)
+    ref_in = logits.float().clone().requires_grad_(True)
     o_logprob.log_softmax_and_gather(ref_in, index, None, temperature).backward(upstream)
-    lg = logits.to(DEV).requires_grad_(True)
+    lg = logits.clone().to(DEV).requires_grad_(True)
     model_utils.log_softmax_and_gather(lg, index.to(DEV), temperature=temperature).backward(upstream.to(DEV))
     assert lg.grad.dtype == dtype and lg.grad.shape == logits.shape
     err = (lg.grad.float().cpu() - ref_in.grad).abs().max().item()
