@@ -13,8 +13,9 @@
 // Tile: 256 x 256 x 64 per 512-thread workgroup, 8 waves as 4 (m) x 2 (n), each wave 64 x 128 =
 // 2 x 4 MFMA 32x32x16 accumulators.  With vocabulary as the m dim a lane's 16 accumulator
 // registers of one MFMA tile belong to ONE token (column), so the softmax statistics reduce
-// inside the lane.  LDS: two buffers of (A + B) tiles with rows padded to 72 bf16 (144 B), which
-// keeps the 16-byte fragment reads of 32 consecutive rows on distinct banks.
+// inside the lane.  LDS: a ring of four 32 KB stages of (A + B) k-tiles filled by direct global->LDS
+// loads; rows are unpadded and their 16-byte chunks XOR-permuted so that fragment reads stay free of
+// bank conflicts.
 #include "oi_common.h"
 
 namespace {
@@ -22,14 +23,14 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int BM = 256, BN = 256, BK = 32;
 constexpr int NTHREADS = 512;
-constexpr int LDS_STRIDE = BK + 8;             // bf16 elements per padded tile row
-constexpr int TILE_ELEMS = BM * LDS_STRIDE;    // one operand tile
-constexpr int BUF_ELEMS = 2 * TILE_ELEMS;      // A + B
-constexpr int LDS_BYTES = 2 * BUF_ELEMS * 2;   // two buffers, 147456 B
-constexpr int STAGE_STRIDE = 256 + 8;          // bf16 per row of the dZ staging tile
-static_assert(256 * STAGE_STRIDE * 2 <= LDS_BYTES, "dZ staging tile must fit in the main-loop LDS");
+constexpr int NSTAGE = 4;                       // LDS ring: one k-tile being read, three in flight
+constexpr int TILE_ELEMS = BM * BK;             // one operand tile in LDS, rows of 64 B, unpadded
+constexpr int STAGE_ELEMS = 2 * TILE_ELEMS;     // A + B = 32 KB
+constexpr int STAGE_STRIDE = 256 + 8;           // bf16 per row of the dZ staging tile
+constexpr int LDS_ELEMS = 256 * STAGE_STRIDE;   // 135168 B: covers the ring (131072 B) and the dZ staging tile
+static_assert(NSTAGE * STAGE_ELEMS <= LDS_ELEMS, "the main-loop ring must fit");
 
 typedef f32x16 AccTile[2][4];
 
@@ -50,8 +51,33 @@ inline unsigned grid_for_tiles(int64_t tiles_m, int64_t tiles_n) {
     return (unsigned)(((nst + 7) / 8) * 8 * 32);
 }
 
+// LDS tile layout: row r of an operand tile holds its 32 k-values as four 16-byte chunks; chunk c
+// is stored at position c ^ swz(r).  With that permutation the 16-byte fragment reads of 32
+// consecutive rows at one logical chunk fall on distinct banks, and the rows stay unpadded, which
+// the direct global->LDS loads need (a wave's 64 lanes fill 1 KB of consecutive LDS).
+__device__ __forceinline__ int swz(int row) { return (row >> 2) & 3; }
+
+#define OI_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define OI_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+// Wait until at most PENDING of this wave's global->LDS loads are still in flight, then meet the
+// other waves.  A bare s_barrier (no fence) keeps the compiler from draining the loads that were
+// issued for later k-tiles.
+template <int PENDING>
+__device__ __forceinline__ void wait_loads_and_barrier() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PENDING) : "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // acc = A[m0 : m0+256, :K] * B[n0 : n0+256, :K]^T.  Rows past M / N are clamped onto the last
-// valid row (their results are discarded by the epilogues); K must be a multiple of 64.
+// valid row (their results are discarded by the epilogues); K must be a multiple of 32.
+//
+// The k loop is bound by how many bytes a CU keeps in flight towards L2/HBM, so the LDS is a ring
+// of four 32 KB stages (k-tile of 32) filled by direct global->LDS loads (no VGPR staging, no LDS
+// store instructions): while k-tile t is multiplied, the loads of t+1 .. t+3 are outstanding.
+// Wave w owns rows [32 w, 32 w + 32) of both operand tiles: 4 loads of 1 KB per k-tile.
+constexpr int LOADS_PER_STAGE = 4;
 __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restrict__ A, int64_t lda, int64_t m0,
                                           int64_t M, const uint16_t* __restrict__ B, int64_t ldb, int64_t n0,
                                           int64_t N, int64_t K, uint16_t* lds) {
@@ -66,74 +92,89 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // global -> LDS staging: 2048 16-byte chunks per operand tile, 4 per thread
-    const int lrow = tid >> 3, kc = tid & 7;
-    const uint16_t* ap[4];
-    const uint16_t* bp[4];
-    int soff[4];
+    // loader side: lane -> (row, stored chunk) inside a block of 16 rows
+    const uint16_t* ap[2];
+    const uint16_t* bp[2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int r = lrow + i * 64;
+    for (int b = 0; b < 2; ++b) {
+        const int r = wave * 32 + b * 16 + (lane >> 2);
+        const int c = (lane & 3) ^ swz(r);
         int64_t ga = m0 + r, gb = n0 + r;
         ga = ga < M ? ga : M - 1;
         gb = gb < N ? gb : N - 1;
-        ap[i] = A + ga * lda + kc * 8;
-        bp[i] = B + gb * ldb + kc * 8;
-        soff[i] = r * LDS_STRIDE + kc * 8;
+        ap[b] = A + ga * lda + c * 8;
+        bp[b] = B + gb * ldb + c * 8;
     }
-    oi_u32x4 sa[4], sb[4];
+    uint16_t* my_rows = lds + wave * 32 * BK;
+    auto issue = [&](int64_t kt) {
+        uint16_t* dst = my_rows + (int)(kt & (NSTAGE - 1)) * STAGE_ELEMS;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        sa[i] = *reinterpret_cast<const oi_u32x4*>(ap[i]);
-        sb[i] = *reinterpret_cast<const oi_u32x4*>(bp[i]);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        *reinterpret_cast<oi_u32x4*>(lds + soff[i]) = sa[i];
-        *reinterpret_cast<oi_u32x4*>(lds + TILE_ELEMS + soff[i]) = sb[i];
-    }
-    __syncthreads();
-
-    const int frag_off = (lane & 31) * LDS_STRIDE + (lane >> 5) * 8;
-    const int a_off = wm * 64 * LDS_STRIDE + frag_off;
-    const int b_off = TILE_ELEMS + wn * 128 * LDS_STRIDE + frag_off;
-
-    const int64_t ktiles = K / BK;
-    for (int64_t kt = 0; kt < ktiles; ++kt) {
-        const bool more = kt + 1 < ktiles;
-        if (more) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                sa[i] = *reinterpret_cast<const oi_u32x4*>(ap[i] + (kt + 1) * BK);
-                sb[i] = *reinterpret_cast<const oi_u32x4*>(bp[i] + (kt + 1) * BK);
-            }
+        for (int b = 0; b < 2; ++b) {
+            __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(ap[b] + kt * BK), OI_LDS_PTR(dst + b * 16 * BK), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(bp[b] + kt * BK), OI_LDS_PTR(dst + TILE_ELEMS + b * 16 * BK),
+                                             16, 0, 0);
         }
-        const uint16_t* cur = lds + (kt & 1) * BUF_ELEMS;
+    };
+    const int64_t ktiles = K / BK;
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 af[2], bf[4];
+    for (int t = 0; t < NSTAGE - 1; ++t)
+        if (t < ktiles) issue(t);
+
+    // consumer side: element offsets of this lane's fragments; k-step ks flips the stored chunk by
+    // (2 ks); rows 32 apart share the same permutation
+    const int lr = lane & 31, h = lane >> 5;
+    const int ra = wm * 64 + lr, rb = wn * 128 + lr;
+    const int pg = h ^ swz(lr);
+    int a_off[2], b_off[2];
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                af[i] = *reinterpret_cast<const bf16x8*>(cur + a_off + i * 32 * LDS_STRIDE + ks * 16);
+    for (int ks = 0; ks < 2; ++ks) {
+        a_off[ks] = ra * BK + (((2 * ks) ^ pg) * 8);
+        b_off[ks] = TILE_ELEMS + rb * BK + (((2 * ks) ^ pg) * 8);
+    }
+    auto load_frags = [&](int64_t kt, int ks, bf16x8(&af)[2], bf16x8(&bf)[4]) {
+        const uint16_t* cur = lds + (int)(kt & (NSTAGE - 1)) * STAGE_ELEMS;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) af[i] = *reinterpret_cast<const bf16x8*>(cur + a_off[ks] + i * 32 * BK);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(cur + b_off[ks] + j * 32 * BK);
+    };
+    auto mma = [&](const bf16x8(&af)[2], const bf16x8(&bf)[4]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                bf[j] = *reinterpret_cast<const bf16x8*>(cur + b_off + j * 32 * LDS_STRIDE + ks * 16);
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    };
+
+    // Software pipeline over the two k-steps of a k-tile: the barrier that publishes k-tile t+1 sits
+    // between the two MFMA batches of k-tile t, and the fragments of the next batch are always
+    // requested before the current batch is issued, so LDS latency and the barrier are covered by
+    // MFMA work instead of leaving the matrix pipe idle at the top of every k-tile.
+    bf16x8 a0[2], b0[4], a1[2], b1[4];
+    if (ktiles >= 3) wait_loads_and_barrier<2 * LOADS_PER_STAGE>();
+    else if (ktiles == 2) wait_loads_and_barrier<LOADS_PER_STAGE>();
+    else wait_loads_and_barrier<0>();
+    load_frags(0, 0, a0, b0);
+    for (int64_t kt = 0; kt < ktiles; ++kt) {
+        load_frags(kt, 1, a1, b1);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(a0, b0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kt + 1 < ktiles) {
+            // k-tile kt+1 must have landed; kt+2 may stay in flight.  After the barrier every wave has
+            // finished k-tile kt-1, whose stage is reused for k-tile kt+3.
+            if (kt + 2 < ktiles) wait_loads_and_barrier<LOADS_PER_STAGE>();
+            else wait_loads_and_barrier<0>();
+            if (kt + NSTAGE - 1 < ktiles) issue(kt + NSTAGE - 1);
+            load_frags(kt + 1, 0, a0, b0);
         }
-        if (more) {
-            uint16_t* nxt = lds + ((kt + 1) & 1) * BUF_ELEMS;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                *reinterpret_cast<oi_u32x4*>(nxt + soff[i]) = sa[i];
-                *reinterpret_cast<oi_u32x4*>(nxt + TILE_ELEMS + soff[i]) = sb[i];
-            }
-        }
-        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        mma(a1, b1);
+        __builtin_amdgcn_sched_barrier(0);
     }
+    // every wave is done reading before the caller reuses the LDS (epilogue staging, next tile)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 }
 
 // Accumulator geometry of one wave: element (i, j, r) of lane `lane` is
@@ -203,7 +244,7 @@ __global__ void __launch_bounds__(NTHREADS)
                       const int64_t* __restrict__ labels, int64_t n_tokens, int64_t hdim, int64_t vocab, float c,
                       int64_t n_splits, int64_t tiles_per_split, int64_t n_pad, float4* __restrict__ partial,
                       float* __restrict__ zy) {
-    __shared__ __align__(16) uint16_t lds[LDS_BYTES / 2];
+    __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
     const int64_t token_tiles = (n_tokens + BN - 1) / BN;
     int64_t split, tt;
     if (!tile_of_block(n_splits, token_tiles, &split, &tt)) return;
@@ -314,7 +355,7 @@ __global__ void __launch_bounds__(NTHREADS)
                      const float* __restrict__ grad, int64_t n_tokens, int64_t hdim, int64_t vocab, float c,
                      float inv_t, int64_t v_begin, int64_t chunk_cols, int64_t n_pad, uint16_t* __restrict__ dz,
                      uint16_t* __restrict__ dzt) {
-    __shared__ __align__(16) uint16_t lds[LDS_BYTES / 2];
+    __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
     const int64_t token_tiles = n_pad / BN, vocab_tiles = chunk_cols / BM;
     int64_t vt, tt;
     if (!tile_of_block(vocab_tiles, token_tiles, &vt, &tt)) return;
@@ -394,7 +435,7 @@ __global__ void __launch_bounds__(NTHREADS)
     gemm_store_kernel(const uint16_t* __restrict__ A, int64_t lda, int64_t M, const uint16_t* __restrict__ B,
                       int64_t ldb, int64_t N, int64_t K, int mode, float* out_f32, uint16_t* out_bf16, int64_t ldo,
                       int64_t m_valid) {
-    __shared__ __align__(16) uint16_t lds[LDS_BYTES / 2];
+    __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     int64_t tm, tn;
     if (!tile_of_block(tiles_m, tiles_n, &tm, &tn)) return;
@@ -489,7 +530,7 @@ BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab, int want_dw) {
 int check_lmhead(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens, int64_t hdim,
                  int64_t vocab, float inv_t) {
     OI_RETURN_IF(n_tokens < 0 || hdim <= 0 || vocab <= 0, OI_EINVAL);
-    OI_RETURN_IF(hdim % BK != 0, OI_EINVAL);
+    OI_RETURN_IF(hdim % 64 != 0, OI_EINVAL);
     OI_RETURN_IF(!(inv_t >= 1.0e-6f) || !(inv_t <= 1.0e6f), OI_EINVAL);
     OI_RETURN_IF(n_tokens > (int64_t)1 << 30 || vocab > (int64_t)1 << 30, OI_EINVAL);
     if (n_tokens == 0) return OI_OK;
@@ -588,5 +629,21 @@ extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const 
                                hidden_dim, valid);
         }
     }
+    return oi_launch_status();
+}
+
+extern "C" int oi_gemm_bf16_tn(const void* A, int64_t lda, int64_t M, const void* B, int64_t ldb, int64_t N, int64_t K,
+                               float* out_f32, void* out_bf16, int64_t ldo, int accumulate, void* stream) {
+    OI_RETURN_IF(M <= 0 || N <= 0 || K <= 0 || K % 64 != 0 || ldo < N, OI_EINVAL);
+    OI_RETURN_IF(lda < 0 || ldb < 0 || lda % 8 != 0 || ldb % 8 != 0, OI_EINVAL);
+    OI_RETURN_IF((lda != 0 && lda < K) || (ldb != 0 && ldb < K), OI_EINVAL);
+    OI_RETURN_IF(!A || !B || (!out_f32 && !out_bf16) || (out_f32 && out_bf16), OI_ENULL);
+    OI_RETURN_IF(accumulate && !out_f32, OI_EINVAL);
+    OI_RETURN_IF(!oi_aligned(A, 16) || !oi_aligned(B, 16), OI_EALIGN);
+    const int mode = out_f32 ? (accumulate ? 1 : 0) : 2;
+    hipLaunchKernelGGL(gemm_store_kernel, dim3(grid_for_tiles((M + BM - 1) / BM, (N + BN - 1) / BN)), dim3(NTHREADS),
+                       0, static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(A), lda, M,
+                       static_cast<const uint16_t*>(B), ldb, N, K, mode, out_f32, static_cast<uint16_t*>(out_bf16), ldo,
+                       M);
     return oi_launch_status();
 }
