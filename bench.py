@@ -1,6 +1,6 @@
 """Benchmark of the policy-loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c1|c5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c1|c4|c5]
 
 Prints ONE JSON line.  A "step" is one pass of the hot path (forward + backward) over one batch of
 synthetic inputs that already live in HBM.  Workloads are the BASELINE configs:
@@ -9,6 +9,7 @@ synthetic inputs that already live in HBM.  Workloads are the BASELINE configs:
       Llama-3.1-8B shape: hidden bf16 [32768, 4096], W bf16 [128256, 4096], 70 % response tokens.
   c2: GRPO loss on materialised bf16 logits [64, 1024, 128256], fwd + bwd (HBM-bound).
   c1: logprob + entropy + masked_mean on fp32 logits [4, 512, 32000], forward only.
+  c4: packed batch at OLMo-2-7B shape (16 sequences, cu_seqlens, V=100352), per-sequence sums + GRPO loss.
   c5: DPO at Llama-3.1-70B head shape: hidden [32768, 8192], W [128256, 8192], bwd to dHidden only.
 
 `roofline` describes the dominant kernel of the workload, timed with HIP events on the stream it
@@ -194,6 +195,61 @@ def make_c1(torch, oi):
     return step, info
 
 
+def make_c4(torch, oi, hdim=4096, vocab=100352, n_seqs=16, budget=32768):
+    """Packed (padding-free) batch: per-sequence summed logprobs through cu_seqlens plus the GRPO loss
+    with masked_mean(axis=1) over the packed row, forward and backward."""
+    dev = "cuda:0"
+    torch.manual_seed(0)
+    lens = torch.randint(128, 4097, (n_seqs,)).tolist()
+    kept, total = [], 0
+    for n in lens:  # greedy truncation to the token budget
+        n = min(n, budget - total)
+        if n <= 1:
+            break
+        kept.append(n)
+        total += n
+    cu = torch.tensor([0] + list(torch.tensor(kept).cumsum(0)), dtype=torch.int32, device=dev)
+    n_tokens = total
+    hidden = torch.randn(n_tokens, hdim, device=dev).bfloat16().requires_grad_(True)
+    weight = (torch.randn(vocab, hdim, device=dev) * 0.02).bfloat16().requires_grad_(True)
+    labels = torch.randint(0, vocab, (1, n_tokens), device=dev)
+    labels[0, cu[:-1].long()] = -100  # first token of every sequence is never a target
+    shifted = oi.padding_free_collator.shift_labels(labels)
+    mask = (shifted != -100).view(-1)
+    adv = torch.randn(n_tokens, device=dev)
+    cfg = _cfg()
+    with torch.no_grad():
+        lp0, _ = oi.fused_lm_head_logprobs(hidden, weight, shifted.view(-1), mask=mask)
+    old = lp0 + 0.05 * torch.randn(n_tokens, device=dev)
+    ref = lp0 + 0.1 * torch.randn(n_tokens, device=dev)
+    n_eff = int(mask.sum().item())
+    fwd_timer = EventTimer(torch)
+
+    def step():
+        hidden.grad = None
+        weight.grad = None
+        with fwd_timer:
+            lp, ent = oi.fused_lm_head_logprobs(hidden, weight, shifted.view(-1), mask=mask, return_entropy=True)
+        seq_logps = oi.padding_free_collator.get_batch_logps(lp.view(1, -1), labels, cu)
+        loss, _ = oi.grpo_utils.grpo_loss_fused(
+            lp[None], old[None], ref[None], adv[None], mask[None], cfg, entropy=ent[None], axis=1
+        )
+        (loss + 1e-6 * seq_logps.mean()).backward()
+        return loss
+
+    flops_fwd = 2.0 * n_eff * hdim * vocab
+    info = {
+        "tokens": n_tokens,
+        "rows_multiplied": n_eff,
+        "flops_step": 3.0 * flops_fwd,
+        "kernel": "lmhead_fwd_kernel (fused lm_head forward: MFMA tiles + online softmax statistics)",
+        "alg_per_launch": flops_fwd,
+        "bound": "mfma",
+        "timer": fwd_timer,
+    }
+    return step, info
+
+
 # ------------------------------------------------------------------------------------------------
 # CPU baseline: the oracle's restatement of the reference path on a bounded sample
 # ------------------------------------------------------------------------------------------------
@@ -205,11 +261,11 @@ def cpu_baseline(torch, workload):
     threads = torch.get_num_threads()
     cfg = _cfg()
     torch.manual_seed(0)
-    if workload in ("c3", "c5"):
-        hdim = 4096 if workload == "c3" else 8192
-        vocab, n = 128256, 256
+    if workload in ("c3", "c4", "c5"):
+        hdim = 8192 if workload == "c5" else 4096
+        vocab, n = (100352 if workload == "c4" else 128256), 256
         hidden = torch.randn(n, hdim).bfloat16().requires_grad_(True)
-        weight = (torch.randn(vocab, hdim) * 0.02).bfloat16().requires_grad_(workload == "c3")
+        weight = (torch.randn(vocab, hdim) * 0.02).bfloat16().requires_grad_(workload != "c5")
         labels = torch.randint(0, vocab, (n,))
         mask = torch.rand(n) < 0.7
         adv, noise = torch.randn(n), torch.randn(n)
@@ -294,7 +350,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c5"])
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-library-gemm", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -316,6 +372,10 @@ def main():
     if args.workload == "c3":
         step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02)
         name = "c3: fused lm_head+logprob+entropy+GRPO loss fwd+bwd, hidden bf16 [32768,4096], W bf16 [128256,4096], 70% response tokens (rows compacted)"
+        dtype = "bf16"
+    elif args.workload == "c4":
+        step, info = make_c4(torch, oi)
+        name = "c4: packed OLMo-2-7B shape, 16 sequences via cu_seqlens, hidden bf16 [N<=32768,4096], W bf16 [100352,4096]; per-sequence logprob sums + GRPO loss masked_mean(axis=1), fwd+bwd"
         dtype = "bf16"
     elif args.workload == "c5":
         step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True)
@@ -371,7 +431,8 @@ def main():
         roofline["whole_step_frac"] = roofline["whole_step_tflops"] / PEAK_BF16_TFLOPS
         if not args.no_library_gemm:
             hdim = 8192 if args.workload == "c5" else 4096
-            roofline["library_bf16_gemm_tflops"] = library_gemm_tflops(torch, 32768, hdim, 128256)
+            vocab = 100352 if args.workload == "c4" else 128256
+            roofline["library_bf16_gemm_tflops"] = library_gemm_tflops(torch, 32768, hdim, vocab)
     if "bytes_step" in info:
         roofline["whole_step_gbs"] = info["bytes_step"] / (ms_per_step * 1e-3) / 1e9
         roofline["whole_step_frac"] = roofline["whole_step_gbs"] / PEAK_HBM_GBS

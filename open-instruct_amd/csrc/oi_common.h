@@ -33,16 +33,15 @@ typedef float oi_f32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float oi_bf16lo_to_f32(uint32_t packed) { return __uint_as_float(packed << 16); }
 __device__ __forceinline__ float oi_bf16hi_to_f32(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
 
-// round-to-nearest-even f32 -> bf16 bits (NaN kept quiet)
-__device__ __forceinline__ uint32_t oi_f32_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
-}
+// f32 -> bf16, round to nearest even: one v_cvt_pk_bf16_f32 per pair on gfx950
+typedef __bf16 oi_bf16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t oi_pack_bf16x2(float lo, float hi) {
-    return oi_f32_to_bf16_bits(lo) | (oi_f32_to_bf16_bits(hi) << 16);
+    const oi_bf16x2 v = {(__bf16)lo, (__bf16)hi};
+    uint32_t u;
+    __builtin_memcpy(&u, &v, 4);
+    return u;
 }
+__device__ __forceinline__ uint32_t oi_f32_to_bf16_bits(float f) { return oi_pack_bf16x2(f, 0.f) & 0xffffu; }
 
 __device__ __forceinline__ float oi_f16bits_to_f32(uint16_t h) {
     _Float16 v;

@@ -492,13 +492,13 @@ FwdPlan plan_fwd(int64_t n_tokens, int64_t vocab) {
     p.token_tiles = (n_tokens + BN - 1) / BN;
     p.vocab_tiles = (vocab + BM - 1) / BM;
     p.n_pad = p.token_tiles * BN;
-    // enough workgroups for ~4 rounds over 256 CUs, but at least 8 vocabulary tiles per split
-    int64_t want = (1024 + p.token_tiles - 1) / p.token_tiles;
-    int64_t max_splits = (p.vocab_tiles + 7) / 8;
-    if (max_splits < 1) max_splits = 1;
-    int64_t s = want < max_splits ? want : max_splits;
-    if (s < 1) s = 1;
-    p.tiles_per_split = (p.vocab_tiles + s - 1) / s;
+    // Many short workgroups (8 vocabulary tiles each) rather than a few long ones: the grid is a
+    // whole number of 256-CU rounds only by luck, and the idle tail of the last round costs one
+    // workgroup's run time, so that run time is kept small.  Fewer tiles per split only when the
+    // problem is too small to give every CU work otherwise.
+    int64_t tps = 8;
+    while (tps > 1 && ((p.vocab_tiles + tps - 1) / tps) * p.token_tiles < 512) tps /= 2;
+    p.tiles_per_split = tps;
     p.n_splits = (p.vocab_tiles + p.tiles_per_split - 1) / p.tiles_per_split;
     return p;
 }

@@ -228,7 +228,7 @@ __global__ void __launch_bounds__(256) lsg_bwd_kernel(const typename R::elem_t* 
     const float ng = -g;
 
     int64_t i = tid;
-    constexpr int U = 2;
+    constexpr int U = 4;
     for (; i + (int64_t)(U - 1) * nthr < nvec; i += (int64_t)U * nthr) {
         float z[U][VEC];
 #pragma unroll
