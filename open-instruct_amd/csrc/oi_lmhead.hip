@@ -106,19 +106,21 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
         bp[b] = B + gb * ldb + c * 8;
     }
     uint16_t* my_rows = lds + wave * 32 * BK;
+    const int64_t ktiles = K / BK;
+    // k-tiles past the end re-read the last one into a stage nobody reads any more: the loop body
+    // stays free of branches, which lets the scheduler interleave loads, LDS reads and MFMAs
     auto issue = [&](int64_t kt) {
+        const int64_t src = kt < ktiles ? kt : ktiles - 1;
         uint16_t* dst = my_rows + (int)(kt & (NSTAGE - 1)) * STAGE_ELEMS;
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
-            __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(ap[b] + kt * BK), OI_LDS_PTR(dst + b * 16 * BK), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(bp[b] + kt * BK), OI_LDS_PTR(dst + TILE_ELEMS + b * 16 * BK),
+            __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(ap[b] + src * BK), OI_LDS_PTR(dst + b * 16 * BK), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(bp[b] + src * BK), OI_LDS_PTR(dst + TILE_ELEMS + b * 16 * BK),
                                              16, 0, 0);
         }
     };
-    const int64_t ktiles = K / BK;
 #pragma unroll
-    for (int t = 0; t < NSTAGE - 1; ++t)
-        if (t < ktiles) issue(t);
+    for (int t = 0; t < NSTAGE - 1; ++t) issue(t);
 
     // consumer side: element offsets of this lane's fragments; k-step ks flips the stored chunk by
     // (2 ks); rows 32 apart share the same permutation
@@ -151,27 +153,41 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
     // requested before the current batch is issued, so LDS latency and the barrier are covered by
     // MFMA work instead of leaving the matrix pipe idle at the top of every k-tile.
     bf16x8 a0[2], b0[4], a1[2], b1[4];
-    if (ktiles >= 3) wait_loads_and_barrier<2 * LOADS_PER_STAGE>();
-    else if (ktiles == 2) wait_loads_and_barrier<LOADS_PER_STAGE>();
-    else wait_loads_and_barrier<0>();
+    wait_loads_and_barrier<2 * LOADS_PER_STAGE>();
     load_frags(0, 0, a0, b0);
     for (int64_t kt = 0; kt < ktiles; ++kt) {
         load_frags(kt, 1, a1, b1);
-        __builtin_amdgcn_sched_barrier(0);
         mma(a0, b0);
-        __builtin_amdgcn_sched_barrier(0);
-        if (kt + 1 < ktiles) {
-            // k-tile kt+1 must have landed; kt+2 may stay in flight.  After the barrier every wave has
-            // finished k-tile kt-1, whose stage is reused for k-tile kt+3.
-            if (kt + 2 < ktiles) wait_loads_and_barrier<LOADS_PER_STAGE>();
-            else wait_loads_and_barrier<0>();
-            if (kt + NSTAGE - 1 < ktiles) issue(kt + NSTAGE - 1);
-            load_frags(kt + 1, 0, a0, b0);
+        // 6 LDS reads spread over the 8 MFMAs
+#pragma unroll
+        for (int q = 0; q < 6; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_barrier(0);
+        // k-tile kt+1 must have landed, kt+2 may stay in flight.  After the barrier every wave has
+        // finished k-tile kt-1, whose stage is reused for k-tile kt+3.
+        wait_loads_and_barrier<LOADS_PER_STAGE>();
+        issue(kt + NSTAGE - 1);
+        load_frags(kt + 1, 0, a0, b0);
         mma(a1, b1);
+        // 4 global->LDS loads and 6 LDS reads spread over the 8 MFMAs
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_barrier(0);
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // every wave is done reading before the caller reuses the LDS (epilogue staging, next tile)
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
