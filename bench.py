@@ -34,6 +34,16 @@ if ROOT not in sys.path:
 PEAK_HBM_GBS = 8000.0
 PEAK_BF16_TFLOPS = 2500.0
 
+# HBM-side bytes per launch of each workload's dominant kernel, from two `rocprofv3 --pmc` runs of
+# this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter
+# reads for a 1 GiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000 on MI355X).  Counters cannot
+# be read from inside the process, so the figures are carried here from the committed summaries in
+# profiles/; workloads without a counter run report null.
+MEASURED_TRAFFIC_BYTES = {
+    "c3": 36.24e9 + 0.04e9,  # lmhead_fwd_kernel: L2 misses of the tiled operand re-reads (1.24 GB unique)
+    "c2": 16.83e9 + 0.0e9,  # lsg_entropy_fwd_kernel: 1.00x the logits
+}
+
 
 def _cfg():
     return types.SimpleNamespace(loss_fn="dapo", clip_lower=0.2, clip_higher=0.28, beta=0.05, kl_estimator=2)
@@ -421,7 +431,8 @@ def main():
         "peak": peak,
         "unit": unit,
         "frac": achieved / peak,
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+        "traffic_unit": "bytes/launch",
         "kernel": info["kernel"],
         "kernel_ms": kernel_ms,
         "algorithmic_per_launch": info["alg_per_launch"],
