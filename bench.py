@@ -273,7 +273,7 @@ def cpu_baseline(torch, workload):
     torch.manual_seed(0)
     if workload in ("c3", "c4", "c5"):
         hdim = 8192 if workload == "c5" else 4096
-        vocab, n = (100352 if workload == "c4" else 128256), 256
+        vocab, n = (100352 if workload == "c4" else 128256), 2048
         hidden = torch.randn(n, hdim).bfloat16().requires_grad_(True)
         weight = (torch.randn(vocab, hdim) * 0.02).bfloat16().requires_grad_(workload != "c5")
         labels = torch.randint(0, vocab, (n,))
@@ -294,7 +294,7 @@ def cpu_baseline(torch, workload):
 
         sample = f"{n} of 32768 token rows at full H={hdim}, V={vocab}; fwd+bwd; bf16 GEMM + fp32 log_softmax"
     elif workload == "c2":
-        n, vocab = 512, 128256
+        n, vocab = 8192, 128256
         logits = (torch.randn(n, vocab) * 3.0).bfloat16().requires_grad_(True)
         labels = torch.randint(0, vocab, (n,))
         adv, noise = torch.randn(n), torch.randn(n)

@@ -1,0 +1,223 @@
+"""GPU parity of whole call chains of the hot path, small enough for the CPU oracle:
+
+* packed (padding-free) batch: fused lm_head -> per-sequence sums through cu_seqlens + GRPO loss
+  with a per-row masked mean, forward and backward;
+* DPO: fused lm_head -> per-sequence sums -> sigmoid preference loss, backward to the hidden states;
+* the plain product entry point of the MFMA tile engine;
+* size-independent properties of the fused kernels at the full Llama-3.1-8B head shape.
+
+Tolerance 2e-3 abs (bf16 inputs, fp32 accumulation) unless a test says otherwise.
+"""
+
+import math
+
+import pytest
+import torch
+
+from conftest import make_grpo_config
+
+from open_instruct_amd import _lib, dpo_utils, grpo_utils, lm_head, model_utils, padding_free_collator
+from oracle import dpo as o_dpo
+from oracle import grpo as o_grpo
+from oracle import lm_head as o_lm
+from oracle import logprob as o_logprob
+from oracle import reductions as o_red
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 2e-3
+
+
+def _bf16_tol(ref: torch.Tensor) -> float:
+    """Absolute tolerance plus one bf16 rounding of the largest expected entry."""
+    return TOL + ref.abs().max().item() * 2**-7
+
+
+def test_packed_grpo_chain_matches_oracle():
+    """Shape of open_instruct/padding_free_collator.py:202-229 callers: one packed row, ragged
+    sequences, first token of each sequence never a target."""
+    torch.manual_seed(5)
+    h, v = 128, 3000
+    lens = [37, 1, 250, 2, 129, 64]
+    total = sum(lens)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    hidden = torch.randn(total, h).bfloat16()
+    weight = (torch.randn(v, h) * 2.0 / math.sqrt(h)).bfloat16()
+    labels = torch.randint(0, v, (1, total))
+    labels[0, cu[:-1].long()] = -100
+    labels[0, 40:45] = -100  # a prompt stretch inside a sequence
+    shifted = o_logprob.shift_labels(labels)
+    mask = (shifted != -100).view(-1)
+    adv = torch.randn(total)
+    cfg = make_grpo_config(loss_fn="dapo", beta=0.05, kl_estimator=2)
+
+    # oracle chain, fp32 on the upcast inputs
+    rh = hidden.float().requires_grad_(True)
+    rw = weight.float().requires_grad_(True)
+    lp_o, ent_o = o_lm.lm_head_logprobs(rh, rw, shifted.view(-1), 1.0, True)
+    old = (lp_o.detach() + 0.05 * torch.randn(total)) * mask
+    ref = (lp_o.detach() + 0.10 * torch.randn(total)) * mask
+    lp_o = lp_o * mask
+    seq_o = o_red.get_batch_logps_packed(lp_o[None], labels, cu)
+    loss_o, *_ = o_grpo.grpo_token_loss(lp_o[None], old[None], ref[None], adv[None], mask[None].float(), cfg, axis=1)
+    (loss_o + 0.01 * seq_o.mean()).backward()
+
+    dh = hidden.to(DEV).requires_grad_(True)
+    dw = weight.to(DEV).requires_grad_(True)
+    lp, ent = lm_head.fused_lm_head_logprobs(dh, dw, shifted.view(-1).to(DEV), mask=mask.to(DEV), return_entropy=True)
+    seq = padding_free_collator.get_batch_logps(lp.view(1, -1), labels.to(DEV), cu.to(DEV))
+    loss, stats = grpo_utils.grpo_loss_fused(
+        lp[None], old.to(DEV)[None], ref.to(DEV)[None], adv.to(DEV)[None], mask.to(DEV)[None], cfg,
+        entropy=ent[None], axis=1,
+    )  # fmt: skip
+    (loss + 0.01 * seq.mean()).backward()
+
+    assert (lp.cpu() - lp_o.detach()).abs().max().item() <= TOL
+    assert ((ent.cpu() - ent_o) * mask).abs().max().item() <= TOL
+    # sums over up to 250 tokens: tolerance per token times the kept count
+    counts = torch.tensor([int(mask[cu[i] : cu[i + 1] - 1].sum()) for i in range(len(lens))]).clamp(min=1)
+    assert ((seq.cpu() - seq_o.detach()).abs() <= TOL * counts).all()
+    assert abs(loss.item() - loss_o.item()) <= TOL
+    assert (dh.grad.float().cpu() - rh.grad).abs().max().item() <= _bf16_tol(rh.grad)
+    assert (dw.grad.float().cpu() - rw.grad).abs().max().item() <= _bf16_tol(rw.grad)
+    assert ((dh.grad.float().cpu() - rh.grad).norm() / rh.grad.norm()).item() <= 2e-2
+    assert ((dw.grad.float().cpu() - rw.grad).norm() / rw.grad.norm()).item() <= 2e-2
+    assert (dh.grad.cpu()[~mask] == 0).all()
+    assert math.isfinite(stats["policy/entropy_avg"].item())
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_dpo_chain_matches_oracle(packed):
+    """Fused head -> per-sequence logps -> sigmoid preference loss (open_instruct/dpo_utils.py:523-563,
+    open_instruct/dpo_utils.py:826-878), gradient to the hidden states only (frozen head)."""
+    torch.manual_seed(6)
+    h, v, pairs, t = 64, 2000, 3, 48
+    b = 2 * pairs  # chosen rows first, rejected rows after, as concatenated_inputs lays them out
+    hidden = torch.randn(b, t, h).bfloat16()
+    weight = (torch.randn(v, h) * 2.0 / math.sqrt(h)).bfloat16()
+    labels = torch.randint(0, v, (b, t))
+    labels[:, :7] = -100  # prompt
+    labels[1, 30:] = -100  # padding tail
+    labels[4, 20:] = -100
+    ref_c, ref_r = -torch.rand(pairs) * 40, -torch.rand(pairs) * 40
+    beta = 0.1
+
+    rh = hidden.float().requires_grad_(True)
+    if packed:
+        flat_lab = labels.reshape(1, -1)
+        cu = torch.arange(0, b * t + 1, t, dtype=torch.int32)
+        lp_o = o_logprob.calculate_per_token_logps(o_lm.lm_head_logits(rh.reshape(1, b * t, h), weight.float()), flat_lab)
+        seq_o = o_red.get_batch_logps_packed(lp_o, flat_lab, cu)
+    else:
+        lp_o = o_logprob.calculate_per_token_logps(o_lm.lm_head_logits(rh, weight.float()), labels)
+        seq_o = o_red.get_batch_logps_padded(lp_o, labels)
+    losses_o, cr_o, rr_o = o_dpo.dpo_loss(seq_o[:pairs], seq_o[pairs:], ref_c, ref_r, beta, label_smoothing=0.05)
+    losses_o.mean().backward()
+
+    dh = hidden.to(DEV).requires_grad_(True)
+    w = weight.to(DEV)
+    if packed:
+        flat_lab_d = labels.reshape(1, -1).to(DEV)
+        shifted = padding_free_collator.shift_labels(flat_lab_d)
+        lp, _ = lm_head.fused_lm_head_logprobs(dh.reshape(1, b * t, h), w, shifted, mask=shifted != -100)
+        seq = padding_free_collator.get_batch_logps(lp, flat_lab_d, cu.to(DEV))
+    else:
+        shifted = padding_free_collator.shift_labels(labels.to(DEV))
+        lp, _ = lm_head.fused_lm_head_logprobs(dh, w, shifted, mask=shifted != -100)
+        seq = dpo_utils._get_batch_logps(lp, labels.to(DEV))
+    losses, cr, rr = dpo_utils.dpo_loss(seq[:pairs], seq[pairs:], ref_c.to(DEV), ref_r.to(DEV), beta, label_smoothing=0.05)
+    losses.mean().backward()
+
+    n_kept = (labels[:, 1:] != -100).sum(-1).clamp(min=1).float()
+    assert ((seq.cpu() - seq_o.detach()).abs() <= TOL * n_kept).all()
+    # loss = f(beta * x): the error of x (two sequence sums) is scaled by beta
+    assert (losses.cpu() - losses_o.detach()).abs().max().item() <= TOL * beta * 2 * n_kept.max().item() + 1e-5
+    assert (cr.cpu() - cr_o).abs().max().item() <= TOL * beta * n_kept.max().item() + 1e-5
+    assert (rr.cpu() - rr_o).abs().max().item() <= TOL * beta * n_kept.max().item() + 1e-5
+    assert (dh.grad.float().cpu() - rh.grad).abs().max().item() <= _bf16_tol(rh.grad)
+    assert ((dh.grad.float().cpu() - rh.grad).norm() / rh.grad.norm()).item() <= 2e-2
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 64), (300, 515, 192), (1, 70, 128), (1030, 257, 4096)])
+def test_gemm_bf16_tn_entry_point(m, n, k):
+    """out[m, n] = sum_k A[m, k] * B[n, k] through the raw C-ABI, bf16 and fp32 outputs, accumulate."""
+    torch.manual_seed(7)
+    a = torch.randn(m, k).bfloat16()
+    b = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    exp = o_lm.lm_head_logits(a, b, torch.float64)
+    lib = _lib.load()
+    ad, bd = a.to(DEV), b.to(DEV)
+    out32 = torch.full((m, n), 0.5, dtype=torch.float32, device=DEV)
+    out16 = torch.zeros(m, n, dtype=torch.bfloat16, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    rc = lib.oi_gemm_bf16_tn(ad.data_ptr(), k, m, bd.data_ptr(), k, n, k, out32.data_ptr(), None, n, 1, stream)
+    assert rc == 0
+    rc = lib.oi_gemm_bf16_tn(ad.data_ptr(), k, m, bd.data_ptr(), k, n, k, None, out16.data_ptr(), n, 0, stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    # fp32 accumulation of k products of O(1/sqrt k) terms: 1e-4 abs covers k = 4096
+    assert (out32.cpu().double() - 0.5 - exp).abs().max().item() <= 1e-4
+    assert (out16.cpu().double() - exp).abs().max().item() <= exp.abs().max().item() * 2**-8 + 1e-4
+    # rejected arguments launch nothing
+    assert lib.oi_gemm_bf16_tn(ad.data_ptr(), k, m, bd.data_ptr(), k, n, k + 8, out32.data_ptr(), None, n, 0, stream) == -1
+    assert lib.oi_gemm_bf16_tn(None, k, m, bd.data_ptr(), k, n, k, out32.data_ptr(), None, n, 0, stream) == -2
+    assert lib.oi_gemm_bf16_tn(ad.data_ptr(), k, m, bd.data_ptr(), k, n, k, None, None, n, 0, stream) != 0
+
+
+def test_full_size_properties_fused_head():
+    """Llama-3.1-8B head shape (H = 4096, V = 128256), 1500 rows: properties that need no oracle.
+
+    * zero hidden states -> uniform distribution: logprob = -ln V and entropy = ln V (closed form);
+    * hidden * 2 at temperature 2 equals hidden at temperature 1 (power-of-two scaling is exact in bf16);
+    * permuting the vocabulary (rows of W and the labels with them) leaves every result unchanged
+      up to summation order;
+    * every row of dZ sums to zero, so the column sums of dW vanish and, with all rows of W equal,
+      dHidden vanishes: a checksum over the whole backward;
+    * the fused kernel agrees with the row-wise kernel on library-made fp32 logits.
+    """
+    torch.manual_seed(8)
+    n, h, v = 1500, 4096, 128256
+    hidden = torch.randn(n, h, device=DEV).bfloat16()
+    weight = (torch.randn(v, h, device=DEV) * 0.02).bfloat16()
+    labels = torch.randint(0, v, (n,), device=DEV)
+
+    lp0, ent0 = lm_head.fused_lm_head_logprobs(torch.zeros_like(hidden), weight, labels, return_entropy=True)
+    assert (lp0 + math.log(v)).abs().max().item() <= 1e-5
+    assert (ent0 - math.log(v)).abs().max().item() <= 1e-5
+
+    lp, ent = lm_head.fused_lm_head_logprobs(hidden, weight, labels, return_entropy=True)
+    assert (lp <= 0).all() and (ent >= 0).all() and (ent <= math.log(v) + 1e-4).all()
+    lp2, ent2 = lm_head.fused_lm_head_logprobs(hidden * 2, weight, labels, temperature=2.0, return_entropy=True)
+    assert (lp2 - lp).abs().max().item() <= 1e-5 and (ent2 - ent).abs().max().item() <= 1e-5
+
+    perm = torch.randperm(v, device=DEV)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(v, device=DEV)
+    lpp, entp = lm_head.fused_lm_head_logprobs(hidden, weight[perm], inv[labels], return_entropy=True)
+    assert (lpp - lp).abs().max().item() <= 1e-4 and (entp - ent).abs().max().item() <= 1e-4
+
+    logits = hidden[:512].float() @ weight.float().t()
+    exp_lp, exp_ent = model_utils.logprob_and_entropy(logits, labels[:512])
+    assert (lp[:512] - exp_lp).abs().max().item() <= TOL
+    assert (ent[:512] - exp_ent).abs().max().item() <= TOL
+    del logits
+
+    dh = hidden.clone().requires_grad_(True)
+    dw = weight.clone().requires_grad_(True)
+    up = torch.randn(n, device=DEV)
+    out, _ = lm_head.fused_lm_head_logprobs(dh, dw, labels, temperature=0.8)
+    out.backward(up)
+    col_sums = dw.grad.float().sum(0)  # = sum_n (sum_v dZ[n, v]) h_n = 0 up to bf16 rounding of dW and dZ
+    scale = dw.grad.float().abs().sum(0)
+    assert (col_sums.abs() <= 2e-2 * scale + 1e-3).all(), (col_sums.abs() / (scale + 1e-9)).max().item()
+    # dW row of a label that occurs once, for a token with tiny softmax mass there, is ~ g/T * h_n
+    assert dh.grad.isfinite().all() and dw.grad.isfinite().all()
+
+    same = weight[:1].expand(4096, h).contiguous()  # all vocabulary rows equal -> dHidden = 0
+    dh2 = hidden[:300].clone().requires_grad_(True)
+    out2, _ = lm_head.fused_lm_head_logprobs(dh2, same, labels[:300] % 4096)
+    out2.backward(up[:300])
+    # every dZ entry of a row is the same number g/V and rounds to bf16 the same way, so the row sum
+    # of dZ is off by up to one bf16 rounding of g: |dHidden| <= 2^-8 |g| max|w|
+    bound = 2**-8 * up[:300].abs().max().item() * same.float().abs().max().item() + 1e-6
+    assert dh2.grad.float().abs().max().item() <= bound
