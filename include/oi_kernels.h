@@ -216,7 +216,8 @@ int oi_dpo_sigmoid_bwd(const float* policy_chosen, const float* policy_rejected,
  * open_instruct/olmo_core_train_modules.py:71-76 (DPOLMHead.forward) and
  * open_instruct/grpo_utils.py:558-572 (forward_for_logprobs); no single reference function
  * computes it.  hidden: bf16 [n_tokens, hidden_dim]; weight: bf16 [vocab, hidden_dim] (both
- * row-major, 16-byte aligned, hidden_dim a multiple of 64); labels int64 [n_tokens], negative
+ * row-major, 16-byte aligned, hidden_dim a multiple of 64; n_tokens, vocab and hidden_dim at most
+ * 2^22 per call); labels int64 [n_tokens], negative
  * labels are scored as token 0 (clamp(min=0) at open_instruct/padding_free_collator.py:15).
  *
  *   z = hidden @ weight^T (bf16 MFMA, fp32 accumulate), logprob/entropy/lse as for oi_lsg_*.
@@ -244,8 +245,8 @@ int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* la
  * The bf16 MFMA main loop of the lm_head kernels as a plain product (no reference counterpart;
  * it exists so that the tile engine can be tested and timed on its own):
  *   out[m, n] (+)= sum_k A[m, k] * B[n, k]      A: bf16 [M, K] (row stride lda), B: bf16 [N, K] (ldb)
- * K must be a multiple of 64, pointers 16-byte aligned, lda/ldb multiples of 8 (or 0 = every row
- * aliases row 0).  Exactly one of out_f32 / out_bf16 is written (row stride ldo); accumulate != 0
+ * K must be a multiple of 64, pointers 16-byte aligned, lda/ldb multiples of 8 and at most 2^22 (or
+ * 0 = every row aliases row 0).  Exactly one of out_f32 / out_bf16 is written (row stride ldo); accumulate != 0
  * adds to the existing fp32 output.
  */
 int oi_gemm_bf16_tn(const void* A, int64_t lda, int64_t M, const void* B, int64_t ldb, int64_t N, int64_t K,

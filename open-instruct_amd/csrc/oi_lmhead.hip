@@ -13,9 +13,9 @@
 // Tile: 256 x 256 x 64 per 512-thread workgroup, 8 waves as 4 (m) x 2 (n), each wave 64 x 128 =
 // 2 x 4 MFMA 32x32x16 accumulators.  With vocabulary as the m dim a lane's 16 accumulator
 // registers of one MFMA tile belong to ONE token (column), so the softmax statistics reduce
-// inside the lane.  LDS: a ring of four 32 KB stages of (A + B) k-tiles filled by direct global->LDS
-// loads; rows are unpadded and their 16-byte chunks XOR-permuted so that fragment reads stay free of
-// bank conflicts.
+// inside the lane.  LDS: two 64 KB stages of (A + B) k-tiles filled by direct global->LDS loads of
+// whole 128-byte row segments; rows are unpadded and their 16-byte chunks XOR-permuted so that
+// fragment reads stay free of bank conflicts.
 #include "oi_common.h"
 
 namespace {
@@ -23,11 +23,11 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 256, BN = 256, BK = 32;
+constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int NTHREADS = 512;
-constexpr int NSTAGE = 4;                       // LDS ring: one k-tile being read, three in flight
-constexpr int TILE_ELEMS = BM * BK;             // one operand tile in LDS, rows of 64 B, unpadded
-constexpr int STAGE_ELEMS = 2 * TILE_ELEMS;     // A + B = 32 KB
+constexpr int NSTAGE = 2;                       // LDS ring: one k-tile being read, one in flight
+constexpr int TILE_ELEMS = BM * BK;             // one operand tile in LDS, rows of 128 B, unpadded
+constexpr int STAGE_ELEMS = 2 * TILE_ELEMS;     // A + B = 64 KB
 constexpr int STAGE_STRIDE = 256 + 8;           // bf16 per row of the dZ staging tile
 constexpr int LDS_ELEMS = 256 * STAGE_STRIDE;   // 135168 B: covers the ring (131072 B) and the dZ staging tile
 static_assert(NSTAGE * STAGE_ELEMS <= LDS_ELEMS, "the main-loop ring must fit");
@@ -51,11 +51,11 @@ inline unsigned grid_for_tiles(int64_t tiles_m, int64_t tiles_n) {
     return (unsigned)(((nst + 7) / 8) * 8 * 32);
 }
 
-// LDS tile layout: row r of an operand tile holds its 32 k-values as four 16-byte chunks; chunk c
-// is stored at position c ^ swz(r).  With that permutation the 16-byte fragment reads of 32
+// LDS tile layout: row r of an operand tile holds its 64 k-values as eight 16-byte chunks; chunk c
+// is stored at position c ^ swz(r).  With that permutation the 16-byte fragment reads of 16
 // consecutive rows at one logical chunk fall on distinct banks, and the rows stay unpadded, which
 // the direct global->LDS loads need (a wave's 64 lanes fill 1 KB of consecutive LDS).
-__device__ __forceinline__ int swz(int row) { return (row >> 2) & 3; }
+__device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 
 #define OI_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define OI_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
@@ -71,13 +71,16 @@ __device__ __forceinline__ void wait_loads_and_barrier() {
 }
 
 // acc = A[m0 : m0+256, :K] * B[n0 : n0+256, :K]^T.  Rows past M / N are clamped onto the last
-// valid row (their results are discarded by the epilogues); K must be a multiple of 32.
+// valid row (their results are discarded by the epilogues); K must be a multiple of 64.
 //
-// The k loop is bound by how many bytes a CU keeps in flight towards L2/HBM, so the LDS is a ring
-// of four 32 KB stages (k-tile of 32) filled by direct global->LDS loads (no VGPR staging, no LDS
-// store instructions): while k-tile t is multiplied, the loads of t+1 .. t+3 are outstanding.
-// Wave w owns rows [32 w, 32 w + 32) of both operand tiles: 4 loads of 1 KB per k-tile.
-constexpr int LOADS_PER_STAGE = 4;
+// Operand tiles reach the LDS by direct global->LDS loads (no VGPR staging, no LDS store
+// instructions).  Eight consecutive lanes fetch the eight 16-byte chunks of one 128-byte row
+// segment: whole cache lines per row move about 1.7x faster from L2 than half lines do, and at
+// half lines the load path, not the matrix pipe, sets the pace of a 256 x 256 tile.  Two stages of
+// 64 KB: while k-tile t is multiplied the loads of t+1 are outstanding.
+// Wave w owns rows [32 w, 32 w + 32) of both operand tiles: 8 loads of 1 KB per k-tile.
+constexpr int LOADS_PER_STAGE = 8;
+constexpr int64_t MAX_LD = (int64_t)1 << 22;  // 255 rows * ld * 2 bytes must fit 32 bits
 __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restrict__ A, int64_t lda, int64_t m0,
                                           int64_t M, const uint16_t* __restrict__ B, int64_t ldb, int64_t n0,
                                           int64_t N, int64_t K, uint16_t* lds) {
@@ -92,18 +95,19 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // loader side: lane -> (row, stored chunk) inside a block of 16 rows
-    const uint16_t* ap[2];
-    const uint16_t* bp[2];
+    // loader side: lane -> (row, stored chunk) inside a block of 8 rows.  Addresses are a uniform
+    // 64-bit tile base plus a 32-bit byte offset per lane (rows of a tile span < 4 GB).
+    const char* a_tile = reinterpret_cast<const char*>(A + m0 * lda);
+    const char* b_tile = reinterpret_cast<const char*>(B + n0 * ldb);
+    const int a_last = (int)((M - 1 - m0) < 255 ? (M - 1 - m0) : 255);
+    const int b_last = (int)((N - 1 - n0) < 255 ? (N - 1 - n0) : 255);
+    uint32_t ao[4], bo[4];
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-        const int r = wave * 32 + b * 16 + (lane >> 2);
-        const int c = (lane & 3) ^ swz(r);
-        int64_t ga = m0 + r, gb = n0 + r;
-        ga = ga < M ? ga : M - 1;
-        gb = gb < N ? gb : N - 1;
-        ap[b] = A + ga * lda + c * 8;
-        bp[b] = B + gb * ldb + c * 8;
+    for (int b = 0; b < 4; ++b) {
+        const int r = wave * 32 + b * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ swz(r);
+        ao[b] = (uint32_t)(r < a_last ? r : a_last) * (uint32_t)(lda * 2) + c * 16;
+        bo[b] = (uint32_t)(r < b_last ? r : b_last) * (uint32_t)(ldb * 2) + c * 16;
     }
     uint16_t* my_rows = lds + wave * 32 * BK;
     const int64_t ktiles = K / BK;
@@ -111,34 +115,32 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
     // stays free of branches, which lets the scheduler interleave loads, LDS reads and MFMAs
     auto issue = [&](int64_t kt) {
         const int64_t src = kt < ktiles ? kt : ktiles - 1;
+        const char* a_src = a_tile + src * (BK * 2);
+        const char* b_src = b_tile + src * (BK * 2);
         uint16_t* dst = my_rows + (int)(kt & (NSTAGE - 1)) * STAGE_ELEMS;
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(ap[b] + src * BK), OI_LDS_PTR(dst + b * 16 * BK), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(bp[b] + src * BK), OI_LDS_PTR(dst + TILE_ELEMS + b * 16 * BK),
-                                             16, 0, 0);
+        for (int b = 0; b < 4; ++b) {
+            __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(a_src + ao[b]), OI_LDS_PTR(dst + b * 8 * BK), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(b_src + bo[b]), OI_LDS_PTR(dst + TILE_ELEMS + b * 8 * BK), 16,
+                                             0, 0);
         }
     };
-#pragma unroll
-    for (int t = 0; t < NSTAGE - 1; ++t) issue(t);
+    issue(0);
+    issue(1);
 
     // consumer side: element offsets of this lane's fragments; k-step ks flips the stored chunk by
     // (2 ks); rows 32 apart share the same permutation
     const int lr = lane & 31, h = lane >> 5;
     const int ra = wm * 64 + lr, rb = wn * 128 + lr;
     const int pg = h ^ swz(lr);
-    int a_off[2], b_off[2];
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-        a_off[ks] = ra * BK + (((2 * ks) ^ pg) * 8);
-        b_off[ks] = TILE_ELEMS + rb * BK + (((2 * ks) ^ pg) * 8);
-    }
+    const int a_base = ra * BK + pg * 8, b_base = TILE_ELEMS + rb * BK + pg * 8;
     auto load_frags = [&](int64_t kt, int ks, bf16x8(&af)[2], bf16x8(&bf)[4]) {
         const uint16_t* cur = lds + (int)(kt & (NSTAGE - 1)) * STAGE_ELEMS;
+        const int a_off = a_base ^ (ks * 16), b_off = b_base ^ (ks * 16);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) af[i] = *reinterpret_cast<const bf16x8*>(cur + a_off[ks] + i * 32 * BK);
+        for (int i = 0; i < 2; ++i) af[i] = *reinterpret_cast<const bf16x8*>(cur + a_off + i * 32 * BK);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(cur + b_off[ks] + j * 32 * BK);
+        for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(cur + b_off + j * 32 * BK);
     };
     auto mma = [&](const bf16x8(&af)[2], const bf16x8(&bf)[4]) {
 #pragma unroll
@@ -147,18 +149,8 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
             for (int j = 0; j < 4; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
     };
-
-    // Software pipeline over the two k-steps of a k-tile: the barrier that publishes k-tile t+1 sits
-    // between the two MFMA batches of k-tile t, and the fragments of the next batch are always
-    // requested before the current batch is issued, so LDS latency and the barrier are covered by
-    // MFMA work instead of leaving the matrix pipe idle at the top of every k-tile.
-    bf16x8 a0[2], b0[4], a1[2], b1[4];
-    wait_loads_and_barrier<2 * LOADS_PER_STAGE>();
-    load_frags(0, 0, a0, b0);
-    for (int64_t kt = 0; kt < ktiles; ++kt) {
-        load_frags(kt, 1, a1, b1);
-        mma(a0, b0);
-        // 6 LDS reads spread over the 8 MFMAs
+    // 6 LDS reads spread over the 8 MFMAs of one k-step
+    auto interleave_reads = [&]() {
 #pragma unroll
         for (int q = 0; q < 6; ++q) {
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
@@ -166,15 +158,36 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_barrier(0);
-        // k-tile kt+1 must have landed, kt+2 may stay in flight.  After the barrier every wave has
-        // finished k-tile kt-1, whose stage is reused for k-tile kt+3.
-        wait_loads_and_barrier<LOADS_PER_STAGE>();
-        issue(kt + NSTAGE - 1);
+    };
+
+    // Software pipeline over the four k-steps of a k-tile: the fragments of the next k-step are
+    // always requested before the MFMAs of the current one are issued, and the barrier that
+    // publishes k-tile t+1 (and frees the stage of k-tile t for t+2) sits before the last MFMA batch
+    // of k-tile t, so LDS latency and the barrier are covered by MFMA work.
+    bf16x8 a0[2], b0[4], a1[2], b1[4];
+    wait_loads_and_barrier<LOADS_PER_STAGE>();
+    load_frags(0, 0, a0, b0);
+    for (int64_t kt = 0; kt < ktiles; ++kt) {
+        load_frags(kt, 1, a1, b1);
+        mma(a0, b0);
+        interleave_reads();
+        load_frags(kt, 2, a0, b0);
+        mma(a1, b1);
+        interleave_reads();
+        load_frags(kt, 3, a1, b1);
+        mma(a0, b0);
+        interleave_reads();
+        // k-tile kt+1 must have landed and this wave's last reads of k-tile kt must be complete:
+        // after the barrier the stage of k-tile kt is overwritten with k-tile kt+2
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        issue(kt + NSTAGE);
         load_frags(kt + 1, 0, a0, b0);
         mma(a1, b1);
-        // 4 global->LDS loads and 6 LDS reads spread over the 8 MFMAs
+        // 8 global->LDS loads and 6 LDS reads spread over the 8 MFMAs
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < 6; ++q) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
@@ -182,9 +195,8 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_barrier(0);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -548,7 +560,9 @@ int check_lmhead(const void* hidden, const void* weight, const int64_t* labels, 
     OI_RETURN_IF(n_tokens < 0 || hdim <= 0 || vocab <= 0, OI_EINVAL);
     OI_RETURN_IF(hdim % 64 != 0, OI_EINVAL);
     OI_RETURN_IF(!(inv_t >= 1.0e-6f) || !(inv_t <= 1.0e6f), OI_EINVAL);
-    OI_RETURN_IF(n_tokens > (int64_t)1 << 30 || vocab > (int64_t)1 << 30, OI_EINVAL);
+    // row strides of every operand (hidden_dim, padded vocabulary, padded token count) are folded
+    // into 32-bit byte offsets inside a 256-row tile
+    OI_RETURN_IF(n_tokens > MAX_LD || vocab > MAX_LD || hdim > MAX_LD, OI_EINVAL);
     if (n_tokens == 0) return OI_OK;
     OI_RETURN_IF(!hidden || !weight || !labels, OI_ENULL);
     OI_RETURN_IF(!oi_aligned(hidden, 16) || !oi_aligned(weight, 16), OI_EALIGN);
@@ -653,6 +667,7 @@ extern "C" int oi_gemm_bf16_tn(const void* A, int64_t lda, int64_t M, const void
     OI_RETURN_IF(M <= 0 || N <= 0 || K <= 0 || K % 64 != 0 || ldo < N, OI_EINVAL);
     OI_RETURN_IF(lda < 0 || ldb < 0 || lda % 8 != 0 || ldb % 8 != 0, OI_EINVAL);
     OI_RETURN_IF((lda != 0 && lda < K) || (ldb != 0 && ldb < K), OI_EINVAL);
+    OI_RETURN_IF(lda > MAX_LD || ldb > MAX_LD, OI_EINVAL);
     OI_RETURN_IF(!A || !B || (!out_f32 && !out_bf16) || (out_f32 && out_bf16), OI_ENULL);
     OI_RETURN_IF(accumulate && !out_f32, OI_EINVAL);
     OI_RETURN_IF(!oi_aligned(A, 16) || !oi_aligned(B, 16), OI_EALIGN);
