@@ -193,6 +193,18 @@ int oi_seq_logp_bwd(const float* grad_out, const int64_t* labels, const int32_t*
                     int64_t n_seqs, int64_t total, int average, float* d_per_token_logps, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Debug statistics of locally recomputed logprobs against the sampler's logprobs.  Carries
+ * open_instruct/grpo_utils.py:345-369 (compute_vllm_local_debug_metrics) in one launch.
+ * A position is valid where mask != 0 and other_logprobs is not NaN.  out_stats (fp32[4]):
+ *   [0] mean |local - other|, [1] max |local - other|, [2] unbiased std of |local - other|
+ *   (0 when fewer than 2 valid positions), [3] mean exp(other) * (other - local); all 0 when no
+ *   position is valid.  Sums are accumulated in fp64.
+ * ------------------------------------------------------------------------------------------ */
+#define OI_LOGPROB_DIFF_NUM_STATS 4
+int oi_logprob_diff_stats(const float* local_logprobs, const float* other_logprobs, const uint8_t* mask, int64_t n,
+                          float* out_stats, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Sigmoid preference loss per pair.  Carries open_instruct/dpo_utils.py:523-563 (dpo_loss) and,
  * with ref pointers NULL and `margin` = gamma/beta, open_instruct/dpo_utils.py:617-642
  * (simpo_loss):   x = (pc - pr) - (rc - rr) - margin

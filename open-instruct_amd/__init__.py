@@ -19,6 +19,6 @@ from . import (  # noqa: F401
     rl_utils,
 )
 from .grpo_utils import INVALID_LOGPROB  # noqa: F401
-from .lm_head import fused_lm_head_logprobs  # noqa: F401
+from .lm_head import fused_linear_cross_entropy, fused_lm_head_logprobs  # noqa: F401
 
 __version__ = "0.1.0"

@@ -45,6 +45,7 @@ SIGNATURES: dict[str, tuple] = {
     "oi_masked_mean_bwd": (_I, [_P, _P, _I, _P, _I64, _I64, _I64, _P, _P]),
     "oi_seq_logp_fwd": (_I, [_P, _P, _P, _I64, _I64, _I, _P, _P, _P]),
     "oi_seq_logp_bwd": (_I, [_P, _P, _P, _P, _I64, _I64, _I, _P, _P]),
+    "oi_logprob_diff_stats": (_I, [_P, _P, _P, _I64, _P, _P]),
     "oi_dpo_sigmoid_fwd": (_I, [_P, _P, _P, _P, _P, _I64, _F, _F, _F, _P, _P, _P, _P]),
     "oi_dpo_sigmoid_bwd": (_I, [_P, _P, _P, _P, _P, _P, _I64, _F, _F, _F, _P, _P, _P]),
     "oi_lmhead_fwd_workspace_bytes": (_SZ, [_I64, _I64, _I64]),

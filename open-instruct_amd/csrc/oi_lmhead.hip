@@ -285,7 +285,7 @@ __global__ void __launch_bounds__(NTHREADS)
     const int64_t n0 = tt * BN;
 
     float st_m[4], st_s[4], st_t[4];
-    int64_t lab[4];
+    int lab[4];  // vocabulary ids fit 32 bits (vocab <= 2^22)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         st_m[j] = OI_NEG_BIG;
@@ -293,7 +293,7 @@ __global__ void __launch_bounds__(NTHREADS)
         st_t[j] = 0.f;
         const int64_t n = n0 + acc_col(wn, j, lane);
         int64_t y = n < n_tokens ? labels[n] : 0;
-        lab[j] = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
+        lab[j] = (int)(y < 0 ? 0 : (y >= vocab ? vocab - 1 : y));
     }
 
     for (int64_t vt = vt_begin; vt < vt_end; ++vt) {
@@ -301,13 +301,13 @@ __global__ void __launch_bounds__(NTHREADS)
         const int64_t m0 = vt * BM;
         gemm_tile(acc, W, hdim, m0, vocab, hidden, hdim, n0, n_tokens, hdim, lds);
         const bool partial_tile = m0 + BM > vocab;
-        const int64_t wave_row0 = m0 + wm * 64;
+        const int wave_row0 = (int)m0 + wm * 64;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             // the target logit, when its row falls into this wave's 64 rows
-            const int64_t rel = lab[j] - wave_row0;
+            const int rel = lab[j] - wave_row0;
             if (rel >= 0 && rel < 64) {
-                const int ri = (int)rel >> 5, rr = (int)rel & 31;
+                const int ri = rel >> 5, rr = rel & 31;
                 if (((rr >> 2) & 1) == (lane >> 5)) {
                     const int reg = (rr >> 3) * 4 + (rr & 3);
                     float v = 0.f;

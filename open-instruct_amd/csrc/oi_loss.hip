@@ -533,6 +533,63 @@ int check_cfg(int loss_fn, int kl_estimator) {
     return OI_OK;
 }
 
+// ---- debug statistics of two logprob tensors over a mask (one workgroup, fp64 accumulation) ----
+__global__ void __launch_bounds__(1024)
+    logprob_diff_stats_kernel(const float* __restrict__ local, const float* __restrict__ other,
+                              const uint8_t* __restrict__ mask, int64_t n, float* __restrict__ out) {
+    __shared__ double red[5][16];
+    double cnt = 0.0, sd = 0.0, sd2 = 0.0, skl = 0.0;
+    float mx = 0.f;
+    bool bad = false;
+    for (int64_t i = threadIdx.x; i < n; i += 1024) {
+        const float o = other[i];
+        if (!mask[i] || o != o) continue;
+        const float l = local[i];
+        const float d = fabsf(l - o);
+        cnt += 1.0;
+        sd += (double)d;
+        sd2 += (double)d * (double)d;
+        skl += (double)(__expf(o) * (o - l));
+        bad |= d != d;
+        mx = fmaxf(mx, d);
+    }
+    if (bad) mx = __builtin_nanf("");
+    cnt = oi_wave_sum(cnt);
+    sd = oi_wave_sum(sd);
+    sd2 = oi_wave_sum(sd2);
+    skl = oi_wave_sum(skl);
+    float wmx = oi_wave_max(mx);
+    const unsigned long long any_bad = __ballot(bad);
+    if (any_bad) wmx = __builtin_nanf("");
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) {
+        red[0][wave] = cnt;
+        red[1][wave] = sd;
+        red[2][wave] = sd2;
+        red[3][wave] = skl;
+        red[4][wave] = (double)wmx;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double c = 0, a = 0, b = 0, k = 0, m = 0;
+        bool nan_max = false;
+        for (int w = 0; w < 16; ++w) {
+            c += red[0][w];
+            a += red[1][w];
+            b += red[2][w];
+            k += red[3][w];
+            nan_max |= red[4][w] != red[4][w];
+            m = red[4][w] > m ? red[4][w] : m;
+        }
+        double var = c > 1.0 ? (b - a * a / c) / (c - 1.0) : 0.0;
+        var = var > 0.0 ? var : (var != var ? var : 0.0);
+        out[0] = c > 0.0 ? (float)(a / c) : 0.f;
+        out[1] = c > 0.0 ? (nan_max ? __builtin_nanf("") : (float)m) : 0.f;
+        out[2] = c > 1.0 ? (float)sqrt(var) : 0.f;
+        out[3] = c > 0.0 ? (float)(k / c) : 0.f;
+    }
+}
+
 }  // namespace
 
 extern "C" int oi_grpo_terms_fwd(const float* new_logprobs, const float* ratio, const float* advantages,
@@ -761,7 +818,17 @@ extern "C" int oi_rho_correction(const float* old_logprobs, const float* vllm_lo
     return oi_launch_status();
 }
 
-extern "C" int oi_version(void) { return 1000; }
+extern "C" int oi_logprob_diff_stats(const float* local_logprobs, const float* other_logprobs, const uint8_t* mask,
+                                     int64_t n, float* out_stats, void* stream) {
+    OI_RETURN_IF(n < 0, OI_EINVAL);
+    OI_RETURN_IF(!out_stats, OI_ENULL);
+    OI_RETURN_IF(n > 0 && (!local_logprobs || !other_logprobs || !mask), OI_ENULL);
+    hipLaunchKernelGGL(logprob_diff_stats_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream),
+                       local_logprobs, other_logprobs, mask, n, out_stats);
+    return oi_launch_status();
+}
+
+extern "C" int oi_version(void) { return 1001; }
 
 extern "C" const char* oi_error_string(int code) {
     switch (code) {

@@ -2,14 +2,18 @@
 
 Names and signatures follow open_instruct/dpo_utils.py in the reference (``dpo_loss`` :523-563,
 ``wpo_loss`` :566-613, ``simpo_loss`` :617-642, ``compute_loss`` :645-686, ``_get_batch_logps``
-:689-712, ``concatenated_inputs`` :734-763, ``concatenated_forward`` :826-878).
+:689-712, ``concatenated_inputs`` :734-763, ``concatenated_forward`` :826-878,
+``build_reference_logprobs_cache`` :405-520 without its multi-process steps).
 """
 
 from __future__ import annotations
 
+import pathlib
+from collections.abc import Callable, Iterable
+
 import torch
 
-from . import _lib, padding_free_collator
+from . import _lib, model_utils, padding_free_collator
 from .padding_free_collator import get_batch_logps_padded
 
 
@@ -208,3 +212,51 @@ def concatenated_forward(model, batch: dict, average_log_prob: bool = False, pac
     else:
         logps = _get_batch_logps(per_token, labels, average_log_prob)
     return logps[:bs], logps[bs:], None
+
+
+def build_reference_logprobs_cache(
+    model: torch.nn.Module,
+    dataloader: Iterable[dict],
+    average_log_prob: bool,
+    forward_fn: Callable,
+    full_dataset_size: int,
+    device: torch.device,
+    cache_path: pathlib.Path | str | None = None,
+    forward_kwargs: dict | None = None,
+) -> model_utils.TensorCache:
+    """Reference-policy logps of every sample, computed once; open_instruct/dpo_utils.py:405-520.
+
+    One no-grad pass over ``dataloader``: ``forward_fn(model, batch, average_log_prob=...)`` returns
+    ``(chosen_logps, rejected_logps, aux)``, which are scattered to ``batch["index"]``.  Batches
+    flagged ``is_padding`` are skipped; an index that no batch covered raises, as in the reference.
+    An existing ``cache_path`` is loaded instead of recomputed, a new cache is written there.
+    This is the one-process form: the reference's barriers and MAX all-reduce across ranks
+    (open_instruct/dpo_utils.py:456,494-495,518) belong to the caller's launcher.
+    """
+    cache_path = pathlib.Path(cache_path) if cache_path is not None else None
+    if cache_path is not None and cache_path.exists():
+        return model_utils.TensorCache.from_disk(cache_path, device=device)
+    was_training = model.training
+    model.eval()
+    chosen = torch.full((full_dataset_size,), float("-inf"), dtype=torch.float32, device=device)
+    rejected = torch.full((full_dataset_size,), float("-inf"), dtype=torch.float32, device=device)
+    with torch.no_grad():
+        for batch in dataloader:
+            chosen_logps, rejected_logps, _ = forward_fn(
+                model, batch, average_log_prob=average_log_prob, **(forward_kwargs or {})
+            )
+            if batch.get("is_padding", False):
+                continue
+            index = batch["index"].to(device).long()
+            chosen[index] = chosen_logps.float()
+            rejected[index] = rejected_logps.float()
+    missing = torch.where((chosen == float("-inf")) | (rejected == float("-inf")))[0]
+    if len(missing) > 0:
+        raise RuntimeError(
+            f"Missing {len(missing)} indices during reference logprobs caching. First 10: {missing[:10].tolist()}"
+        )
+    model.train(was_training)
+    cache = model_utils.TensorCache(tensors={"chosen_logps": chosen, "rejected_logps": rejected})
+    if cache_path is not None:
+        cache.to_disk(cache_path)
+    return cache

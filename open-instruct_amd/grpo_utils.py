@@ -344,6 +344,42 @@ def group_advantages(scores: torch.Tensor, group_size: int, normalization: str =
 
 
 # ----------------------------------------------------------------------------------------------
+# sampler-vs-trainer logprob debug metrics
+# ----------------------------------------------------------------------------------------------
+VLLM_LOCAL_DEBUG_KEYS = (
+    "debug/vllm_vs_local_logprob_diff_mean",
+    "debug/vllm_vs_local_logprob_diff_max",
+    "debug/vllm_vs_local_logprob_diff_std",
+    "debug/vllm_local_reverse_kl",
+)
+
+
+def vllm_local_debug_stats(
+    local_logprobs: torch.Tensor, vllm_logprobs: torch.Tensor, response_mask: torch.Tensor
+) -> torch.Tensor:
+    """The four statistics of :func:`compute_vllm_local_debug_metrics` as one device vector
+    (order of ``VLLM_LOCAL_DEBUG_KEYS``), one launch, no host synchronisation."""
+    _lib.require_gpu(local_logprobs, vllm_logprobs, response_mask)
+    if local_logprobs.shape != vllm_logprobs.shape or local_logprobs.shape != response_mask.shape:
+        raise ValueError("local_logprobs, vllm_logprobs and response_mask must have one shape")
+    lo, vl, m = _lib.f32c(local_logprobs.detach()), _lib.f32c(vllm_logprobs.detach()), _lib.mask_u8(response_mask)
+    out = torch.empty(len(VLLM_LOCAL_DEBUG_KEYS), dtype=torch.float32, device=lo.device)
+    _lib.call("oi_logprob_diff_stats", lo.data_ptr(), vl.data_ptr(), m.data_ptr(), lo.numel(), out.data_ptr(),
+              _lib.stream_of(lo))  # fmt: skip
+    return out
+
+
+def compute_vllm_local_debug_metrics(
+    local_logprobs: torch.Tensor, vllm_logprobs: torch.Tensor, response_mask: torch.Tensor
+) -> dict[str, float]:
+    """Mean / max / std of ``|local - vllm|`` and the mean reverse KL over valid response tokens;
+    drop-in for open_instruct/grpo_utils.py:345-369 (returns Python floats, i.e. synchronises,
+    exactly as the reference does)."""
+    values = vllm_local_debug_stats(local_logprobs, vllm_logprobs, response_mask).tolist()
+    return dict(zip(VLLM_LOCAL_DEBUG_KEYS, values))
+
+
+# ----------------------------------------------------------------------------------------------
 # model forward -> logprobs
 # ----------------------------------------------------------------------------------------------
 def forward_for_logprobs(

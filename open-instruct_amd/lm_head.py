@@ -3,6 +3,11 @@
 There is no single counterpart in the reference: this replaces the pair "lm_head GEMM, then
 ``calculate_per_token_logps`` / ``log_softmax_and_gather`` (+ ``entropy_from_logits``)" at
 open_instruct/olmo_core_train_modules.py:71-76 and open_instruct/grpo_utils.py:558-572.
+
+``fused_linear_cross_entropy`` is the supervised fine-tuning loss through the same kernels: the
+causal-LM cross-entropy that the reference obtains from the model's own forward
+(open_instruct/finetune.py:818-824) or from a fused linear + cross-entropy implementation
+(open_instruct/finetune.py:571-586, ``loss_implementation`` at open_instruct/olmo_core_utils.py:64-66).
 """
 
 from __future__ import annotations
@@ -103,3 +108,38 @@ def fused_lm_head_logprobs(
         ent = torch.zeros(hid2.shape[0], dtype=torch.float32, device=hidden.device).index_copy(0, idx, ent_c)
         ent = ent.reshape(lead)
     return lp.reshape(lead), ent
+
+
+def fused_linear_cross_entropy(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor | None = None,
+    *,
+    shift_labels: torch.Tensor | None = None,
+    num_items_in_batch: torch.Tensor | int | float | None = None,
+    ignore_index: int = -100,
+) -> torch.Tensor:
+    """Causal-LM cross-entropy of ``hidden @ weight.T`` against next-token labels, scalar fp32.
+
+    ``labels`` ``[B, T]`` are shifted here (position ``t`` is scored against ``labels[:, t + 1]``,
+    the last position is ignored); pass ``shift_labels`` instead when the caller has already
+    shifted them (sequence-parallel batches, open_instruct/finetune.py:826-829).  Positions whose
+    label equals ``ignore_index`` are never multiplied.  The result is the mean over kept tokens,
+    or ``sum / num_items_in_batch`` when that count is given (gradient accumulation over several
+    micro-batches).  Differentiable with respect to ``hidden`` and ``weight``.
+    """
+    if (labels is None) == (shift_labels is None):
+        raise ValueError("pass exactly one of labels / shift_labels")
+    if shift_labels is None:
+        shift_labels = torch.full_like(labels, ignore_index)
+        shift_labels[..., :-1] = labels[..., 1:]
+    if shift_labels.shape != hidden.shape[:-1]:
+        raise ValueError(f"labels {tuple(shift_labels.shape)} do not match hidden {tuple(hidden.shape)}")
+    keep = shift_labels != ignore_index
+    logps, _ = fused_lm_head_logprobs(hidden, weight, shift_labels, mask=keep)
+    total = -logps.sum()
+    if num_items_in_batch is None:
+        return total / keep.sum().clamp(min=1)
+    if torch.is_tensor(num_items_in_batch):
+        num_items_in_batch = num_items_in_batch.to(total.device)
+    return total / num_items_in_batch

@@ -11,9 +11,38 @@ to the logits' dtype) - pass ``out_dtype=logits.dtype`` to get the reference's d
 
 from __future__ import annotations
 
+import pathlib
+import tempfile
+from dataclasses import dataclass
+
 import torch
 
 from . import _lib
+
+
+@dataclass
+class TensorCache:
+    """Tensors indexed by dataset index (the reference-logprob cache of DPO); same fields and
+    methods as open_instruct/model_utils.py:92-115."""
+
+    tensors: dict[str, torch.Tensor]
+
+    def __getitem__(self, indices: torch.Tensor) -> dict[str, torch.Tensor]:
+        return {k: v[indices.long()] for k, v in self.tensors.items()}
+
+    def to_disk(self, path: str | pathlib.Path) -> None:
+        """Write atomically: temporary file in the target directory, then rename."""
+        path = pathlib.Path(path)
+        path.parent.mkdir(parents=True, exist_ok=True)
+        cpu_tensors = {k: v.cpu() for k, v in self.tensors.items()}
+        with tempfile.NamedTemporaryFile(dir=path.parent, delete=False, suffix=".tmp") as tmp:
+            tmp_path = pathlib.Path(tmp.name)
+            torch.save(cpu_tensors, tmp_path)
+        tmp_path.rename(path)
+
+    @classmethod
+    def from_disk(cls, path: str | pathlib.Path, device: torch.device) -> "TensorCache":
+        return cls(tensors=torch.load(path, weights_only=True, map_location=device))
 
 
 def _row_layout(logits: torch.Tensor) -> tuple[torch.Tensor, int, int, int, int]:

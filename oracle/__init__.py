@@ -26,6 +26,8 @@ grpo.grpo_token_loss           open_instruct/grpo_fast.py:702-724               
 dpo.dpo_loss                   open_instruct/dpo_utils.py:523-563                     closed forms (x=0 -> ln 2, L(x,ls)=L(-x,1-ls)), math.log1p brute force; reference tests (test_dpo_utils.py:30-88)
 dpo.simpo_loss / dpo.wpo_loss  open_instruct/dpo_utils.py:566-642                     closed forms only (no reference known-answer vector)
 lm_head.lm_head_logprobs       HF nn.Linear lm_head + padding_free_collator.py:10-16  textbook F.linear in fp32/fp64 (the GEMM itself lives in third-party code; no reference vector)
+lm_head.linear_cross_entropy   open_instruct/finetune.py:818-824 (HF ForCausalLMLoss)    transformers.loss.loss_utils.ForCausalLMLoss itself (the third-party routine the reference calls), brute force
+grpo.compute_vllm_local_debug_metrics  open_instruct/grpo_utils.py:345-369             pure-Python math / statistics.stdev brute force; empty and single-token masks
 =============================  =====================================================  ==========
 
 Every gradient is taken by ``torch.autograd`` on these restatements (fp64 ``gradcheck`` in

@@ -177,3 +177,21 @@ def forward_for_logprobs(
         with torch.no_grad():
             ent = logprob.entropy_from_logits(z, compute_dtype=compute_dtype, temperature=temperature)
     return lp, ent
+
+
+def compute_vllm_local_debug_metrics(
+    local_logprobs: torch.Tensor, vllm_logprobs: torch.Tensor, response_mask: torch.Tensor
+) -> dict[str, float]:
+    """Restates open_instruct/grpo_utils.py:345-369: statistics of ``|local - vllm|`` and of
+    ``exp(vllm) * (vllm - local)`` over positions that are in the mask and not NaN on the vLLM side."""
+    valid = response_mask.bool() & ~torch.isnan(vllm_logprobs)
+    count = int(valid.sum())
+    zero = torch.tensor(0.0)
+    diff = (local_logprobs - vllm_logprobs).abs().masked_fill(~valid, 0.0)
+    rkl = (torch.exp(vllm_logprobs) * (vllm_logprobs - local_logprobs)).masked_fill(~valid, 0.0)
+    return {
+        "debug/vllm_vs_local_logprob_diff_mean": float(diff.sum() / count if count > 0 else zero),
+        "debug/vllm_vs_local_logprob_diff_max": float(diff.max() if count > 0 else zero),
+        "debug/vllm_vs_local_logprob_diff_std": float(diff[valid].std() if count > 1 else zero),
+        "debug/vllm_local_reverse_kl": float(rkl.sum() / count if count > 0 else zero),
+    }

@@ -46,3 +46,23 @@ def lm_head_logprobs(
     lp = torch.cat(lps) if lps else hidden.new_zeros(0, dtype=compute_dtype)
     ent = (torch.cat(ents) if ents else hidden.new_zeros(0, dtype=compute_dtype)) if return_entropy else None
     return lp, ent
+
+
+def linear_cross_entropy(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    num_items_in_batch=None,
+    ignore_index: int = -100,
+    compute_dtype=torch.float32,
+):
+    """Causal-LM cross-entropy as the HuggingFace model forward computes it for the reference's SFT
+    loop (open_instruct/finetune.py:818-824; third-party ``transformers.loss.loss_utils.ForCausalLMLoss``):
+    labels padded with ``ignore_index`` and shifted left by one, ``F.cross_entropy`` over the
+    flattened positions with reduction "mean", or "sum" divided by ``num_items_in_batch``."""
+    logits = lm_head_logits(hidden, weight, compute_dtype)
+    shifted = F.pad(labels, (0, 1), value=ignore_index)[..., 1:].reshape(-1)
+    flat = logits.reshape(-1, logits.shape[-1])
+    if num_items_in_batch is None:
+        return F.cross_entropy(flat, shifted, ignore_index=ignore_index, reduction="mean")
+    return F.cross_entropy(flat, shifted, ignore_index=ignore_index, reduction="sum") / num_items_in_batch

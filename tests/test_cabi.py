@@ -31,7 +31,7 @@ def _declared():
 def test_library_is_built_and_loads():
     assert os.path.exists(_lib.LIB_PATH), "build with: python -m open_instruct_amd.build"
     lib = _lib.load()
-    assert lib.oi_version() == 1000
+    assert lib.oi_version() >= 1000
 
 
 def test_every_declared_symbol_is_exported_and_bound():

@@ -139,3 +139,41 @@ def test_fused_equals_materialised_path_on_device():
     lp, ent = lm_head.fused_lm_head_logprobs(hidden, weight, labels, return_entropy=True)
     assert (lp - exp_lp).abs().max().item() <= TOL
     assert (ent - exp_ent).abs().max().item() <= TOL
+
+
+@pytest.mark.parametrize("num_items", [None, 37])
+def test_fused_linear_cross_entropy_matches_oracle(num_items):
+    """Supervised fine-tuning loss through the fused head (open_instruct/finetune.py:818-824):
+    value and both gradients against F.cross_entropy on the fp32 product."""
+    from oracle import lm_head as o_head
+
+    torch.manual_seed(9)
+    b, t, h, v = 3, 40, 128, 3000
+    hidden = torch.randn(b, t, h).bfloat16()
+    weight = (torch.randn(v, h) * 2.0 / math.sqrt(h)).bfloat16()
+    labels = torch.randint(0, v, (b, t))
+    labels[:, :6] = -100
+    labels[2, 25:] = -100
+    rh = hidden.float().requires_grad_(True)
+    rw = weight.float().requires_grad_(True)
+    exp = o_head.linear_cross_entropy(rh, rw, labels, num_items_in_batch=num_items)
+    exp.backward()
+    dh = hidden.to(DEV).requires_grad_(True)
+    dw = weight.to(DEV).requires_grad_(True)
+    got = lm_head.fused_linear_cross_entropy(dh, dw, labels.to(DEV), num_items_in_batch=num_items)
+    got.backward()
+    assert got.dtype == torch.float32 and got.ndim == 0
+    assert abs(got.item() - exp.item()) <= TOL
+    assert (dh.grad.float().cpu() - rh.grad).abs().max().item() <= TOL + rh.grad.abs().max().item() * 2**-7
+    assert (dw.grad.float().cpu() - rw.grad).abs().max().item() <= TOL + rw.grad.abs().max().item() * 2**-7
+    assert ((dw.grad.float().cpu() - rw.grad).norm() / rw.grad.norm()).item() <= 2e-2
+    # already shifted labels give the same loss
+    shifted = torch.full_like(labels, -100)
+    shifted[:, :-1] = labels[:, 1:]
+    again = lm_head.fused_linear_cross_entropy(dh, dw, shift_labels=shifted.to(DEV), num_items_in_batch=num_items)
+    assert torch.equal(again, got)
+    with pytest.raises(ValueError):
+        lm_head.fused_linear_cross_entropy(dh, dw)
+    # nothing to score: zero loss, no NaN
+    empty = lm_head.fused_linear_cross_entropy(dh, dw, torch.full_like(labels, -100).to(DEV))
+    assert empty.item() == 0.0

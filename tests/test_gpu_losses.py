@@ -426,3 +426,66 @@ def test_forward_for_logprobs_and_compute_logprobs_with_mock_model():
     assert (out[0][:, 0] == grpo_utils.INVALID_LOGPROB).all()
     counts = grpo_utils.calculate_token_counts(1, data, torch.device(DEV))
     assert counts == {0: float(mask[:, 1:].sum()), 1: 0.0}
+
+
+@pytest.mark.parametrize("shape", [(3, 9), (1, 1), (4, 5000)])
+def test_vllm_local_debug_metrics_parity(shape):
+    """open_instruct/grpo_utils.py:345-369 in one launch; fp64 accumulation on the device, so the
+    comparison is against the oracle run in fp64 (1e-5) and in fp32 (loose: fp32 summation order)."""
+    g = torch.Generator().manual_seed(23)
+    local = -torch.rand(shape, generator=g) * 5
+    vllm = local + 0.1 * torch.randn(shape, generator=g)
+    mask = torch.rand(shape, generator=g) > 0.3
+    if shape[1] > 4:
+        vllm[0, 2] = float("nan")
+        mask[0, 2] = True
+    got = grpo_utils.compute_vllm_local_debug_metrics(local.to(DEV), vllm.to(DEV), mask.to(DEV))
+    exp = o_grpo.compute_vllm_local_debug_metrics(local.double(), vllm.double(), mask)
+    assert set(got) == set(exp)
+    for k in exp:
+        assert abs(got[k] - exp[k]) <= 1e-5 * max(1.0, abs(exp[k])), (k, got[k], exp[k])
+    none = grpo_utils.compute_vllm_local_debug_metrics(local.to(DEV), vllm.to(DEV), torch.zeros_like(mask).to(DEV))
+    assert all(x == 0.0 for x in none.values())
+    vec = grpo_utils.vllm_local_debug_stats(local.to(DEV), vllm.to(DEV), mask.to(DEV))
+    assert vec.shape == (4,) and vec.is_cuda
+    with pytest.raises(ValueError):
+        grpo_utils.vllm_local_debug_stats(local.to(DEV), vllm.to(DEV)[..., :-1], mask.to(DEV))
+
+
+def test_reference_cache_build_through_concatenated_forward():
+    """open_instruct/dpo_utils.py:405-520 over open_instruct/dpo_utils.py:826-878 with a stub model:
+    the cache holds, per dataset index, what a direct oracle evaluation of that sample gives."""
+    g = torch.Generator().manual_seed(24)
+    v, t, n_samples = 50, 12, 4
+    table = torch.randn(64, v, generator=g)  # logits depend on the token id only
+
+    class Model(torch.nn.Module):
+        def forward(self, input_ids, attention_mask=None, **kw):
+            return table.to(input_ids.device)[input_ids]
+
+    def sample(i):
+        ids_c = torch.randint(0, 64, (1, t), generator=g)
+        ids_r = torch.randint(0, 64, (1, t), generator=g)
+        lab_c, lab_r = ids_c.clone() % v, ids_r.clone() % v
+        lab_c[:, :3] = -100
+        lab_r[:, :5] = -100
+        return {
+            "chosen_input_ids": ids_c, "chosen_labels": lab_c, "chosen_attention_mask": torch.ones_like(ids_c),
+            "rejected_input_ids": ids_r, "rejected_labels": lab_r, "rejected_attention_mask": torch.ones_like(ids_r),
+            "index": torch.tensor([i]),
+        }  # fmt: skip
+
+    samples = [sample(i) for i in (2, 0, 3, 1)]
+    batches = [{k: val.to(DEV) for k, val in s.items()} for s in samples]
+    cache = dpo_utils.build_reference_logprobs_cache(
+        Model(), batches, False, dpo_utils.concatenated_forward, n_samples, torch.device(DEV)
+    )
+    for s in samples:
+        i = int(s["index"])
+        for side in ("chosen", "rejected"):
+            per_token = o_logprob.calculate_per_token_logps(table[s[f"{side}_input_ids"]], s[f"{side}_labels"])
+            exp = o_red.get_batch_logps_padded(per_token, s[f"{side}_labels"])
+            got = cache.tensors[f"{side}_logps"][i].item()
+            assert abs(got - exp.item()) <= 1e-4, (side, i, got, exp.item())
+    picked = cache[torch.tensor([1, 3], device=DEV)]
+    assert picked["chosen_logps"].shape == (2,)

@@ -115,3 +115,44 @@ def test_metrics_from_loss_stats():
     assert out["val/ratio"] == pytest.approx(2.5)
     assert out["loss/total_avg"] == pytest.approx(3.5)
     assert out["val/ratio_var"] == pytest.approx(0.25 * 1.5**2 + 0.75 * 0.5**2)
+
+
+def test_tensor_cache_roundtrip_and_reference_cache_builder(tmp_path):
+    """open_instruct/model_utils.py:92-115 and open_instruct/dpo_utils.py:405-520 (one-process form):
+    scatter by index, padding batches skipped, missing indices raise, disk round trip."""
+    cache = model_utils.TensorCache(tensors={"chosen_logps": torch.arange(5.0), "rejected_logps": -torch.arange(5.0)})
+    picked = cache[torch.tensor([3, 1])]
+    assert picked["chosen_logps"].tolist() == [3.0, 1.0] and picked["rejected_logps"].tolist() == [-3.0, -1.0]
+    path = tmp_path / "sub" / "cache.pt"
+    cache.to_disk(path)
+    again = model_utils.TensorCache.from_disk(path, device=torch.device("cpu"))
+    assert torch.equal(again.tensors["chosen_logps"], cache.tensors["chosen_logps"])
+
+    calls = []
+
+    def forward_fn(model, batch, average_log_prob=False, scale=1.0):
+        calls.append((model.training, average_log_prob, torch.is_grad_enabled()))
+        idx = batch["index"].float()
+        return idx * scale, -idx * scale, None
+
+    model = torch.nn.Linear(2, 2)
+    batches = [
+        {"index": torch.tensor([2, 0])},
+        {"index": torch.tensor([1, 3])},
+        {"index": torch.tensor([0, 0]), "is_padding": True},
+    ]
+    built = dpo_utils.build_reference_logprobs_cache(
+        model, batches, True, forward_fn, 4, torch.device("cpu"), tmp_path / "ref.pt", forward_kwargs={"scale": 2.0}
+    )
+    assert built.tensors["chosen_logps"].tolist() == [0.0, 2.0, 4.0, 6.0]
+    assert built.tensors["rejected_logps"].tolist() == [0.0, -2.0, -4.0, -6.0]
+    assert calls == [(False, True, False)] * 3 and model.training
+    assert (tmp_path / "ref.pt").exists()
+    # an existing file is loaded, not recomputed
+    n_calls = len(calls)
+    loaded = dpo_utils.build_reference_logprobs_cache(
+        model, batches, True, forward_fn, 4, torch.device("cpu"), tmp_path / "ref.pt"
+    )
+    assert len(calls) == n_calls and torch.equal(loaded.tensors["chosen_logps"], built.tensors["chosen_logps"])
+    with pytest.raises(RuntimeError, match="Missing 1 indices"):
+        dpo_utils.build_reference_logprobs_cache(model, batches[:2], False, forward_fn, 5, torch.device("cpu"))

@@ -457,3 +457,70 @@ def test_oracle_gradients_gradcheck():
     pr = torch.randn(4, generator=g, dtype=torch.float64, requires_grad=True)
     rc, rr = torch.randn(4, generator=g, dtype=torch.float64), torch.randn(4, generator=g, dtype=torch.float64)
     assert torch.autograd.gradcheck(lambda a, b: dpo.dpo_loss(a, b, rc, rr, 0.5, False, 0.1)[0], (pc, pr))
+
+
+def test_linear_cross_entropy_against_hf_loss_and_brute_force():
+    """The SFT loss is computed inside third-party code in the reference (HF model forward,
+    open_instruct/finetune.py:818-824).  transformers ships in this image, so the oracle is pinned
+    against ``ForCausalLMLoss`` itself, and against an explicit per-token loop."""
+    import math
+
+    g = torch.Generator().manual_seed(21)
+    b, t, h, v = 2, 7, 8, 11
+    hidden = torch.randn(b, t, h, generator=g)
+    weight = torch.randn(v, h, generator=g)
+    labels = torch.randint(0, v, (b, t), generator=g)
+    labels[0, :3] = -100
+    labels[1, -1] = -100
+    got_mean = lm_head.linear_cross_entropy(hidden, weight, labels)
+    got_sum = lm_head.linear_cross_entropy(hidden, weight, labels, num_items_in_batch=5)
+    # brute force: position i predicts labels[i + 1]
+    total, count = 0.0, 0
+    for bi in range(b):
+        for i in range(t - 1):
+            y = int(labels[bi, i + 1])
+            if y == -100:
+                continue
+            z = [sum(float(hidden[bi, i, k]) * float(weight[j, k]) for k in range(h)) for j in range(v)]
+            mx = max(z)
+            lse = mx + math.log(sum(math.exp(x - mx) for x in z))
+            total += lse - z[y]
+            count += 1
+    assert abs(got_mean.item() - total / count) < 1e-5
+    assert abs(got_sum.item() - total / 5) < 1e-5
+    hf = pytest.importorskip("transformers.loss.loss_utils")
+    logits = lm_head.lm_head_logits(hidden, weight)
+    assert abs(hf.ForCausalLMLoss(logits, labels, v).item() - got_mean.item()) < 1e-6
+    assert abs(hf.ForCausalLMLoss(logits, labels, v, num_items_in_batch=5).item() - got_sum.item()) < 1e-6
+
+
+def test_vllm_local_debug_metrics_against_python_statistics():
+    """open_instruct/grpo_utils.py:345-369 restated; checked with the statistics module."""
+    import math
+    import statistics
+
+    g = torch.Generator().manual_seed(22)
+    local = -torch.rand(3, 9, generator=g) * 5
+    vllm = local + 0.1 * torch.randn(3, 9, generator=g)
+    vllm[0, 2] = float("nan")
+    mask = torch.rand(3, 9, generator=g) > 0.3
+    mask[0, 2] = True
+    got = grpo.compute_vllm_local_debug_metrics(local, vllm, mask)
+    diffs, rkls = [], []
+    for i in range(3):
+        for j in range(9):
+            if mask[i, j] and not math.isnan(float(vllm[i, j])):
+                lo, vl = float(local[i, j]), float(vllm[i, j])
+                diffs.append(abs(lo - vl))
+                rkls.append(math.exp(vl) * (vl - lo))
+    assert abs(got["debug/vllm_vs_local_logprob_diff_mean"] - statistics.fmean(diffs)) < 1e-6
+    assert abs(got["debug/vllm_vs_local_logprob_diff_max"] - max(diffs)) < 1e-6
+    assert abs(got["debug/vllm_vs_local_logprob_diff_std"] - statistics.stdev(diffs)) < 1e-6
+    assert abs(got["debug/vllm_local_reverse_kl"] - statistics.fmean(rkls)) < 1e-6
+    empty = grpo.compute_vllm_local_debug_metrics(local, vllm, torch.zeros_like(mask))
+    assert all(x == 0.0 for x in empty.values())
+    one = torch.zeros_like(mask)
+    one[1, 1] = True
+    single = grpo.compute_vllm_local_debug_metrics(local, vllm, one)
+    assert single["debug/vllm_vs_local_logprob_diff_std"] == 0.0
+    assert abs(single["debug/vllm_vs_local_logprob_diff_mean"] - abs(float(local[1, 1] - vllm[1, 1]))) < 1e-7
