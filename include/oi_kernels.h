@@ -222,6 +222,31 @@ int oi_dpo_sigmoid_bwd(const float* policy_chosen, const float* policy_rejected,
                        float* d_policy_rejected, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Packing of query/response pairs into training rows.  Carries the per-token part of
+ * open_instruct/rl_utils.py:227-375 (pack_sequences: concatenation with padding tokens dropped
+ * from the responses, document-id response mask, intra-pack attention ids, per-document position
+ * ids (open_instruct/rl_utils.py:215-224), `dones`, sampler logprobs with NaN on query tokens)
+ * and the advantage broadcast of open_instruct/data_loader.py:1509-1514 in one launch.
+ *
+ * Inputs are the ragged lists in CSR form: q_tokens / r_tokens (int64, all queries / responses
+ * back to back), q_offsets / r_offsets (int64 [n_seqs + 1]), r_tool_mask (one byte per response
+ * token, may be NULL unless mask_tool_use), r_logprobs (fp32 per response token).  The greedy
+ * assignment of sequences to rows is O(n_seqs) scalar work and stays with the caller, who passes
+ *   dst_offsets[i] = position of sequence i's first token in the flat outputs (rows back to back),
+ *   mask_base[i]   = index of the first sequence in sequence i's row (attention id = i + 1 - base).
+ * Outputs (flat, one entry per kept token): query_responses, attention_masks, position_ids,
+ * response_masks (0 on query tokens, i + 1 on response tokens, or only where r_tool_mask != 0 when
+ * mask_tool_use), dones (i + 1 on the last token of sequence i, else 0), vllm_logprobs and, when
+ * `advantages` (fp32 [n_seqs]) is given, out_advantages = advantages[i] where response_masks != 0.
+ * ------------------------------------------------------------------------------------------ */
+int oi_pack_sequences(const int64_t* q_tokens, const int64_t* q_offsets, const int64_t* r_tokens,
+                      const int64_t* r_offsets, const uint8_t* r_tool_mask, const float* r_logprobs,
+                      const float* advantages, const int64_t* dst_offsets, const int32_t* mask_base, int64_t n_seqs,
+                      int64_t pad_token_id, int mask_tool_use, int64_t* query_responses, int64_t* attention_masks,
+                      int64_t* position_ids, int64_t* response_masks, int64_t* dones, float* vllm_logprobs,
+                      float* out_advantages, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Fused lm_head projection + per-token logprob / entropy, logits never materialised.
  *
  * Replaces the pair "lm_head GEMM -> calculate_per_token_logps" of

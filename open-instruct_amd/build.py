@@ -13,7 +13,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
-SOURCES = ["oi_rowwise.hip", "oi_loss.hip", "oi_lmhead.hip"]
+SOURCES = ["oi_rowwise.hip", "oi_loss.hip", "oi_pack.hip", "oi_lmhead.hip"]
 OUTPUT = os.path.join(CSRC, "liboi_kernels.so")
 
 HIPCC_FLAGS = [

@@ -28,13 +28,15 @@ dpo.simpo_loss / dpo.wpo_loss  open_instruct/dpo_utils.py:566-642               
 lm_head.lm_head_logprobs       HF nn.Linear lm_head + padding_free_collator.py:10-16  textbook F.linear in fp32/fp64 (the GEMM itself lives in third-party code; no reference vector)
 lm_head.linear_cross_entropy   open_instruct/finetune.py:818-824 (HF ForCausalLMLoss)    transformers.loss.loss_utils.ForCausalLMLoss itself (the third-party routine the reference calls), brute force
 grpo.compute_vllm_local_debug_metrics  open_instruct/grpo_utils.py:345-369             pure-Python math / statistics.stdev brute force; empty and single-token masks
+packing.pack_sequences         open_instruct/rl_utils.py:215-375                      reference known-answer vectors (test_rl_utils.py:125-158), reference test properties (test_rl_utils.py:98-123,299-334)
+packing.broadcast_advantages   open_instruct/data_loader.py:1509-1514                 hand-written example
 =============================  =====================================================  ==========
 
 Every gradient is taken by ``torch.autograd`` on these restatements (fp64 ``gradcheck`` in
 ``tests/``); the reference defines no backward code of its own.
 """
 
-from oracle import dpo, grpo, lm_head, logprob, reductions  # noqa: F401
+from oracle import dpo, grpo, lm_head, logprob, packing, reductions  # noqa: F401
 
 INVALID_LOGPROB = 1.0  # open_instruct/utils.py:83
 IGNORE_LABEL = -100  # open_instruct/dpo_utils.py:62

@@ -524,3 +524,42 @@ def test_vllm_local_debug_metrics_against_python_statistics():
     single = grpo.compute_vllm_local_debug_metrics(local, vllm, one)
     assert single["debug/vllm_vs_local_logprob_diff_std"] == 0.0
     assert abs(single["debug/vllm_vs_local_logprob_diff_mean"] - abs(float(local[1, 1] - vllm[1, 1]))) < 1e-7
+
+
+def test_pack_sequences_reference_vectors_and_properties(golden):
+    """open_instruct/test_rl_utils.py:98-158,299-334: known masks of the tool-use test, packed rows
+    hold query + response back to back, min_num_batches splits further without losing tokens."""
+    from oracle import packing
+
+    case = golden["pack_sequences_mask_tool_use"]
+    args = (case["queries"], case["responses"], case["masks"], case["pack_length"], case["pad_token_id"], case["vllm_logprobs"])
+    for flag, key in ((True, "with_masking"), (False, "without_masking")):
+        out = packing.pack_sequences(*args, mask_tool_use=flag)
+        assert out["query_responses"] == case["expected_query_responses"]
+        assert [[m != 0 for m in row] for row in out["response_masks"]] == case[key]
+    # three pairs; the first two fit one row, the third starts a new one (test_rl_utils.py:98-115)
+    queries = [[5, 6, 7, 8], [9, 10, 11], [12, 13]]
+    responses = [[20, 21, 22], [23], [24, 25, 26, 27]]
+    masks = [[1] * len(r) for r in responses]
+    lps = [[-0.5] * len(r) for r in responses]
+    out = packing.pack_sequences(queries, responses, masks, 12, 0, lps)
+    assert out["query_responses"] == [[5, 6, 7, 8, 20, 21, 22, 9, 10, 11, 23], [12, 13, 24, 25, 26, 27]]
+    assert out["attention_masks"] == [[1] * 7 + [2] * 4, [1] * 6]
+    assert out["position_ids"] == [[0, 1, 2, 3, 4, 5, 6, 0, 1, 2, 3], [0, 1, 2, 3, 4, 5]]
+    assert out["response_masks"] == [[0, 0, 0, 0, 1, 1, 1, 0, 0, 0, 2], [0, 0, 3, 3, 3, 3]]
+    assert out["dones"] == [[0, 0, 0, 0, 0, 0, 1, 0, 0, 0, 2], [0, 0, 0, 0, 0, 3]]
+    assert out["num_actions"] == [[3, 1], [4]] and out["packed_seq_lens"] == [[7, 4], [6]]
+    assert all(math.isnan(x) for x in out["vllm_logprobs"][0][:4]) and out["vllm_logprobs"][0][4:7] == [-0.5] * 3
+    split = packing.pack_sequences(queries, responses, masks, 12, 0, lps, min_num_batches=3)
+    assert len(split["query_responses"]) == 3 and all(len(r) > 0 for r in split["query_responses"])
+    assert sum(len(r) for r in split["query_responses"]) == sum(len(r) for r in out["query_responses"])
+    # padding tokens inside a response are dropped together with their mask and logprob entries
+    padded = packing.pack_sequences([[1]], [[7, 0, 8, 0]], [[1, 1, 0, 1]], 16, 0, [[-1.0, -2.0, -3.0, -4.0]], mask_tool_use=True)
+    assert padded["query_responses"] == [[1, 7, 8]] and padded["response_masks"] == [[0, 1, 0]]
+    assert padded["vllm_logprobs"][0][1:] == [-1.0, -3.0] and padded["num_actions"] == [[2]]
+    # a sequence longer than the row length still gets a row of its own
+    long = packing.pack_sequences([[1, 2]], [[3, 4, 5, 6]], [[1] * 4], 3, 0, [[0.0] * 4])
+    assert long["query_responses"] == [[1, 2, 3, 4, 5, 6]]
+    assert packing.broadcast_advantages([0.5, -1.5, 2.0], out["response_masks"]) == [
+        [0, 0, 0, 0, 0.5, 0.5, 0.5, 0, 0, 0, -1.5], [0, 0, 2.0, 2.0, 2.0, 2.0],
+    ]  # fmt: skip
