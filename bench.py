@@ -260,6 +260,51 @@ def make_c4(torch, oi, hdim=4096, vocab=100352, n_seqs=16, budget=32768):
     return step, info
 
 
+def _pack_case(n=512, max_q=512, max_r=3584, pad=0, seed=0):
+    import random
+
+    rng = random.Random(seed)
+    queries = [[rng.randrange(1, 50000) for _ in range(rng.randrange(1, max_q + 1))] for _ in range(n)]
+    responses = [[rng.randrange(1, 50000) for _ in range(rng.randrange(1, max_r + 1))] for _ in range(n)]
+    masks = [[1] * len(r) for r in responses]
+    lps = [[-rng.random()] * len(r) for r in responses]
+    adv = [rng.gauss(0, 1) for _ in range(n)]
+    return queries, responses, masks, lps, adv
+
+
+def make_pack(torch, oi):
+    """Packing of 512 query/response pairs (about a million tokens) into rows of 35840 tokens plus the
+    advantage broadcast: the step is the whole call (list flattening on the host, upload, one kernel)."""
+    queries, responses, masks, lps, adv = _pack_case()
+    n_tokens = sum(len(q) + len(r) for q, r in zip(queries, responses))
+    timer = EventTimer(torch)
+    plain_call = oi._lib.call
+
+    def timed_call(name, *args):
+        if name != "oi_pack_sequences":
+            return plain_call(name, *args)
+        with timer:
+            return plain_call(name, *args)
+
+    oi._lib.call = timed_call
+
+    def step():
+        packed = oi.rl_utils.pack_sequences(queries, responses, masks, 35840, 0, lps, advantages=adv, device="cuda:0")
+        return packed.advantages[0].sum()
+
+    # per token: read id 8 B + logprob 4 B (+ 1 B tool mask, not read here), write 5 x 8 B + 2 x 4 B
+    info = {
+        "tokens": n_tokens,
+        "rows_multiplied": n_tokens,
+        "bytes_step": 60.0 * n_tokens,
+        "kernel": "pack_scatter_kernel (one workgroup per sequence, seven per-token outputs)",
+        "alg_per_launch": 60.0 * n_tokens,
+        "bound": "hbm",
+        "timer": timer,
+    }
+    return step, info
+
+
 # ------------------------------------------------------------------------------------------------
 # CPU baseline: the oracle's restatement of the reference path on a bounded sample
 # ------------------------------------------------------------------------------------------------
@@ -308,6 +353,18 @@ def cpu_baseline(torch, workload):
             loss.backward()
 
         sample = f"{n} of 65536 rows of bf16 logits at V={vocab}; fwd+bwd"
+    elif workload == "pack":
+        from oracle import packing as o_pack
+
+        queries, responses, masks, lps, adv = _pack_case()
+        n = sum(len(q) + len(r) for q, r in zip(queries, responses))
+        threads = 1
+
+        def run():
+            out = o_pack.pack_sequences(queries, responses, masks, 35840, 0, lps)
+            o_pack.broadcast_advantages(adv, out["response_masks"])
+
+        sample = "the full workload (512 pairs), list-based restatement of the reference loop, one thread"
     else:
         n = 2048
         logits = torch.randn(4, 512, 32000) * 2.0
@@ -360,7 +417,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "pack"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-library-gemm", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -395,6 +452,10 @@ def main():
         step, info = make_c2(torch, oi)
         name = "c2: GRPO loss on materialised bf16 logits [64,1024,128256], fwd+bwd"
         dtype = "bf16"
+    elif args.workload == "pack":
+        step, info = make_pack(torch, oi)
+        name = "pack: 512 query/response pairs (~1M tokens) into rows of 35840 tokens + advantage broadcast, whole call from Python lists"
+        dtype = "int64"
     else:
         step, info = make_c1(torch, oi)
         name = "c1: logprob+entropy+masked_mean on fp32 logits [4,512,32000], forward"

@@ -4,6 +4,7 @@ open_instruct/rl_utils.py (``masked_mean`` :426-448, ``pack_sequences`` :227-375
 
 from __future__ import annotations
 
+import itertools
 from dataclasses import dataclass
 
 import numpy as np
@@ -124,7 +125,7 @@ def _csr(seqs: list, dtype) -> tuple[np.ndarray, np.ndarray]:
     lens = np.fromiter((len(x) for x in seqs), dtype=np.int64, count=len(seqs))
     offsets = np.zeros(len(seqs) + 1, dtype=np.int64)
     np.cumsum(lens, out=offsets[1:])
-    flat = np.fromiter((t for x in seqs for t in x), dtype=dtype, count=int(offsets[-1]))
+    flat = np.fromiter(itertools.chain.from_iterable(seqs), dtype=dtype, count=int(offsets[-1]))
     return flat, offsets
 
 
@@ -165,7 +166,7 @@ def pack_sequences(
         raise RuntimeError("pack_sequences writes its outputs on an AMD GPU; there is no CPU implementation")
     q_flat, q_off = _csr(queries, np.int64)
     r_flat, r_off = _csr(responses, np.int64)
-    m_flat, _ = _csr(masks, np.int64)
+    m_flat = _csr(masks, np.int64)[0] if mask_tool_use else None  # only read when tool tokens are masked out
     lp_flat, _ = _csr(vllm_logprobs, np.float32)
     kept = r_flat != pad_token_id
     kept_before = np.zeros(len(r_flat) + 1, dtype=np.int64)
@@ -205,11 +206,11 @@ def pack_sequences(
         adv_dev = up(adv_np)
     lens_dev = up(np.stack([r_len, seq_len])) if n else torch.zeros(2, 0, dtype=torch.int64, device=dev)
     if n:
-        ins = [up(q_flat), up(q_off), up(r_flat), up(r_off), up(m_flat != 0).view(torch.uint8), up(lp_flat),
-               up(dst[:-1]), up(mask_base)]  # fmt: skip
+        tool = up(m_flat != 0).view(torch.uint8) if mask_tool_use else None
+        ins = [up(q_flat), up(q_off), up(r_flat), up(r_off), tool, up(lp_flat), up(dst[:-1]), up(mask_base)]
         _lib.call(
             "oi_pack_sequences", ins[0].data_ptr(), ins[1].data_ptr(), ins[2].data_ptr(), ins[3].data_ptr(),
-            ins[4].data_ptr(), ins[5].data_ptr(), _lib.ptr(adv_dev), ins[6].data_ptr(), ins[7].data_ptr(), n,
+            _lib.ptr(ins[4]), ins[5].data_ptr(), _lib.ptr(adv_dev), ins[6].data_ptr(), ins[7].data_ptr(), n,
             int(pad_token_id), int(bool(mask_tool_use)), out_i64[0].data_ptr(), out_i64[1].data_ptr(),
             out_i64[2].data_ptr(), out_i64[3].data_ptr(), out_i64[4].data_ptr(), out_f32[0].data_ptr(),
             out_f32[1].data_ptr() if adv_dev is not None else None, torch.cuda.current_stream(dev).cuda_stream,
