@@ -115,7 +115,13 @@ def test_closed_forms_on_device():
 
 @pytest.mark.parametrize(
     "shape,vocab,dtype",
-    [((3, 17), 32000, torch.float32), ((2, 9), 128256, torch.bfloat16), ((5,), 4099, torch.bfloat16), ((2, 3), 10, torch.float32)],
+    [
+        ((3, 17), 32000, torch.float32),
+        ((2, 9), 128256, torch.bfloat16),  # long rows: the 1024-thread pipelined kernel
+        ((2, 3), 50000, torch.float32),  # long fp32 rows
+        ((5,), 4099, torch.bfloat16),
+        ((2, 3), 10, torch.float32),
+    ],
 )
 @pytest.mark.parametrize("temperature", [1.0, 0.7])
 def test_backward_matches_oracle_autograd(shape, vocab, dtype, temperature):
@@ -213,3 +219,34 @@ def test_full_size_properties_bf16_rows():
     lg = logits[:512].clone().requires_grad_(True)
     model_utils.log_softmax_and_gather(lg, index[:512]).sum().backward()
     assert lg.grad.float().sum(-1).abs().max().item() <= 0.05
+
+
+def test_backward_long_rows_with_tail_and_in_place():
+    """Rows long enough for the pipelined 1024-thread kernel, vocabulary not a multiple of the
+    16-byte vector (scalar tail), logits a strided view; then the same call in place through the
+    C-ABI (dlogits aliasing logits), which must give the same bits."""
+    g = torch.Generator().manual_seed(31)
+    vocab, width = 100003, 100008
+    full = (torch.randn(3, width, generator=g) * 3.0).bfloat16()
+    index = torch.randint(0, vocab, (3,), generator=g)
+    index[0] = vocab - 1  # label in the scalar tail
+    upstream = torch.tensor([0.3, -0.4, 0.0])
+    ref_in = full[:, :vocab].float().clone().requires_grad_(True)
+    o_logprob.log_softmax_and_gather(ref_in, index, None, 0.8).backward(upstream)
+    dev_full = full.to(DEV).requires_grad_(True)
+    model_utils.log_softmax_and_gather(dev_full[:, :vocab], index.to(DEV), temperature=0.8).backward(upstream.to(DEV))
+    grad = dev_full.grad
+    assert (grad[:, :vocab].float().cpu() - ref_in.grad).abs().max().item() <= _tol(torch.bfloat16)
+    assert (grad[:, vocab:] == 0).all() and (grad[2] == 0).all()
+    # in place through the raw entry point
+    from open_instruct_amd import _lib
+
+    work = full.to(DEV).clone()
+    lse = torch.logsumexp(full[:, :vocab].float() / 0.8, dim=-1).to(DEV)
+    index_d, upstream_d = index.to(DEV), upstream.to(DEV)  # kept alive until the kernel has run
+    _lib.call(
+        "oi_lsg_bwd", work.data_ptr(), 1, 1, 3, 0, width, vocab, index_d.data_ptr(), lse.data_ptr(),
+        upstream_d.data_ptr(), 1.0 / 0.8, work.data_ptr(), 0, width, torch.cuda.current_stream().cuda_stream,
+    )  # fmt: skip
+    torch.cuda.synchronize()
+    assert (work[:, :vocab].float() - grad[:, :vocab].float()).abs().max().item() <= 2.0**-8 * 0.5
