@@ -149,12 +149,14 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
             for (int j = 0; j < 4; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
     };
-    // 6 LDS reads spread over the 8 MFMAs of one k-step
+    // 6 LDS reads spread over the 8 MFMAs of one k-step.  An MFMA goes first: its wait for the
+    // current fragments then precedes every read of the next ones (a read issued ahead of that wait
+    // would be waited for as well, a full LDS round trip with the matrix pipe idle).
     auto interleave_reads = [&]() {
 #pragma unroll
         for (int q = 0; q < 6; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -182,22 +184,32 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        issue(kt + NSTAGE);
-        load_frags(kt + 1, 0, a0, b0);
-        mma(a1, b1);
-        // 8 global->LDS loads and 6 LDS reads spread over the 8 MFMAs
+        // last k-step of the k-tile: 8 MFMAs with the 8 global->LDS loads of k-tile kt+2 and the 6
+        // fragment reads of k-tile kt+1 placed between them one by one (nothing may move across the
+        // scheduling barriers: loads issued back to back would hold up the wave's MFMA issue)
+        {
+            const int64_t nkt = kt + NSTAGE;
+            const int64_t src = nkt < ktiles ? nkt : ktiles - 1;
+            const char* a_src = a_tile + src * (BK * 2);
+            const char* b_src = b_tile + src * (BK * 2);
+            uint16_t* dst = my_rows + (int)(nkt & (NSTAGE - 1)) * STAGE_ELEMS;
+            const uint16_t* nxt = lds + (int)((kt + 1) & (NSTAGE - 1)) * STAGE_ELEMS;
 #pragma unroll
-        for (int q = 0; q < 6; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            for (int q = 0; q < 8; ++q) {
+                acc[q >> 2][q & 3] =
+                    __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1[q >> 2], b1[q & 3], acc[q >> 2][q & 3], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (q & 1)
+                    __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(b_src + bo[q >> 1]),
+                                                     OI_LDS_PTR(dst + TILE_ELEMS + (q >> 1) * 8 * BK), 16, 0, 0);
+                else
+                    __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(a_src + ao[q >> 1]), OI_LDS_PTR(dst + (q >> 1) * 8 * BK),
+                                                     16, 0, 0);
+                if (q < 2) a0[q] = *reinterpret_cast<const bf16x8*>(nxt + a_base + q * 32 * BK);
+                else if (q < 6) b0[q - 2] = *reinterpret_cast<const bf16x8*>(nxt + b_base + (q - 2) * 32 * BK);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // every wave is done reading before the caller reuses the LDS (epilogue staging, next tile)
