@@ -36,14 +36,19 @@ typedef f32x16 AccTile[2][4];
 
 // XCD-aware tile order.  Consecutive workgroup ids go round-robin to the 8 XCDs, each with its own
 // L2; the 32 workgroups resident on one XCD form an 8 (m) x 4 (n) super-tile so that they share
-// operand slabs in that L2, and the 8 XCDs take super-tiles that are neighbours along m.
+// operand slabs in that L2.  The 8 XCDs take super-tiles that are neighbours along n and the sweep
+// over n completes before m advances: the chip as a whole then works on one slab of A (the larger
+// operand: lm_head rows, dZ rows) at a time, which stays in the memory-side cache while every n
+// tile passes over it, instead of streaming all of A from HBM once per n super-tile.  Measured:
+// +4 to +7 % on every shape of the lm_head path (the kernel runs at the chip's power limit, and
+// HBM traffic costs power).
 __device__ __forceinline__ bool tile_of_block(int64_t tiles_m, int64_t tiles_n, int64_t* tm, int64_t* tn) {
     const int64_t pid = blockIdx.x;
     const int64_t xcd = pid & 7, local = pid >> 3;
-    const int64_t nsm = (tiles_m + 7) / 8;
+    const int64_t nsn = (tiles_n + 3) / 4;
     const int64_t st = (local >> 5) * 8 + xcd, inner = local & 31;
-    *tm = (st % nsm) * 8 + (inner & 7);
-    *tn = (st / nsm) * 4 + (inner >> 3);
+    *tm = (st / nsn) * 8 + (inner & 7);
+    *tn = (st % nsn) * 4 + (inner >> 3);
     return *tm < tiles_m && *tn < tiles_n;
 }
 inline unsigned grid_for_tiles(int64_t tiles_m, int64_t tiles_n) {
