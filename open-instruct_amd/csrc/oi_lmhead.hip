@@ -527,7 +527,7 @@ __global__ void __launch_bounds__(256)
 
 inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
-constexpr int64_t BWD_VOCAB_CHUNK = 16384;
+constexpr int64_t BWD_VOCAB_CHUNK = 32768;
 
 struct FwdPlan {
     int64_t token_tiles, vocab_tiles, n_splits, tiles_per_split, n_pad;
