@@ -69,6 +69,18 @@ def test_rejected_arguments_return_codes_without_launching():
     assert lib.oi_grpo_terms_fwd(None, None, None, None, None, 4, 0, 0.8, 1.2, 2, None, None, None, None) == -2
     assert lib.oi_group_advantages(None, 2, 0, 0, None, None) == -1
     assert lib.oi_seq_logp_fwd(None, None, None, 2, 0, 0, None, None, None) == -1
+    # row strides beyond 2^22 elements do not fit the tile engine's 32-bit lane offsets
+    big = (1 << 22) + 64
+    assert lib.oi_lmhead_logp_fwd(None, None, None, 4, big, 32, 1.0, None, None, None, None, 0, None) == -1
+    assert lib.oi_lmhead_logp_fwd(None, None, None, big, 64, 32, 1.0, None, None, None, None, 0, None) == -1
+    assert lib.oi_gemm_bf16_tn(None, big, 4, None, 64, 4, 64, None, None, 4, 0, None) == -1
+    assert lib.oi_gemm_bf16_tn(None, 72, 4, None, 72, 4, 72, None, None, 4, 0, None) == -1  # K % 64
+    # packing and logprob statistics: missing pointers / sizes
+    assert lib.oi_pack_sequences(*([None] * 9), -1, 0, 0, *([None] * 8)) == -1
+    assert lib.oi_pack_sequences(*([None] * 9), 3, 0, 0, *([None] * 8)) == -2
+    assert lib.oi_pack_sequences(*([None] * 9), 0, 0, 0, *([None] * 8)) == 0
+    assert lib.oi_logprob_diff_stats(None, None, None, 4, None, None) == -2
+    assert lib.oi_logprob_diff_stats(None, None, None, -1, None, None) == -1
     assert lib.oi_masked_mean_workspace_bytes(4, 2, 3) == (4 + 1) * 2 * 1 * 4
     assert lib.oi_lmhead_fwd_workspace_bytes(0, 64, 10) == 0
     assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1) > lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 0)
