@@ -436,6 +436,7 @@ __global__ void __launch_bounds__(NTHREADS)
                         if (v == y) val += g;
                     }
                     d[e] = val;
+                    acc[i][j][r] = val;  // kept for the transposed copy below
                 }
                 const int vl = acc_row(wm, i, q * 4, lane);
                 uint2 pk = make_uint2(oi_pack_bf16x2(d[0], d[1]), oi_pack_bf16x2(d[2], d[3]));
@@ -452,21 +453,37 @@ __global__ void __launch_bounds__(NTHREADS)
         const oi_u32x4 v = *reinterpret_cast<const oi_u32x4*>(stage + row * STAGE_STRIDE + ch * 8);
         *reinterpret_cast<oi_u32x4*>(dz + (n0 + row) * chunk_cols + vcol0 + ch * 8) = v;
     }
-    // [vocab, token] order: every thread gathers 8 tokens of one vocabulary row
+    // [vocab, token] order: second pass through the same LDS buffer, transposed.  Neighbouring lanes
+    // hold neighbouring tokens of the same vocabulary rows, so one DPP swap per pair of rows gives
+    // every lane two tokens of one row: 4-byte LDS writes, then the same coalesced 16-byte row copy
+    // as above (a row of the tile is 512 contiguous bytes of dZ^T).
     if (dzt) {
-#pragma unroll 2
+        __syncthreads();  // everyone is done reading the [token, vocab] image
+        const bool odd = lane & 1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int nl = acc_col(wn, j, lane) & ~1;
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const float own0 = acc[i][j][2 * t], own1 = acc[i][j][2 * t + 1];
+                    const float send = odd ? own0 : own1;
+                    const float recv = __int_as_float(
+                        __builtin_amdgcn_mov_dpp(__float_as_int(send), 0xB1 /* quad_perm 1,0,3,2 */, 0xF, 0xF, true));
+                    // even lane: row 2t, tokens (nl, nl+1) = (own, neighbour); odd lane: row 2t+1
+                    const float lo = odd ? recv : own0, hi = odd ? own1 : recv;
+                    const int vl = acc_row(wm, i, 2 * t, lane) + (odd ? 1 : 0);
+                    *reinterpret_cast<uint32_t*>(stage + vl * STAGE_STRIDE + nl) = oi_pack_bf16x2(lo, hi);
+                }
+        }
+        __syncthreads();
+#pragma unroll 4
         for (int it = 0; it < 16; ++it) {
             const int cidx = tid + it * NTHREADS;
-            const int vrow = cidx & 255, nch = cidx >> 8;
-            uint32_t w[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const uint32_t lo = stage[(nch * 8 + 2 * e) * STAGE_STRIDE + vrow];
-                const uint32_t hi = stage[(nch * 8 + 2 * e + 1) * STAGE_STRIDE + vrow];
-                w[e] = lo | (hi << 16);
-            }
-            const oi_u32x4 v = {w[0], w[1], w[2], w[3]};
-            *reinterpret_cast<oi_u32x4*>(dzt + (vcol0 + vrow) * n_pad + n0 + nch * 8) = v;
+            const int row = cidx >> 5, ch = cidx & 31;
+            const oi_u32x4 v = *reinterpret_cast<const oi_u32x4*>(stage + row * STAGE_STRIDE + ch * 8);
+            *reinterpret_cast<oi_u32x4*>(dzt + (vcol0 + row) * n_pad + n0 + ch * 8) = v;
         }
     }
 }
