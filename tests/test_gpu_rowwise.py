@@ -121,6 +121,9 @@ def test_closed_forms_on_device():
         ((2, 3), 50000, torch.float32),  # long fp32 rows
         ((5,), 4099, torch.bfloat16),
         ((2, 3), 10, torch.float32),
+        ((2, 9), 50257, torch.float16),  # scalar path (rows not 16-byte aligned)
+        ((2, 3), 50264, torch.float16),  # vectorised fp16
+        ((1, 2), 131072, torch.float16),  # long fp16 rows: the pipelined kernel
     ],
 )
 @pytest.mark.parametrize("temperature", [1.0, 0.7])
