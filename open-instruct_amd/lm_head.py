@@ -19,7 +19,7 @@ from . import _lib
 
 class _FusedLMHead(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, labels, inv_temperature, want_entropy):
+    def forward(ctx, hidden, weight, labels, inv_temperature, want_entropy, compact_backward=False):
         dev = _lib.require_gpu(hidden, weight, labels)
         if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
             raise ValueError("fused lm_head expects bf16 hidden states and weight")
@@ -45,6 +45,7 @@ class _FusedLMHead(torch.autograd.Function):
             )  # fmt: skip
         ctx.save_for_backward(hid, w, lab, lse)
         ctx.inv_temperature = inv_temperature
+        ctx.compact_backward = bool(compact_backward)
         if want_entropy:
             ctx.mark_non_differentiable(entropy)
         return logprob, entropy
@@ -56,8 +57,18 @@ class _FusedLMHead(torch.autograd.Function):
         v = w.shape[0]
         need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if grad_logprob is None or not (need_h or need_w):
-            return None, None, None, None, None
+            return None, None, None, None, None, None
         g = _lib.f32c(grad_logprob)
+        keep = None
+        if ctx.compact_backward and n > 0:
+            # rows whose upstream gradient is exactly zero (zero advantage, clipped ratio with no KL
+            # term) contribute nothing to either gradient: leave them out of the three products.
+            # torch.nonzero synchronises with the host, which is why this is opt-in.
+            nz = torch.nonzero(g != 0, as_tuple=False).squeeze(1)
+            if nz.numel() < n:
+                keep, full_n = nz, n
+                hid, lab, lse, g = hid.index_select(0, nz), lab.index_select(0, nz), lse.index_select(0, nz), g.index_select(0, nz)
+                n = nz.numel()
         d_hidden = torch.empty_like(hid)
         d_weight = torch.empty_like(w) if need_w else None
         if n > 0:
@@ -70,7 +81,9 @@ class _FusedLMHead(torch.autograd.Function):
             )  # fmt: skip
         elif d_weight is not None:
             d_weight.zero_()
-        return (d_hidden if need_h else None), d_weight, None, None, None
+        if keep is not None:
+            d_hidden = torch.zeros(full_n, h, dtype=d_hidden.dtype, device=d_hidden.device).index_copy_(0, keep, d_hidden)
+        return (d_hidden if need_h else None), d_weight, None, None, None, None
 
 
 def fused_lm_head_logprobs(
@@ -80,6 +93,7 @@ def fused_lm_head_logprobs(
     temperature: float = 1.0,
     mask: torch.Tensor | None = None,
     return_entropy: bool = False,
+    compact_backward: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """``log_softmax(hidden @ weight.T / temperature)[labels]`` (+ entropy) per token, fp32.
 
@@ -88,7 +102,10 @@ def fused_lm_head_logprobs(
     (the reference's ``clamp(min=0)``, open_instruct/padding_free_collator.py:15).  ``mask`` (bool,
     same leading shape) selects the rows that are computed at all: masked-out rows cost nothing,
     return 0 and receive a zero gradient.  Differentiable with respect to ``hidden`` and
-    ``weight``; the entropy carries no gradient, as in the reference.
+    ``weight``; the entropy carries no gradient, as in the reference.  ``compact_backward=True``
+    additionally drops rows whose upstream gradient is exactly zero from the backward products
+    (zero-advantage completions, clipped ratios without a KL term); it costs one host
+    synchronisation in the backward pass and changes no result.
     """
     lead = hidden.shape[:-1]
     hid2 = hidden.reshape(-1, hidden.shape[-1])
@@ -97,11 +114,13 @@ def fused_lm_head_logprobs(
     if not float(temperature) > 0.0:
         raise ValueError(f"temperature must be positive, got {temperature}")
     if mask is None:
-        lp, ent = _FusedLMHead.apply(hid2, weight, lab1, inv_t, return_entropy)
+        lp, ent = _FusedLMHead.apply(hid2, weight, lab1, inv_t, return_entropy, compact_backward)
         return lp.reshape(lead), (ent.reshape(lead) if ent is not None else None)
     keep = mask.reshape(-1).bool()
     idx = torch.nonzero(keep, as_tuple=False).squeeze(1)
-    lp_c, ent_c = _FusedLMHead.apply(hid2.index_select(0, idx), weight, lab1.index_select(0, idx), inv_t, return_entropy)
+    lp_c, ent_c = _FusedLMHead.apply(
+        hid2.index_select(0, idx), weight, lab1.index_select(0, idx), inv_t, return_entropy, compact_backward
+    )
     lp = torch.zeros(hid2.shape[0], dtype=torch.float32, device=hidden.device).index_copy(0, idx, lp_c)
     ent = None
     if ent_c is not None:

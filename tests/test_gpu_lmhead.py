@@ -177,3 +177,28 @@ def test_fused_linear_cross_entropy_matches_oracle(num_items):
     # nothing to score: zero loss, no NaN
     empty = lm_head.fused_linear_cross_entropy(dh, dw, torch.full_like(labels, -100).to(DEV))
     assert empty.item() == 0.0
+
+
+def test_compact_backward_leaves_gradients_unchanged():
+    """Rows with an exactly zero upstream gradient may be left out of the backward products."""
+    hidden, weight, labels = _case(600, 128, 3000, seed=11, w_scale=3.0 / math.sqrt(128))
+    g = torch.Generator().manual_seed(12)
+    upstream = torch.randn(600, generator=g)
+    upstream[torch.rand(600, generator=g) < 0.6] = 0.0
+    grads = []
+    for compact in (False, True):
+        dh = hidden.to(DEV).requires_grad_(True)
+        dw = weight.to(DEV).requires_grad_(True)
+        out, _ = lm_head.fused_lm_head_logprobs(dh, dw, labels.to(DEV), 0.9, compact_backward=compact)
+        out.backward(upstream.to(DEV))
+        grads.append((dh.grad.float().cpu(), dw.grad.float().cpu()))
+    (h0, w0), (h1, w1) = grads
+    assert torch.equal(h0[upstream == 0], torch.zeros_like(h0[upstream == 0])) and torch.equal(h1[upstream == 0], h0[upstream == 0])
+    assert (h0 - h1).abs().max().item() <= h0.abs().max().item() * 2**-7
+    assert (w0 - w1).abs().max().item() <= w0.abs().max().item() * 2**-7 + 1e-6
+    # nothing to propagate at all
+    dh = hidden.to(DEV).requires_grad_(True)
+    dw = weight.to(DEV).requires_grad_(True)
+    out, _ = lm_head.fused_lm_head_logprobs(dh, dw, labels.to(DEV), compact_backward=True)
+    out.backward(torch.zeros(600, device=DEV))
+    assert not dh.grad.any() and not dw.grad.any()
