@@ -7,7 +7,8 @@ synthetic inputs that already live in HBM.  Workloads are the BASELINE configs:
 
   c3 (default, the headline metric): fused lm_head + logprob + entropy + GRPO loss, fwd + bwd, at
       Llama-3.1-8B shape: hidden bf16 [32768, 4096], W bf16 [128256, 4096], 70 % response tokens.
-  c2: GRPO loss on materialised bf16 logits [64, 1024, 128256], fwd + bwd (HBM-bound).
+  c2: GRPO loss on materialised bf16 logits [64, 1024, 128256], fwd + bwd (HBM-bound), single pass;
+      c2-two-pass keeps the reference's order of operations (the logits are read twice).
   c1: logprob + entropy + masked_mean on fp32 logits [4, 512, 32000], forward only.
   c4: packed batch at OLMo-2-7B shape (16 sequences, cu_seqlens, V=100352), per-sequence sums + GRPO loss.
   c5: DPO at Llama-3.1-70B head shape: hidden [32768, 8192], W [128256, 8192], bwd to dHidden only.
@@ -41,7 +42,7 @@ PEAK_BF16_TFLOPS = 2500.0
 # profiles/; workloads without a counter run report null.
 MEASURED_TRAFFIC_BYTES = {
     "c3": 44.57e9 + 0.37e9,  # lmhead_fwd_kernel: L2 misses of the tiled operand re-reads (1.24 GB unique)
-    "c2": 16.83e9 + 0.0e9,  # lsg_entropy_fwd_kernel: 1.00x the logits
+    "c2-two-pass": 16.83e9 + 0.0e9,  # lsg_entropy_fwd_kernel: 1.00x the logits
 }
 
 
@@ -139,7 +140,10 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False):
     return step, info
 
 
-def make_c2(torch, oi, rows_b=64, t=1024, vocab=128256):
+def make_c2(torch, oi, rows_b=64, t=1024, vocab=128256, single_pass=True):
+    """GRPO loss on materialised logits.  single_pass: forward and gradient in one read and one write
+    of the logits (grpo_loss_on_logits); otherwise the reference's order of operations with the
+    logits read twice (log_softmax_and_gather -> loss -> backward)."""
     dev = "cuda:0"
     torch.manual_seed(0)
     logits = torch.empty(rows_b, t, vocab, device=dev, dtype=torch.bfloat16)
@@ -157,7 +161,7 @@ def make_c2(torch, oi, rows_b=64, t=1024, vocab=128256):
     cfg = _cfg()
     fwd_timer = EventTimer(torch)
 
-    def step():
+    def step_two_pass():
         logits.grad = None
         with fwd_timer:
             lp = oi.model_utils.log_softmax_and_gather(logits, labels)
@@ -165,7 +169,33 @@ def make_c2(torch, oi, rows_b=64, t=1024, vocab=128256):
         loss.backward()
         return loss
 
+    plain_call = oi._lib.call
+
+    def timed_call(name, *args):
+        if name != "oi_lsg_grpo_fwd_bwd":
+            return plain_call(name, *args)
+        with fwd_timer:
+            return plain_call(name, *args)
+
+    def step_single_pass():
+        logits.grad = None
+        loss, _, _, _ = oi.grpo_utils.grpo_loss_on_logits(logits, labels, old, ref, adv, mask, cfg)
+        loss.backward()
+        return loss
+
     n = rows_b * t
+    if single_pass:
+        oi._lib.call = timed_call
+        info = {
+            "tokens": n,
+            "rows_multiplied": n,
+            "bytes_step": 2.0 * n * vocab * 2,
+            "kernel": "lsg_grpo_fused_kernel (row held in registers: logprob, entropy, GRPO derivative and dlogits in one read + one write)",
+            "alg_per_launch": 2.0 * n * vocab * 2,
+            "bound": "hbm",
+            "timer": fwd_timer,
+        }
+        return step_single_pass, info
     info = {
         "tokens": n,
         "rows_multiplied": n,
@@ -175,7 +205,7 @@ def make_c2(torch, oi, rows_b=64, t=1024, vocab=128256):
         "bound": "hbm",
         "timer": fwd_timer,
     }
-    return step, info
+    return step_two_pass, info
 
 
 def make_c1(torch, oi):
@@ -338,7 +368,7 @@ def cpu_baseline(torch, workload):
             loss.backward()
 
         sample = f"{n} of 32768 token rows at full H={hdim}, V={vocab}; fwd+bwd; bf16 GEMM + fp32 log_softmax"
-    elif workload == "c2":
+    elif workload in ("c2", "c2-two-pass"):
         n, vocab = 8192, 128256
         logits = (torch.randn(n, vocab) * 3.0).bfloat16().requires_grad_(True)
         labels = torch.randint(0, vocab, (n,))
@@ -417,7 +447,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "pack"])
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c2-two-pass", "c3", "c4", "c5", "pack"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-library-gemm", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -450,7 +480,11 @@ def main():
         dtype = "bf16"
     elif args.workload == "c2":
         step, info = make_c2(torch, oi)
-        name = "c2: GRPO loss on materialised bf16 logits [64,1024,128256], fwd+bwd"
+        name = "c2: GRPO loss on materialised bf16 logits [64,1024,128256], fwd+bwd in one read + one write of the logits"
+        dtype = "bf16"
+    elif args.workload == "c2-two-pass":
+        step, info = make_c2(torch, oi, single_pass=False)
+        name = "c2: GRPO loss on materialised bf16 logits [64,1024,128256], fwd+bwd, reference order (logits read twice)"
         dtype = "bf16"
     elif args.workload == "pack":
         step, info = make_pack(torch, oi)

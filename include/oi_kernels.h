@@ -82,6 +82,31 @@ int oi_lsg_bwd(const void* logits, int dtype, int64_t n_outer, int64_t n_inner, 
                const float* grad_logprob, float inv_temperature, void* dlogits, int64_t out_stride_outer,
                int64_t out_stride_inner, void* stream);
 
+/*
+ * GRPO on materialised logits in one launch: forward (logprob / entropy / lse as
+ * oi_lsg_entropy_fwd) and the gradient of the GRPO loss with respect to the logits.  Every row is
+ * read twice by the same workgroup in close succession, so the second read is served by the
+ * caches: HBM sees one read and one write of the [rows, vocab] tensor instead of two reads and a
+ * write.  Fuses the sequence open_instruct/grpo_utils.py:541-574 (forward_for_logprobs) ->
+ * open_instruct/grpo_utils.py:504-538 (compute_grpo_loss) -> open_instruct/grpo_fast.py:702-724
+ * (masked mean, backward) for callers that hold the logits.
+ *
+ *   ratio = exp(logprob - old) (1 when old_logprobs is NULL), loss_token = pg + beta * kl as in
+ *   oi_grpo_terms_fwd, g = token_coef[row] * d loss_token / d logprob,
+ *   dlogits[row, j] = g * inv_T * (1[j == index] - softmax_j).
+ * token_coef (fp32 per row) carries the loss denominators, which depend on the mask alone:
+ * scale / denominator on response tokens, 0 elsewhere (such rows get a zero gradient row).
+ * Requirement: 16-byte aligned rows (pointers and strides of logits and dlogits); OI_EALIGN
+ * otherwise (use the two-pass entry points).  dlogits must not alias logits.  The scalar loss and
+ * its statistics come from oi_grpo_fused_fwd on `logprob`.
+ */
+int oi_lsg_grpo_fwd_bwd(const void* logits, int dtype, int64_t n_outer, int64_t n_inner, int64_t stride_outer,
+                        int64_t stride_inner, int64_t vocab, const int64_t* index, float inv_temperature,
+                        const float* old_logprobs, const float* ref_logprobs, const float* advantages,
+                        const float* rho_weights, const float* token_coef, int loss_fn, float ratio_lo,
+                        float ratio_hi, int kl_estimator, float beta, float* logprob, float* entropy, float* lse,
+                        void* dlogits, int64_t out_stride_outer, int64_t out_stride_inner, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Per-token GRPO loss terms.  Carries open_instruct/grpo_utils.py:504-538 (compute_grpo_loss)
  * with open_instruct/model_utils.py:793-818 (estimate_kl) for the selected estimator.

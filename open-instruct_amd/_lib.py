@@ -26,6 +26,10 @@ SIGNATURES: dict[str, tuple] = {
     "oi_error_string": (c_char_p, [_I]),
     "oi_lsg_entropy_fwd": (_I, [_P, _I, _I64, _I64, _I64, _I64, _I64, _P, _F, _P, _P, _P, _P]),
     "oi_lsg_bwd": (_I, [_P, _I, _I64, _I64, _I64, _I64, _I64, _P, _P, _P, _F, _P, _I64, _I64, _P]),
+    "oi_lsg_grpo_fwd_bwd": (
+        _I,
+        [_P, _I, _I64, _I64, _I64, _I64, _I64, _P, _F, _P, _P, _P, _P, _P, _I, _F, _F, _I, _F, _P, _P, _P, _P, _I64, _I64, _P],
+    ),
     "oi_grpo_terms_fwd": (_I, [_P, _P, _P, _P, _P, _I64, _I, _F, _F, _I, _P, _P, _P, _P]),
     "oi_grpo_terms_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I64, _I, _F, _F, _I, _P, _P, _P]),
     "oi_grpo_fused_workspace_bytes": (_SZ, [_I64, _I64]),

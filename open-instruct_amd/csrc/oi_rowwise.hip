@@ -6,16 +6,20 @@
 // waves through LDS.  The kernel is HBM-bound: 2 (bf16) or 4 (fp32) bytes per logit, nothing
 // else of size [rows, vocab] is read or written by the forward.
 #include "oi_common.h"
+#include "oi_grpo_math.h"
 
 namespace {
 
 struct F32Row {
     typedef float elem_t;
     static constexpr int VEC = 4;
-    static __device__ __forceinline__ void load_vec(const elem_t* p, float (&z)[VEC]) {
-        oi_f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const oi_f32x4*>(p));
-        z[0] = v.x; z[1] = v.y; z[2] = v.z; z[3] = v.w;
+    typedef oi_f32x4 raw_t;
+    static __device__ __forceinline__ raw_t load_raw(const elem_t* p) {
+        return __builtin_nontemporal_load(reinterpret_cast<const oi_f32x4*>(p));
     }
+    static __device__ __forceinline__ raw_t load_raw_cached(const elem_t* p) { return *reinterpret_cast<const oi_f32x4*>(p); }
+    static __device__ __forceinline__ void unpack(raw_t v, float (&z)[VEC]) { z[0] = v.x; z[1] = v.y; z[2] = v.z; z[3] = v.w; }
+    static __device__ __forceinline__ void load_vec(const elem_t* p, float (&z)[VEC]) { unpack(load_raw(p), z); }
     static __device__ __forceinline__ float load_one(const elem_t* p) { return *p; }
     static __device__ __forceinline__ void store_vec(elem_t* p, const float (&z)[VEC]) {
         oi_f32x4 v = {z[0], z[1], z[2], z[3]};
@@ -27,13 +31,18 @@ struct F32Row {
 struct BF16Row {
     typedef uint16_t elem_t;
     static constexpr int VEC = 8;
-    static __device__ __forceinline__ void load_vec(const elem_t* p, float (&z)[VEC]) {
-        oi_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const oi_u32x4*>(p));
+    typedef oi_u32x4 raw_t;
+    static __device__ __forceinline__ raw_t load_raw(const elem_t* p) {
+        return __builtin_nontemporal_load(reinterpret_cast<const oi_u32x4*>(p));
+    }
+    static __device__ __forceinline__ raw_t load_raw_cached(const elem_t* p) { return *reinterpret_cast<const oi_u32x4*>(p); }
+    static __device__ __forceinline__ void unpack(raw_t v, float (&z)[VEC]) {
         z[0] = oi_bf16lo_to_f32(v.x); z[1] = oi_bf16hi_to_f32(v.x);
         z[2] = oi_bf16lo_to_f32(v.y); z[3] = oi_bf16hi_to_f32(v.y);
         z[4] = oi_bf16lo_to_f32(v.z); z[5] = oi_bf16hi_to_f32(v.z);
         z[6] = oi_bf16lo_to_f32(v.w); z[7] = oi_bf16hi_to_f32(v.w);
     }
+    static __device__ __forceinline__ void load_vec(const elem_t* p, float (&z)[VEC]) { unpack(load_raw(p), z); }
     static __device__ __forceinline__ float load_one(const elem_t* p) { return __uint_as_float((uint32_t)(*p) << 16); }
     static __device__ __forceinline__ void store_vec(elem_t* p, const float (&z)[VEC]) {
         oi_u32x4 v = {oi_pack_bf16x2(z[0], z[1]), oi_pack_bf16x2(z[2], z[3]), oi_pack_bf16x2(z[4], z[5]),
@@ -46,8 +55,12 @@ struct BF16Row {
 struct F16Row {
     typedef uint16_t elem_t;
     static constexpr int VEC = 8;
-    static __device__ __forceinline__ void load_vec(const elem_t* p, float (&z)[VEC]) {
-        oi_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const oi_u32x4*>(p));
+    typedef oi_u32x4 raw_t;
+    static __device__ __forceinline__ raw_t load_raw(const elem_t* p) {
+        return __builtin_nontemporal_load(reinterpret_cast<const oi_u32x4*>(p));
+    }
+    static __device__ __forceinline__ raw_t load_raw_cached(const elem_t* p) { return *reinterpret_cast<const oi_u32x4*>(p); }
+    static __device__ __forceinline__ void unpack(raw_t v, float (&z)[VEC]) {
         uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -55,6 +68,7 @@ struct F16Row {
             z[2 * i + 1] = oi_f16bits_to_f32((uint16_t)(w[i] >> 16));
         }
     }
+    static __device__ __forceinline__ void load_vec(const elem_t* p, float (&z)[VEC]) { unpack(load_raw(p), z); }
     static __device__ __forceinline__ float load_one(const elem_t* p) { return oi_f16bits_to_f32(*p); }
     static __device__ __forceinline__ void store_vec(elem_t* p, const float (&z)[VEC]) {
         uint32_t w[4];
@@ -404,6 +418,186 @@ int launch_bwd(const void* logits, int64_t rows, int64_t n_inner, int64_t so, in
     return oi_launch_status();
 }
 
+// ---------------------------------------------------------------------------------------------
+// GRPO on materialised logits in one launch: forward statistics and the gradient with respect to
+// the logits, with the second read of a row served by the caches instead of HBM.
+//
+// A token's upstream gradient depends on nothing but that token's own logprob and side inputs
+// (old / reference logprobs, advantage, weight) once the loss denominators are known, and those
+// depend on the mask alone.  So one 1024-thread workgroup per row reduces the softmax statistics
+// (ordinary loads, so that the row stays in the memory-side cache), evaluates the GRPO derivative
+// of the token and immediately streams the same row again (non-temporal loads, it is not needed
+// any more) to write d logits.  Only a few hundred rows (one or two per CU, 256 KB each at a 128 k
+// vocabulary) are between their two reads at any time, far less than the 256 MB of that cache.
+// A version that kept the row in registers between the passes (512 threads x 32 vectors) was
+// slower than two separate kernels: one workgroup per CU with nothing to overlap its load, compute
+// and store phases.  `token_coef` carries scale / denominator per token (0 on masked-out tokens).
+// ---------------------------------------------------------------------------------------------
+constexpr int FUSED_ROW_THREADS = 1024;
+constexpr int FUSED_ROW_U = 4;
+
+template <typename R>
+__global__ void __launch_bounds__(FUSED_ROW_THREADS)
+    lsg_grpo_fused_kernel(const typename R::elem_t* __restrict__ logits, int64_t n_inner, int64_t stride_outer,
+                          int64_t stride_inner, int64_t vocab, const int64_t* __restrict__ index, float inv_t,
+                          const float* __restrict__ old_lp, const float* __restrict__ ref_lp,
+                          const float* __restrict__ adv, const float* __restrict__ rho,
+                          const float* __restrict__ token_coef, GrpoCfg cfg, float beta,
+                          float* __restrict__ logprob, float* __restrict__ entropy, float* __restrict__ lse_out,
+                          typename R::elem_t* __restrict__ dlogits, int64_t out_stride_outer,
+                          int64_t out_stride_inner) {
+    constexpr int VEC = R::VEC;
+    constexpr int NW = FUSED_ROW_THREADS / OI_WAVE;
+    constexpr int U = FUSED_ROW_U;
+    constexpr int64_t nthr = FUSED_ROW_THREADS;
+    __shared__ float sm[3][NW];
+    __shared__ float bcast[2];
+    const int64_t row = blockIdx.x;
+    const typename R::elem_t* p = logits + row_offset(row, n_inner, stride_outer, stride_inner);
+    typename R::elem_t* q = dlogits + row_offset(row, n_inner, out_stride_outer, out_stride_inner);
+    const int tid = threadIdx.x;
+    const int64_t nvec = vocab / VEC;
+    const float c = inv_t * OI_LOG2E;
+
+    RowStat st = {OI_NEG_BIG, 0.f, 0.f};
+    {
+        int64_t i = tid;
+        for (; i + (U - 1) * nthr < nvec; i += U * nthr) {
+            typename R::raw_t raw[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) raw[u] = R::load_raw_cached(p + (i + u * nthr) * VEC);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float z[VEC];
+                R::unpack(raw[u], z);
+                stat_update<VEC, true>(st, z, c);
+            }
+        }
+        for (; i < nvec; i += nthr) {
+            float z[VEC];
+            R::unpack(R::load_raw_cached(p + i * VEC), z);
+            stat_update<VEC, true>(st, z, c);
+        }
+        for (int64_t j = nvec * VEC + tid; j < vocab; j += nthr) stat_update1<true>(st, R::load_one(p + j), c);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        RowStat o;
+        o.m = __shfl_xor(st.m, off, OI_WAVE);
+        o.s = __shfl_xor(st.s, off, OI_WAVE);
+        o.t = __shfl_xor(st.t, off, OI_WAVE);
+        st = stat_merge(st, o);
+    }
+    const int wave = tid >> 6, lane = tid & 63;
+    if (lane == 0) {
+        sm[0][wave] = st.m;
+        sm[1][wave] = st.s;
+        sm[2][wave] = st.t;
+    }
+    __syncthreads();
+    int64_t y = index[row];
+    y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
+    if (tid == 0) {
+        RowStat tot = {sm[0][0], sm[1][0], sm[2][0]};
+        for (int w = 1; w < NW; ++w) {
+            RowStat o = {sm[0][w], sm[1][w], sm[2][w]};
+            tot = stat_merge(tot, o);
+        }
+        const double ln2 = 0.69314718055994530942;
+        const double log2s = log2((double)tot.s);
+        const double lse = ((double)tot.m + log2s) * ln2;
+        const float zy = R::load_one(p + y);
+        const float lp = (float)((double)zy * (double)inv_t - lse);
+        logprob[row] = lp;
+        if (entropy) entropy[row] = (float)((log2s - (double)tot.t / (double)tot.s) * ln2);
+        if (lse_out) lse_out[row] = (float)lse;
+        const float coef = token_coef[row];
+        float g = 0.f;
+        if (coef != 0.f) {
+            const float ratio = old_lp ? expf(lp - old_lp[row]) : 1.f;
+            const float w = rho ? rho[row] : 1.f;
+            g = coef * grpo_token_dnew(lp, ratio, adv[row], ref_lp != nullptr, ref_lp ? ref_lp[row] : 0.f, w, cfg, beta);
+        }
+        bcast[0] = g * inv_t;
+        bcast[1] = (float)lse * OI_LOG2E;
+    }
+    __syncthreads();
+    const float g = bcast[0], l2 = bcast[1];
+    const float ng = -g;
+    if (g == 0.f) {
+        float zero[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) zero[j] = 0.f;
+        for (int64_t i = tid; i < nvec; i += nthr) R::store_vec(q + i * VEC, zero);
+        for (int64_t j = nvec * VEC + tid; j < vocab; j += nthr) R::store_one(q + j, 0.f);
+        return;
+    }
+    // second pass: the row was read moments ago by this workgroup
+    int64_t i = tid;
+    float z[U][VEC], zn[U][VEC];
+    if (i + (U - 1) * nthr < nvec) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) R::load_vec(p + (i + u * nthr) * VEC, z[u]);
+    }
+    for (; i + (U - 1) * nthr < nvec; i += U * nthr) {
+        const int64_t nx = i + U * nthr;
+        const bool more = nx + (U - 1) * nthr < nvec;
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) R::load_vec(p + (nx + u * nthr) * VEC, zn[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t base = (i + u * nthr) * VEC;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) z[u][j] = ng * __builtin_amdgcn_exp2f(fmaf(z[u][j], c, -l2));
+            if (y >= base && y < base + VEC) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    if (base + j == y) z[u][j] += g;
+            }
+            R::store_vec(q + base, z[u]);
+        }
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) z[u][j] = zn[u][j];
+        }
+    }
+    for (; i < nvec; i += nthr) {
+        float w[VEC];
+        const int64_t base = i * VEC;
+        R::load_vec(p + base, w);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            w[j] = ng * __builtin_amdgcn_exp2f(fmaf(w[j], c, -l2));
+            if (base + j == y) w[j] += g;
+        }
+        R::store_vec(q + base, w);
+    }
+    for (int64_t j = nvec * VEC + tid; j < vocab; j += nthr) {
+        float d = ng * __builtin_amdgcn_exp2f(fmaf(R::load_one(p + j), c, -l2));
+        if (j == y) d += g;
+        R::store_one(q + j, d);
+    }
+}
+
+template <typename R>
+int launch_grpo_fused(const void* logits, int64_t rows, int64_t n_inner, int64_t so, int64_t si, int64_t vocab,
+                      const int64_t* index, float inv_t, const float* old_lp, const float* ref_lp, const float* adv,
+                      const float* rho, const float* coef, GrpoCfg cfg, float beta, float* logprob, float* entropy,
+                      float* lse, void* dlogits, int64_t oso, int64_t osi, hipStream_t stream) {
+    typedef typename R::elem_t E;
+    const bool vec = oi_aligned(logits, 16) && oi_aligned(dlogits, 16) && (so % R::VEC == 0) && (si % R::VEC == 0) &&
+                     (oso % R::VEC == 0) && (osi % R::VEC == 0);
+    OI_RETURN_IF(!vec, OI_EALIGN);
+    hipLaunchKernelGGL((lsg_grpo_fused_kernel<R>), dim3((unsigned)rows), dim3(FUSED_ROW_THREADS), 0, stream,
+                       static_cast<const E*>(logits), n_inner, so, si, vocab, index, inv_t, old_lp, ref_lp, adv, rho, coef,
+                       cfg, beta, logprob, entropy, lse, static_cast<E*>(dlogits), oso, osi);
+    return oi_launch_status();
+}
+
 int check_rows(const void* logits, int64_t n_outer, int64_t n_inner, int64_t so, int64_t si, int64_t vocab,
                const int64_t* index, float inv_t, int64_t* rows) {
     OI_RETURN_IF(n_outer < 0 || n_inner < 0 || vocab <= 0, OI_EINVAL);
@@ -473,5 +667,42 @@ extern "C" int oi_lsg_bwd(const void* logits, int dtype, int64_t n_outer, int64_
         default:
             return launch_bwd<F16Row>(logits, rows, n_inner, stride_outer, stride_inner, vocab, index, lse,
                                       grad_logprob, inv_temperature, dlogits, out_stride_outer, out_stride_inner, s);
+    }
+}
+
+extern "C" int oi_lsg_grpo_fwd_bwd(const void* logits, int dtype, int64_t n_outer, int64_t n_inner, int64_t stride_outer,
+                                   int64_t stride_inner, int64_t vocab, const int64_t* index, float inv_temperature,
+                                   const float* old_logprobs, const float* ref_logprobs, const float* advantages,
+                                   const float* rho_weights, const float* token_coef, int loss_fn, float ratio_lo,
+                                   float ratio_hi, int kl_estimator, float beta, float* logprob, float* entropy,
+                                   float* lse, void* dlogits, int64_t out_stride_outer, int64_t out_stride_inner,
+                                   void* stream) {
+    int64_t rows = 0;
+    const int rc = check_rows(logits, n_outer, n_inner, stride_outer, stride_inner, vocab, index, inv_temperature, &rows);
+    if (rc != OI_OK) return rc;
+    OI_RETURN_IF(dtype != OI_DTYPE_F32 && dtype != OI_DTYPE_BF16 && dtype != OI_DTYPE_F16, OI_EDTYPE);
+    OI_RETURN_IF(loss_fn != OI_LOSS_DAPO && loss_fn != OI_LOSS_CISPO, OI_EINVAL);
+    OI_RETURN_IF(kl_estimator < 0 || kl_estimator > 3, OI_EINVAL);
+    if (rows == 0) return OI_OK;
+    OI_RETURN_IF(!advantages || !token_coef || !logprob || !dlogits, OI_ENULL);
+    OI_RETURN_IF(out_stride_outer < 0 || out_stride_inner < 0 || (out_stride_inner < vocab && n_inner > 1), OI_EINVAL);
+    const GrpoCfg cfg = {loss_fn, ratio_lo, ratio_hi, kl_estimator};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case OI_DTYPE_F32:
+            return launch_grpo_fused<F32Row>(logits, rows, n_inner, stride_outer, stride_inner, vocab, index,
+                                             inv_temperature, old_logprobs, ref_logprobs, advantages, rho_weights,
+                                             token_coef, cfg, beta, logprob, entropy, lse, dlogits, out_stride_outer,
+                                             out_stride_inner, s);
+        case OI_DTYPE_BF16:
+            return launch_grpo_fused<BF16Row>(logits, rows, n_inner, stride_outer, stride_inner, vocab, index,
+                                              inv_temperature, old_logprobs, ref_logprobs, advantages, rho_weights,
+                                              token_coef, cfg, beta, logprob, entropy, lse, dlogits, out_stride_outer,
+                                              out_stride_inner, s);
+        default:
+            return launch_grpo_fused<F16Row>(logits, rows, n_inner, stride_outer, stride_inner, vocab, index,
+                                             inv_temperature, old_logprobs, ref_logprobs, advantages, rho_weights,
+                                             token_coef, cfg, beta, logprob, entropy, lse, dlogits, out_stride_outer,
+                                             out_stride_inner, s);
     }
 }

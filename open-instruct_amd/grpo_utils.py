@@ -323,6 +323,134 @@ def grpo_loss_fused(
     return loss, {name: stats[i] for i, name in enumerate(GRPO_STAT_NAMES)}
 
 
+# ----------------------------------------------------------------------------------------------
+# GRPO on materialised logits: forward + gradient in one read and one write of the logits
+# ----------------------------------------------------------------------------------------------
+def _token_coef(mask: torch.Tensor, axis: int | None, loss_denominator: float | None, dp_scale: float) -> torch.Tensor:
+    """``scale / denominator`` on response tokens, 0 elsewhere: the factor that ``masked_mean``
+    (open_instruct/rl_utils.py:426-448) puts in front of every token's loss.  Device arithmetic only."""
+    m = mask.to(torch.float32)
+    if axis is None:
+        den = m.sum() if loss_denominator is None else torch.full((), float(loss_denominator), device=m.device)
+        inv = torch.where(den > 0, 1.0 / den.clamp(min=1e-30), torch.zeros_like(den))
+        return m * (inv * float(dp_scale))
+    den = m.sum(dim=1, keepdim=True) if loss_denominator is None else torch.full_like(m[:, :1], float(loss_denominator))
+    inv = torch.where(den > 0, 1.0 / den.clamp(min=1e-30), torch.zeros_like(den))
+    return m * (inv * (float(dp_scale) / m.shape[0]))
+
+
+def _single_pass_ok(view: torch.Tensor, so: int, si: int) -> bool:
+    """Rows must start on 16-byte boundaries for the fused kernel (the gradient tensor is allocated
+    contiguous here, so with an aligned vocabulary size it qualifies whenever the logits do)."""
+    vec = 16 // view.element_size()
+    return view.data_ptr() % 16 == 0 and so % vec == 0 and si % vec == 0 and view.shape[-1] % vec == 0
+
+
+def _grpo_on_logits_launch(logits, labels, old, ref, adv, rho, coef, inv_temperature, cfg, drop_last):
+    """One launch: logprob, entropy and the gradient of the loss with respect to ``logits``."""
+    dev = _lib.require_gpu(logits, labels, adv, coef)
+    view = logits[..., :-1, :] if drop_last else logits
+    view, n_outer, n_inner, so, si = model_utils._row_layout(view)
+    dlogits = torch.empty(logits.shape, dtype=logits.dtype, device=dev)
+    out_view = dlogits[..., :-1, :] if drop_last else dlogits
+    if drop_last:
+        dlogits[..., -1, :].zero_()
+    _, _, _, oso, osi = model_utils._row_layout(out_view)
+    loss_fn, lo, hi, kl_estimator, beta = cfg
+    logprob = torch.empty(labels.shape, dtype=torch.float32, device=dev)
+    entropy = torch.empty(labels.shape, dtype=torch.float32, device=dev)
+    if n_outer * n_inner > 0:
+        _lib.call(
+            "oi_lsg_grpo_fwd_bwd", view.data_ptr(), _lib.DTYPE_TAGS[view.dtype], n_outer, n_inner, so, si,
+            view.shape[-1], labels.data_ptr(), inv_temperature, _lib.ptr(old), _lib.ptr(ref), adv.data_ptr(),
+            _lib.ptr(rho), coef.data_ptr(), loss_fn, lo, hi, kl_estimator, beta, logprob.data_ptr(),
+            entropy.data_ptr(), None, out_view.data_ptr(), oso, osi, _lib.stream_of(view),
+        )  # fmt: skip
+    return logprob, entropy, dlogits
+
+
+class _AttachLogitsGrad(torch.autograd.Function):
+    """Identity on the loss value whose backward hands out the gradient computed in the forward."""
+
+    @staticmethod
+    def forward(ctx, loss, logits, dlogits):
+        ctx.save_for_backward(dlogits)
+        return loss.clone()
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        (dlogits,) = ctx.saved_tensors
+        # the usual upstream gradient of a loss is exactly 1: then the stored tensor is the answer
+        # as it is; anything else costs one more pass over it (and one host synchronisation here)
+        if float(grad_loss) != 1.0:
+            dlogits = dlogits * grad_loss.to(dlogits.dtype)
+        return None, dlogits, None
+
+
+def grpo_loss_on_logits(
+    logits: torch.Tensor,
+    labels: torch.Tensor,
+    old_logprobs: torch.Tensor | None,
+    ref_logprobs: torch.Tensor | None,
+    advantages: torch.Tensor,
+    response_mask: torch.Tensor,
+    config,
+    temperature: float = 1.0,
+    rho_weights: torch.Tensor | None = None,
+    loss_denominator: float | None = None,
+    axis: int | None = None,
+    dp_scale: float = 1.0,
+    drop_last: bool = False,
+) -> tuple[torch.Tensor, dict[str, torch.Tensor], torch.Tensor, torch.Tensor]:
+    """GRPO loss straight from materialised logits; returns ``(loss, stats, logprobs, entropy)``.
+
+    Same result as ``forward_for_logprobs`` → ``grpo_loss_fused`` (open_instruct/grpo_utils.py:541-574,
+    open_instruct/grpo_fast.py:702-724) and the same gradient with respect to ``logits`` after
+    ``loss.backward()``, but HBM sees the ``[B, T, V]`` tensor read once and its gradient written
+    once (the second read of a row comes from the caches): a token's upstream gradient depends only on its own logprob and side inputs once the
+    denominators are known, and those come from the mask.  The gradient is computed in the
+    forward call and stored (one tensor of the logits' shape and dtype, which the backward pass
+    would allocate anyway).  ``logits`` is ``[B, T, V]`` (``[B, T + 1, V]`` with ``drop_last``),
+    ``labels`` and the side tensors ``[B, T]``.  ``old_logprobs=None`` means ``old =
+    new.detach()``.  ``logprobs`` and ``entropy`` are returned detached, for logging.  Rows that do
+    not fit the single-pass kernel (vocabulary not a multiple of the 16-byte vector, more than
+    16384 vectors, unaligned views) go through the two-pass kernels with identical results.
+    """
+    if axis not in (None, 1, -1):
+        raise ValueError("axis must be None or the token axis (1)")
+    if loss_denominator is not None and float(loss_denominator) <= 0.0:
+        raise ValueError("loss_denominator must be positive when given")
+    if labels.ndim != 2 or tuple(response_mask.shape) != tuple(labels.shape):
+        raise ValueError("labels and response_mask must be [B, T]")
+    inv_t = model_utils._inv_temperature(temperature)
+    view = logits[..., :-1, :] if drop_last else logits
+    if tuple(view.shape[:-1]) != tuple(labels.shape):
+        raise ValueError(f"labels {tuple(labels.shape)} do not match logits rows {tuple(view.shape[:-1])}")
+    layout_view, _, _, so, si = model_utils._row_layout(view)
+    if not logits.requires_grad or not _single_pass_ok(layout_view, so, si) or logits.dtype not in _lib.DTYPE_TAGS:
+        logprob, entropy = model_utils.logprob_and_entropy(logits, labels, temperature=temperature, drop_last=drop_last)
+        loss, stats = grpo_loss_fused(
+            logprob, old_logprobs, ref_logprobs, advantages, response_mask, config, rho_weights=rho_weights,
+            entropy=entropy, loss_denominator=loss_denominator, axis=axis, dp_scale=dp_scale,
+        )  # fmt: skip
+        return loss, stats, logprob.detach(), entropy
+    lo, hi = _clip_bounds(config)
+    cfg = (_loss_fn_tag(config), lo, hi, int(config.kl_estimator), float(config.beta))
+    mask = response_mask if response_mask.dtype == torch.bool else response_mask != 0
+    coef = _token_coef(mask, None if axis is None else 1, loss_denominator, dp_scale).contiguous()
+    f32 = lambda t: None if t is None else _lib.f32c(t.detach())  # noqa: E731
+    with torch.no_grad():
+        logprob, entropy, dlogits = _grpo_on_logits_launch(
+            logits.detach(), labels.long().contiguous(), f32(old_logprobs), f32(ref_logprobs), f32(advantages),
+            f32(rho_weights), coef, inv_t, cfg, drop_last,
+        )  # fmt: skip
+        loss, stats = grpo_loss_fused(
+            logprob, old_logprobs, ref_logprobs, advantages, response_mask, config, rho_weights=rho_weights,
+            entropy=entropy, loss_denominator=loss_denominator, axis=axis, dp_scale=dp_scale,
+        )  # fmt: skip
+    return _AttachLogitsGrad.apply(loss, logits, dlogits), stats, logprob, entropy
+
+
 def group_advantages(scores: torch.Tensor, group_size: int, normalization: str = "standard") -> torch.Tensor:
     """Group-normalised advantages; open_instruct/data_loader.py:1472-1484 on the device.
 

@@ -489,3 +489,113 @@ def test_reference_cache_build_through_concatenated_forward():
             assert abs(got - exp.item()) <= 1e-4, (side, i, got, exp.item())
     picked = cache[torch.tensor([1, 3], device=DEV)]
     assert picked["chosen_logps"].shape == (2,)
+
+
+@pytest.mark.parametrize("dtype,vocab", [(torch.float32, 64), (torch.bfloat16, 4096), (torch.bfloat16, 4099), (torch.float16, 1000)])
+@pytest.mark.parametrize("loss_fn,axis,denominator,with_old,with_ref,drop_last", [
+    ("dapo", None, None, True, True, False),
+    ("dapo", 1, None, True, True, True),
+    ("cispo", None, 77.0, True, False, False),
+    ("dapo", None, None, False, True, True),
+])  # fmt: skip
+def test_grpo_loss_on_logits_single_pass(dtype, vocab, loss_fn, axis, denominator, with_old, with_ref, drop_last):
+    """One read + one write of the logits (open_instruct/grpo_utils.py:541-574 -> :504-538 ->
+    open_instruct/grpo_fast.py:702-724 fused) against the CPU oracle chain and against the two-pass
+    kernels.  vocab 4099 does not fit the single-pass kernel and must fall back with equal results."""
+    g = torch.Generator().manual_seed(41)
+    b, t = 3, 6
+    rows_t = t + 1 if drop_last else t
+    logits = (torch.randn(b, rows_t, vocab, generator=g) * 2.0).to(dtype)
+    labels = torch.randint(0, vocab, (b, t), generator=g)
+    adv = torch.randn(b, t, generator=g)
+    mask = torch.rand(b, t, generator=g) > 0.3
+    mask[1] = False  # a row without response tokens
+    rho = torch.rand(b, t, generator=g) + 0.5
+    cfg = make_grpo_config(loss_fn=loss_fn, beta=0.05, kl_estimator=2, clip_higher=0.28)
+    temperature = 0.9
+    # oracle chain in fp32 on the same (rounded) logits
+    ref_in = logits.float().clone().requires_grad_(True)
+    z = ref_in[:, :-1] if drop_last else ref_in
+    lp_o = o_logprob.log_softmax_and_gather(z, labels, None, temperature)
+    ent_o = o_logprob.entropy_from_logits(z.detach(), None, temperature)
+    old = lp_o.detach() + 0.05 * torch.randn(b, t, generator=g) if with_old else None
+    ref = lp_o.detach() + 0.1 * torch.randn(b, t, generator=g) if with_ref else None
+    loss_o, *_ = o_grpo.grpo_token_loss(
+        lp_o, old if with_old else lp_o.detach(), ref, adv, mask.float(), cfg, rho_weights=rho,
+        loss_denominator=denominator, axis=axis, dp_scale=0.5,
+    )  # fmt: skip
+    # rows without tokens give NaN gradients in the reference formulation (0 * 1/0); the kernels define 0
+    torch.nan_to_num(loss_o, nan=0.0).backward()
+    exp_grad = torch.nan_to_num(ref_in.grad, nan=0.0)
+
+    dev = lambda x: None if x is None else x.to(DEV)  # noqa: E731
+    lg = logits.to(DEV).requires_grad_(True)
+    loss, stats, lp, ent = grpo_utils.grpo_loss_on_logits(
+        lg, dev(labels), dev(old), dev(ref), dev(adv), dev(mask), cfg, temperature=temperature, rho_weights=dev(rho),
+        loss_denominator=denominator, axis=axis, dp_scale=0.5, drop_last=drop_last,
+    )  # fmt: skip
+    loss.backward()
+    tol = 1e-5 if dtype == torch.float32 else 2e-3
+    assert not lp.requires_grad and lp.shape == (b, t)
+    assert (lp.cpu() - lp_o.detach()).abs().max().item() <= tol
+    assert (ent.cpu() - ent_o).abs().max().item() <= tol
+    if axis is None:  # with axis=1 the reference value itself is NaN-free only without empty rows
+        assert abs(loss.item() - loss_o.item()) <= tol
+    assert lg.grad.dtype == dtype and lg.grad.shape == logits.shape
+    assert (lg.grad.float().cpu() - exp_grad).abs().max().item() <= tol
+    if drop_last:
+        assert (lg.grad[:, -1] == 0).all()
+    # the two-pass kernels give the same numbers
+    lg2 = logits.to(DEV).requires_grad_(True)
+    lp2, ent2 = model_utils.logprob_and_entropy(lg2, dev(labels), temperature=temperature, drop_last=drop_last)
+    loss2, stats2 = grpo_utils.grpo_loss_fused(
+        lp2, dev(old), dev(ref), dev(adv), dev(mask), cfg, rho_weights=dev(rho), entropy=ent2,
+        loss_denominator=denominator, axis=axis, dp_scale=0.5,
+    )  # fmt: skip
+    loss2.backward()
+    # another workgroup size, another merge order of the per-lane statistics: last-bit differences
+    assert (lp - lp2.detach()).abs().max().item() <= 4e-6 and (ent - ent2).abs().max().item() <= 4e-6
+    assert abs(loss.item() - loss2.item()) <= 4e-6 * max(1.0, abs(loss2.item()))
+    for k in stats2:
+        assert abs(stats[k].item() - stats2[k].item()) <= 4e-6 * max(1.0, abs(stats2[k].item())), k
+    step = 2.0**-7 if dtype != torch.float32 else 1e-5
+    assert (lg.grad.float() - lg2.grad.float()).abs().max().item() <= step * max(1e-3, lg2.grad.float().abs().max().item())
+    # an upstream gradient other than 1 scales the stored gradient
+    lg3 = logits.to(DEV).requires_grad_(True)
+    loss3, *_ = grpo_utils.grpo_loss_on_logits(
+        lg3, dev(labels), dev(old), dev(ref), dev(adv), dev(mask), cfg, temperature=temperature, rho_weights=dev(rho),
+        loss_denominator=denominator, axis=axis, dp_scale=0.5, drop_last=drop_last,
+    )  # fmt: skip
+    (loss3 * 2.0).backward()
+    assert (lg3.grad.float() - 2.0 * lg.grad.float()).abs().max().item() <= 2.0 * step * max(1e-3, lg.grad.float().abs().max().item())
+
+
+def test_grpo_loss_on_logits_full_vocabulary_rows():
+    """Llama-3 vocabulary (128256, bf16), 300 rows: the single-launch path against the two-pass
+    kernels on the device (the CPU oracle covers small shapes above)."""
+    torch.manual_seed(42)
+    b, t, vocab = 3, 100, 128256
+    logits = (torch.randn(b, t, vocab, device=DEV) * 3.0).bfloat16()
+    labels = torch.randint(0, vocab, (b, t), device=DEV)
+    adv = torch.randn(b, t, device=DEV)
+    mask = torch.rand(b, t, device=DEV) > 0.2
+    cfg = make_grpo_config(loss_fn="dapo", beta=0.05, kl_estimator=2, clip_higher=0.28)
+    with torch.no_grad():
+        lp0 = model_utils.log_softmax_and_gather(logits, labels)
+    old, ref = lp0 + 0.05 * torch.randn_like(lp0), lp0 + 0.1 * torch.randn_like(lp0)
+    a = logits.clone().requires_grad_(True)
+    loss_a, stats_a, lp_a, ent_a = grpo_utils.grpo_loss_on_logits(a, labels, old, ref, adv, mask, cfg)
+    loss_a.backward()
+    c = logits.clone().requires_grad_(True)
+    lp_c, ent_c = model_utils.logprob_and_entropy(c, labels)
+    loss_c, stats_c = grpo_utils.grpo_loss_fused(lp_c, old, ref, adv, mask, cfg, entropy=ent_c)
+    loss_c.backward()
+    assert (lp_a - lp_c.detach()).abs().max().item() <= 1e-5 and (ent_a - ent_c).abs().max().item() <= 1e-5
+    assert abs(loss_a.item() - loss_c.item()) <= 1e-6 + 1e-5 * abs(loss_c.item())
+    ga, gc = a.grad.float(), c.grad.float()
+    assert (ga - gc).abs().max().item() <= 2.0**-7 * gc.abs().max().item()
+    assert (ga[~mask] == 0).all()
+    # every gradient row sums to ~0 and the statistics agree
+    assert ga.sum(-1).abs().max().item() <= 0.05 * ga.abs().max().item() * 8
+    for k in stats_c:
+        assert abs(stats_a[k].item() - stats_c[k].item()) <= 1e-5 * max(1.0, abs(stats_c[k].item())), k
