@@ -9,6 +9,7 @@ C-ABI in ``include/oi_kernels.h``; there is no CPU or eager-PyTorch fallback.
 
 from . import (  # noqa: F401
     _lib,
+    data_loader,
     data_types,
     dpo_utils,
     grpo_utils,

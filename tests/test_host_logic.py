@@ -156,3 +156,41 @@ def test_tensor_cache_roundtrip_and_reference_cache_builder(tmp_path):
     assert len(calls) == n_calls and torch.equal(loaded.tensors["chosen_logps"], built.tensors["chosen_logps"])
     with pytest.raises(RuntimeError, match="Missing 1 indices"):
         dpo_utils.build_reference_logprobs_cache(model, batches[:2], False, forward_fn, 5, torch.device("cpu"))
+
+
+def test_collation_of_packed_rows_for_workers():
+    """open_instruct/data_loader.py:636-641,1205-1289: rank split, per-rank shuffle from numpy's
+    global generator, right padding (pad id for tokens, 0 elsewhere), uneven tails dropped."""
+    import numpy as np
+
+    from open_instruct_amd import data_loader
+    from open_instruct_amd.rl_utils import PackedSequences
+
+    lens = [5, 3, 7, 2, 4]
+    rows = lambda fill, dtype: [torch.full((n,), fill(k), dtype=dtype) for k, n in enumerate(lens)]  # noqa: E731
+    packed = PackedSequences(
+        query_responses=rows(lambda k: 10 + k, torch.long), attention_masks=rows(lambda k: 1, torch.long),
+        response_masks=rows(lambda k: k + 1, torch.long), original_responses=[],
+        advantages=rows(lambda k: 0.5 * k, torch.float32), position_ids=[torch.arange(n) for n in lens],
+        vllm_logprobs=rows(lambda k: -1.0 * k, torch.float32),
+    )  # fmt: skip
+    np.random.seed(3)
+    got = data_loader.prepare_collated_data_for_workers(packed, 2, 2, pad_token_id=99)
+    np.random.seed(3)
+    orders = [np.random.permutation(2), np.random.permutation(2)]
+    assert len(got) == 2 and all(len(c) == 1 for c in got)  # 5 rows -> 4 kept, 2 per rank, one micro-batch each
+    for rank, (coll, order) in enumerate(zip(got, orders)):
+        src = [2 * rank + int(i) for i in order]
+        qr = coll.query_responses[0]
+        width = max(lens[i] for i in src)
+        assert qr.shape == (2, width)
+        for r, i in enumerate(src):
+            assert qr[r, : lens[i]].tolist() == [10 + i] * lens[i] and qr[r, lens[i] :].tolist() == [99] * (width - lens[i])
+            assert coll.attention_masks[0][r].tolist() == [1] * lens[i] + [0] * (width - lens[i])
+            assert coll.position_ids[0][r, : lens[i]].tolist() == list(range(lens[i]))
+            assert coll.response_masks[0][r].tolist() == [i + 1] * lens[i] + [0] * (width - lens[i])
+            assert coll.advantages[0][r, : lens[i]].tolist() == [0.5 * i] * lens[i]
+            assert coll.vllm_logprobs[0][r, lens[i] :].tolist() == [0.0] * (width - lens[i])
+    single = data_loader.prepare_collated_data_for_workers(packed, 1, 1, pad_token_id=0)
+    assert len(single) == 1 and len(single[0]) == 5 and all(t.shape[0] == 1 for t in single[0].query_responses)
+    assert data_loader.collate_fn([torch.tensor([1, 2, 3])], 0).shape == (1, 3)
