@@ -505,6 +505,41 @@ __global__ void __launch_bounds__(NTHREADS)
     const int64_t m0 = tm * BM, n0 = tn * BN;
     AccTile acc;
     gemm_tile(acc, A, lda, m0, M, B, ldb, n0, N, K, lds);
+    if (mode >= 2 && (ldo & 1) == 0) {
+        // bf16 output: neighbouring lanes hold neighbouring columns of the same rows; after one DPP
+        // swap per pair of rows every lane stores two columns of one row as a 4-byte word (half as
+        // many, twice as wide stores as one bf16 per lane)
+        const bool odd = lane & 1;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int64_t col = n0 + (acc_col(wn, j, lane) & ~1);
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const float own0 = acc[i][j][2 * t], own1 = acc[i][j][2 * t + 1];
+                    const float send = odd ? own0 : own1;
+                    const float recv = __int_as_float(
+                        __builtin_amdgcn_mov_dpp(__float_as_int(send), 0xB1 /* quad_perm 1,0,3,2 */, 0xF, 0xF, true));
+                    float lo = odd ? recv : own0, hi = odd ? own1 : recv;
+                    const int64_t row = m0 + acc_row(wm, i, 2 * t, lane) + (odd ? 1 : 0);
+                    if (row >= m_valid || col >= N) continue;
+                    const int64_t o = row * ldo + col;
+                    if (col + 1 < N) {
+                        if (mode == 3) {
+                            const float2 part = *reinterpret_cast<const float2*>(out_f32 + o);
+                            lo += part.x;
+                            hi += part.y;
+                        }
+                        *reinterpret_cast<uint32_t*>(out_bf16 + o) = oi_pack_bf16x2(lo, hi);
+                    } else {
+                        if (mode == 3) lo += out_f32[o];
+                        out_bf16[o] = (uint16_t)oi_f32_to_bf16_bits(lo);
+                    }
+                }
+            }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
