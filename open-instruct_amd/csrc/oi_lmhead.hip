@@ -13,9 +13,9 @@
 // Tile: 256 x 256 x 64 per 512-thread workgroup, 8 waves as 4 (m) x 2 (n), each wave 64 x 128 =
 // 2 x 4 MFMA 32x32x16 accumulators.  With vocabulary as the m dim a lane's 16 accumulator
 // registers of one MFMA tile belong to ONE token (column), so the softmax statistics reduce
-// inside the lane.  LDS: two 64 KB stages of (A + B) k-tiles filled by direct global->LDS loads of
-// whole 128-byte row segments; rows are unpadded and their 16-byte chunks XOR-permuted so that
-// fragment reads stay free of bank conflicts.
+// inside the lane.  LDS: a ring of five 32 KB operand slots (k-tiles of A and of B) filled by
+// direct global->LDS loads of whole 128-byte row segments; rows are unpadded and their 16-byte
+// chunks XOR-permuted so that fragment reads stay free of bank conflicts.
 #include "oi_common.h"
 
 namespace {
@@ -25,12 +25,10 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int NTHREADS = 512;
-constexpr int NSTAGE = 2;                       // LDS ring: one k-tile being read, one in flight
 constexpr int TILE_ELEMS = BM * BK;             // one operand tile in LDS, rows of 128 B, unpadded
-constexpr int STAGE_ELEMS = 2 * TILE_ELEMS;     // A + B = 64 KB
 constexpr int STAGE_STRIDE = 256 + 8;           // bf16 per row of the dZ staging tile
-constexpr int LDS_ELEMS = 256 * STAGE_STRIDE;   // 135168 B: covers the ring (131072 B) and the dZ staging tile
-static_assert(NSTAGE * STAGE_ELEMS <= LDS_ELEMS, "the main-loop ring must fit");
+constexpr int LDS_ELEMS = 5 * TILE_ELEMS;       // 163840 B: the five-slot operand ring, all of a CU's LDS
+static_assert(256 * STAGE_STRIDE <= LDS_ELEMS, "the dZ staging tile must fit");
 
 typedef f32x16 AccTile[2][4];
 
@@ -80,17 +78,25 @@ __device__ __forceinline__ void wait_loads_and_barrier() {
 //
 // Operand tiles reach the LDS by direct global->LDS loads (no VGPR staging, no LDS store
 // instructions).  Eight consecutive lanes fetch the eight 16-byte chunks of one 128-byte row
-// segment: whole cache lines per row move about 1.7x faster from L2 than half lines do, and at
-// half lines the load path, not the matrix pipe, sets the pace of a 256 x 256 tile.  Two stages of
-// 64 KB: while k-tile t is multiplied the loads of t+1 are outstanding.
-// Wave w owns rows [32 w, 32 w + 32) of both operand tiles: 8 loads of 1 KB per k-tile.
-constexpr int LOADS_PER_STAGE = 8;
+// segment, i.e. whole cache lines.  The path from L2 into the LDS delivers a 64 KB k-tile to a CU
+// in about the time the matrix pipe needs to multiply it, so the loads must be in flight all the
+// time: issued in one burst per k-tile they back up in the load unit and hold the issuing waves
+// (and their MFMAs) for twice the MFMA time of that k-step.  Spreading them needs a free
+// destination throughout the k-tile, which two full stages cannot give (the stage being read is
+// the only candidate), hence a ring of FIVE operand slots of 32 KB, all of a CU's 160 KB:
+// k-tile t reads A_t and B_t from two slots, A_(t+1) and B_(t+1) are landing in two more,
+// A_(t+2) goes into the fifth at any time, and B_(t+2) takes A_t's slot once the barrier near the
+// end of k-tile t has passed.
+// Wave w owns rows [32 w, 32 w + 32) of both operand tiles: 4 + 4 loads of 1 KB per k-tile.
+constexpr int NSLOT = 5;
 constexpr int64_t MAX_LD = (int64_t)1 << 22;  // 255 rows * ld * 2 bytes must fit 32 bits
+__device__ __forceinline__ int ring_slot(int s) { return s >= NSLOT ? s - NSLOT : s; }
 __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restrict__ A, int64_t lda, int64_t m0,
                                           int64_t M, const uint16_t* __restrict__ B, int64_t ldb, int64_t n0,
                                           int64_t N, int64_t K, uint16_t* lds) {
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    // the wave index as a scalar: the LDS destinations of the loads (M0) then take no VALU work
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave & 3, wn = wave >> 2;
 
 #pragma unroll
@@ -101,7 +107,8 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     // loader side: lane -> (row, stored chunk) inside a block of 8 rows.  Addresses are a uniform
-    // 64-bit tile base plus a 32-bit byte offset per lane (rows of a tile span < 4 GB).
+    // 64-bit base (tile origin + k offset) plus a 32-bit byte offset per lane (rows of a tile span
+    // < 4 GB).
     const char* a_tile = reinterpret_cast<const char*>(A + m0 * lda);
     const char* b_tile = reinterpret_cast<const char*>(B + n0 * ldb);
     const int a_last = (int)((M - 1 - m0) < 255 ? (M - 1 - m0) : 255);
@@ -116,106 +123,112 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
     }
     uint16_t* my_rows = lds + wave * 32 * BK;
     const int64_t ktiles = K / BK;
-    // k-tiles past the end re-read the last one into a stage nobody reads any more: the loop body
-    // stays free of branches, which lets the scheduler interleave loads, LDS reads and MFMAs
-    auto issue = [&](int64_t kt) {
-        const int64_t src = kt < ktiles ? kt : ktiles - 1;
-        const char* a_src = a_tile + src * (BK * 2);
-        const char* b_src = b_tile + src * (BK * 2);
-        uint16_t* dst = my_rows + (int)(kt & (NSTAGE - 1)) * STAGE_ELEMS;
-#pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(a_src + ao[b]), OI_LDS_PTR(dst + b * 8 * BK), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(b_src + bo[b]), OI_LDS_PTR(dst + TILE_ELEMS + b * 8 * BK), 16,
-                                             0, 0);
-        }
+    // k-tiles past the end re-read the last one into a slot nobody reads any more: the loop body
+    // stays free of branches
+    auto k_src = [&](const char* tile, int64_t kt) {
+        const uint64_t v = reinterpret_cast<uint64_t>(tile + (kt < ktiles ? kt : ktiles - 1) * (BK * 2));
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
     };
-    issue(0);
-    issue(1);
+    // one 1 KB load: 8 rows (block b of this wave's 32) of an operand k-tile into ring slot `slot`
+    auto load_rows = [&](const char* src, uint32_t off, int slot, int b) {
+        __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(src + off), OI_LDS_PTR(my_rows + slot * TILE_ELEMS + b * 8 * BK),
+                                         16, 0, 0);
+    };
+    // ring slots: A_t -> (2 t) mod 5, B_t -> (2 t + 1) mod 5
+    {
+        const char* a_k0 = k_src(a_tile, 0);
+        const char* b_k0 = k_src(b_tile, 0);
+        const char* a_k1 = k_src(a_tile, 1);
+        const char* b_k1 = k_src(b_tile, 1);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) load_rows(a_k0, ao[b], 0, b);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) load_rows(b_k0, bo[b], 1, b);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) load_rows(a_k1, ao[b], 2, b);
+#pragma unroll
+        for (int b = 0; b < 3; ++b) load_rows(b_k1, bo[b], 3, b);
+    }
 
-    // consumer side: element offsets of this lane's fragments; k-step ks flips the stored chunk by
-    // (2 ks); rows 32 apart share the same permutation
+    // consumer side: element offsets of this lane's fragments inside a slot; k-step ks flips the
+    // stored chunk by (2 ks); rows 32 apart share the same permutation
     const int lr = lane & 31, h = lane >> 5;
     const int ra = wm * 64 + lr, rb = wn * 128 + lr;
     const int pg = h ^ swz(lr);
-    const int a_base = ra * BK + pg * 8, b_base = TILE_ELEMS + rb * BK + pg * 8;
-    auto load_frags = [&](int64_t kt, int ks, bf16x8(&af)[2], bf16x8(&bf)[4]) {
-        const uint16_t* cur = lds + (int)(kt & (NSTAGE - 1)) * STAGE_ELEMS;
-        const int a_off = a_base ^ (ks * 16), b_off = b_base ^ (ks * 16);
-#pragma unroll
-        for (int i = 0; i < 2; ++i) af[i] = *reinterpret_cast<const bf16x8*>(cur + a_off + i * 32 * BK);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(cur + b_off + j * 32 * BK);
-    };
-    auto mma = [&](const bf16x8(&af)[2], const bf16x8(&bf)[4]) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
-    };
-    // 6 LDS reads spread over the 8 MFMAs of one k-step.  An MFMA goes first: its wait for the
-    // current fragments then precedes every read of the next ones (a read issued ahead of that wait
-    // would be waited for as well, a full LDS round trip with the matrix pipe idle).
-    auto interleave_reads = [&]() {
-#pragma unroll
-        for (int q = 0; q < 6; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-        __builtin_amdgcn_sched_barrier(0);
-    };
+    const int a_base = ra * BK + pg * 8, b_base = rb * BK + pg * 8;
 
-    // Software pipeline over the four k-steps of a k-tile: the fragments of the next k-step are
-    // always requested before the MFMAs of the current one are issued, and the barrier that
-    // publishes k-tile t+1 (and frees the stage of k-tile t for t+2) sits before the last MFMA batch
-    // of k-tile t, so LDS latency and the barrier are covered by MFMA work.
+    // One k-step: 8 MFMAs on (ac, bc) with the 6 fragment reads of the following k-step (from slots
+    // sa_n / sb_n at k-step ks_n) and this k-step's share of the global->LDS loads placed between
+    // them one by one.  Nothing may move across the scheduling barriers: loads issued back to back
+    // hold up the wave's MFMA issue, and a fragment read issued ahead of the first MFMA would be
+    // waited for together with the current fragments (a full LDS round trip with the matrix pipe
+    // idle).
     bf16x8 a0[2], b0[4], a1[2], b1[4];
-    wait_loads_and_barrier<LOADS_PER_STAGE>();
-    load_frags(0, 0, a0, b0);
+#define OI_KSTEP(ac, bc, an, bn, sa_n, sb_n, ks_n, LOADS_AT)                                                     \
+    {                                                                                                            \
+        const uint16_t* pa = lds + (sa_n) * TILE_ELEMS + (a_base ^ ((ks_n) * 16));                               \
+        const uint16_t* pb = lds + (sb_n) * TILE_ELEMS + (b_base ^ ((ks_n) * 16));                               \
+        _Pragma("unroll") for (int q = 0; q < 8; ++q) {                                                          \
+            acc[q >> 2][q & 3] =                                                                                 \
+                __builtin_amdgcn_mfma_f32_32x32x16_bf16(ac[q >> 2], bc[q & 3], acc[q >> 2][q & 3], 0, 0, 0);     \
+            __builtin_amdgcn_sched_barrier(0);                                                                   \
+            LOADS_AT(q)                                                                                          \
+            if (q < 2) an[q] = *reinterpret_cast<const bf16x8*>(pa + q * 32 * BK);                               \
+            else if (q < 6) bn[q - 2] = *reinterpret_cast<const bf16x8*>(pb + (q - 2) * 32 * BK);                \
+            __builtin_amdgcn_sched_barrier(0);                                                                   \
+        }                                                                                                        \
+    }
+    // the 8 loads of a k-tile iteration, as evenly spread as the slot hand-over allows
+#define OI_LOADS_KS0(q)                               \
+    if (q == 1) load_rows(b_n1, bo[3], s_b1, 3);      \
+    if (q == 5) load_rows(a_n2, ao[0], s_a2, 0);
+#define OI_LOADS_KS1(q) \
+    if (q == 3) load_rows(a_n2, ao[1], s_a2, 1);
+#define OI_LOADS_KS2(q)                               \
+    if (q == 1) load_rows(a_n2, ao[2], s_a2, 2);      \
+    if (q == 5) load_rows(a_n2, ao[3], s_a2, 3);
+#define OI_LOADS_KS3(q)                               \
+    if (q == 0) load_rows(b_n2, bo[0], s_a, 0);       \
+    if (q == 3) load_rows(b_n2, bo[1], s_a, 1);       \
+    if (q == 6) load_rows(b_n2, bo[2], s_a, 2);
+
+    // A_0, B_0 landed (7 younger loads may still be in flight)
+    wait_loads_and_barrier<7>();
+    {
+        const uint16_t* pa = lds + a_base;
+        const uint16_t* pb = lds + TILE_ELEMS + b_base;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) a0[i] = *reinterpret_cast<const bf16x8*>(pa + i * 32 * BK);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b0[j] = *reinterpret_cast<const bf16x8*>(pb + j * 32 * BK);
+    }
+    int sa = 0;  // slot of A_kt
     for (int64_t kt = 0; kt < ktiles; ++kt) {
-        load_frags(kt, 1, a1, b1);
-        mma(a0, b0);
-        interleave_reads();
-        load_frags(kt, 2, a0, b0);
-        mma(a1, b1);
-        interleave_reads();
-        load_frags(kt, 3, a1, b1);
-        mma(a0, b0);
-        interleave_reads();
-        // k-tile kt+1 must have landed and this wave's last reads of k-tile kt must be complete:
-        // after the barrier the stage of k-tile kt is overwritten with k-tile kt+2
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        const int s_a = sa, s_b = ring_slot(sa + 1);                   // being read
+        const int s_a1 = ring_slot(sa + 2), s_b1 = ring_slot(sa + 3);  // k-tile kt+1
+        const int s_a2 = ring_slot(sa + 4);                            // free all along: takes A_(kt+2)
+        const char* b_n1 = k_src(b_tile, kt + 1);
+        const char* a_n2 = k_src(a_tile, kt + 2);
+        const char* b_n2 = k_src(b_tile, kt + 2);
+        OI_KSTEP(a0, b0, a1, b1, s_a, s_b, 1, OI_LOADS_KS0)
+        OI_KSTEP(a1, b1, a0, b0, s_a, s_b, 2, OI_LOADS_KS1)
+        OI_KSTEP(a0, b0, a1, b1, s_a, s_b, 3, OI_LOADS_KS2)
+        // k-tile kt+1 must have landed (its last load was issued in the first k-step above; the
+        // four younger ones may stay in flight) and this wave's reads of k-tile kt must be
+        // complete: after the barrier A_kt's slot is overwritten with B_(kt+2)
+        asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        // last k-step of the k-tile: 8 MFMAs with the 8 global->LDS loads of k-tile kt+2 and the 6
-        // fragment reads of k-tile kt+1 placed between them one by one (nothing may move across the
-        // scheduling barriers: loads issued back to back would hold up the wave's MFMA issue)
-        {
-            const int64_t nkt = kt + NSTAGE;
-            const int64_t src = nkt < ktiles ? nkt : ktiles - 1;
-            const char* a_src = a_tile + src * (BK * 2);
-            const char* b_src = b_tile + src * (BK * 2);
-            uint16_t* dst = my_rows + (int)(nkt & (NSTAGE - 1)) * STAGE_ELEMS;
-            const uint16_t* nxt = lds + (int)((kt + 1) & (NSTAGE - 1)) * STAGE_ELEMS;
-#pragma unroll
-            for (int q = 0; q < 8; ++q) {
-                acc[q >> 2][q & 3] =
-                    __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1[q >> 2], b1[q & 3], acc[q >> 2][q & 3], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-                if (q & 1)
-                    __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(b_src + bo[q >> 1]),
-                                                     OI_LDS_PTR(dst + TILE_ELEMS + (q >> 1) * 8 * BK), 16, 0, 0);
-                else
-                    __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(a_src + ao[q >> 1]), OI_LDS_PTR(dst + (q >> 1) * 8 * BK),
-                                                     16, 0, 0);
-                if (q < 2) a0[q] = *reinterpret_cast<const bf16x8*>(nxt + a_base + q * 32 * BK);
-                else if (q < 6) b0[q - 2] = *reinterpret_cast<const bf16x8*>(nxt + b_base + (q - 2) * 32 * BK);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
+        OI_KSTEP(a1, b1, a0, b0, s_a1, s_b1, 0, OI_LOADS_KS3)
+        sa = s_a1;
     }
+#undef OI_KSTEP
+#undef OI_LOADS_KS0
+#undef OI_LOADS_KS1
+#undef OI_LOADS_KS2
+#undef OI_LOADS_KS3
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // every wave is done reading before the caller reuses the LDS (epilogue staging, next tile)
     __builtin_amdgcn_s_barrier();
