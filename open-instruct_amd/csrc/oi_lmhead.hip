@@ -253,26 +253,43 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
 #pragma unroll
         for (int j = 0; j < 4; ++j) b0[j] = *reinterpret_cast<const bf16x8*>(pb + j * 32 * BK);
     }
-    int sa = 0;  // slot of A_kt
-    for (int64_t kt = 0; kt < ktiles; ++kt) {
-        const int s_a = sa, s_b = ring_slot(sa + 1);                   // being read
-        const int s_a1 = ring_slot(sa + 2), s_b1 = ring_slot(sa + 3);  // k-tile kt+1
-        const int s_a2 = ring_slot(sa + 4);                            // free all along: takes A_(kt+2)
-        const char* b_n1 = k_src(b_tile, kt + 1);
-        const char* a_n2 = k_src(a_tile, kt + 2);
-        const char* b_n2 = k_src(b_tile, kt + 2);
-        OI_KSTEP(a0, b0, a1, b1, s_a, s_b, 1, OI_LOADS_KS0)
-        OI_KSTEP(a1, b1, a0, b0, s_a, s_b, 2, OI_LOADS_KS1)
-        OI_KSTEP(a0, b0, a1, b1, s_a, s_b, 3, OI_LOADS_KS2)
-        // k-tile kt+1 must have landed (its last load was issued in the first k-step above; the
-        // four younger ones may stay in flight) and this wave's reads of k-tile kt must be
-        // complete: after the barrier A_kt's slot is overwritten with B_(kt+2)
-        asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        OI_KSTEP(a1, b1, a0, b0, s_a1, s_b1, 0, OI_LOADS_KS3)
-        sa = s_a1;
+    // One k-tile iteration.  The last two iterations have no later k-tiles to fetch: they run
+    // without those loads (no wasted traffic, nothing to drain before the epilogue).
+#define OI_KTILE(L0, L1, L2, L3, PENDING)                                                                       \
+    {                                                                                                            \
+        const int s_a = sa, s_b = ring_slot(sa + 1);                  /* being read */                          \
+        const int s_a1 = ring_slot(sa + 2), s_b1 = ring_slot(sa + 3); /* k-tile kt+1 */                         \
+        const int s_a2 = ring_slot(sa + 4);                           /* free all along: takes A_(kt+2) */      \
+        const char* b_n1 = k_src(b_tile, kt + 1);                                                                \
+        const char* a_n2 = k_src(a_tile, kt + 2);                                                                \
+        const char* b_n2 = k_src(b_tile, kt + 2);                                                                \
+        (void)s_a2; (void)s_b1; (void)b_n1; (void)a_n2; (void)b_n2;                                              \
+        OI_KSTEP(a0, b0, a1, b1, s_a, s_b, 1, L0)                                                                \
+        OI_KSTEP(a1, b1, a0, b0, s_a, s_b, 2, L1)                                                                \
+        OI_KSTEP(a0, b0, a1, b1, s_a, s_b, 3, L2)                                                                \
+        /* k-tile kt+1 must have landed (its last load was issued in the first k-step above; the  */            \
+        /* PENDING younger ones may stay in flight) and this wave's reads of k-tile kt must be     */            \
+        /* complete: after the barrier A_kt's slot is overwritten with B_(kt+2)                    */            \
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(PENDING) : "memory");                                \
+        __builtin_amdgcn_s_barrier();                                                                            \
+        asm volatile("" ::: "memory");                                                                           \
+        OI_KSTEP(a1, b1, a0, b0, s_a1, s_b1, 0, L3)                                                              \
+        sa = s_a1;                                                                                               \
     }
+#define OI_LOADS_NONE(q)
+#define OI_LOADS_KS0_ONLY_B(q) \
+    if (q == 1) load_rows(b_n1, bo[3], s_b1, 3);
+    int sa = 0;  // slot of A_kt
+    int64_t kt = 0;
+    for (; kt + 2 < ktiles; ++kt) OI_KTILE(OI_LOADS_KS0, OI_LOADS_KS1, OI_LOADS_KS2, OI_LOADS_KS3, 4)
+    if (kt + 1 < ktiles) {
+        OI_KTILE(OI_LOADS_KS0_ONLY_B, OI_LOADS_NONE, OI_LOADS_NONE, OI_LOADS_NONE, 0)
+        ++kt;
+    }
+    OI_KTILE(OI_LOADS_NONE, OI_LOADS_NONE, OI_LOADS_NONE, OI_LOADS_NONE, 0)
+#undef OI_KTILE
+#undef OI_LOADS_NONE
+#undef OI_LOADS_KS0_ONLY_B
 #undef OI_KSTEP
 #undef OI_LOADS_KS0
 #undef OI_LOADS_KS1
