@@ -18,6 +18,8 @@
 // chunks XOR-permuted so that fragment reads stay free of bank conflicts.
 #include "oi_common.h"
 
+#include <type_traits>
+
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -138,9 +140,47 @@ __device__ __forceinline__ void wait_loads_and_barrier() {
 constexpr int NSLOT = 5;
 constexpr int64_t MAX_LD = (int64_t)1 << 22;  // 255 rows * ld * 2 bytes must fit 32 bits
 __device__ __forceinline__ int ring_slot(int s) { return s >= NSLOT ? s - NSLOT : s; }
-__device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restrict__ A, int64_t lda, int64_t m0,
-                                          int64_t M, const uint16_t* __restrict__ B, int64_t ldb, int64_t n0,
-                                          int64_t N, int64_t K, uint16_t* lds) {
+
+// One operand of a tile product, in either of two memory layouts.
+//   k-contiguous (KM = false): element (row, k) at p[row * ld + k]; the tile takes rows
+//     [r0, r0 + 256), rows at or past `extent` are clamped onto the last valid one.
+//   k-major (KM = true): element (row, k) at p[k * ld + row]; the tile takes columns
+//     [r0, r0 + 256) of every k row, 16-byte column chunks past `extent` (a multiple of 8) are
+//     clamped onto the last valid chunk, k rows at or past `k_valid` onto the last valid row (the
+//     other operand must hold zeros there).  This is the layout in which a matrix is its own
+//     transpose operand: W [V, H] as the B operand of dZ * W, hidden [N, H] and dZ [N, V] as the
+//     operands of dZ^T * hidden, with no transposed copies in memory.
+// In both cases the results of clamped rows / columns are garbage that the epilogues discard.
+struct Operand {
+    const uint16_t* p;
+    int64_t ld, r0, extent, k_valid;
+};
+
+typedef short v4i16 __attribute__((ext_vector_type(4)));
+
+// acc = A_tile * B_tile^T over k in [0, K), K a multiple of 64.
+//
+// Operand tiles reach the LDS by direct global->LDS loads (no VGPR staging, no LDS store
+// instructions), whole 128-byte cache-line segments per 8 lanes.  The path from L2 into the LDS
+// delivers a 64 KB k-tile to a CU in about the time the matrix pipe needs to multiply it, so the
+// loads must be in flight all the time: issued in one burst per k-tile they back up in the load
+// unit and hold the issuing waves (and their MFMAs) for twice the MFMA time of that k-step.
+// Spreading them needs a free destination throughout the k-tile, which two full stages cannot give
+// (the stage being read is the only candidate), hence a ring of FIVE operand slots of 32 KB, all
+// of a CU's 160 KB: k-tile t reads A_t and B_t from two slots, A_(t+1) and B_(t+1) are landing in
+// two more, A_(t+2) goes into the fifth at any time, and B_(t+2) takes A_t's slot once the barrier
+// near the end of k-tile t has passed.  Every wave issues 4 + 4 loads of 1 KB per k-tile.
+//
+// LDS image of a k-contiguous operand tile: [256 rows][64 k], the eight 16-byte chunks of a row
+// stored at c ^ swz(row); wave w loads rows [32 w, 32 w + 32); fragments are 16-byte reads.
+// LDS image of a k-major operand tile: [64 k][256 columns], the 32 chunks of a k row stored at
+// c ^ 4 (k & 3); wave w loads k rows [8 w, 8 w + 8); fragments come through the transposing read
+// ds_read_b64_tr_b16: in a group of 16 lanes, lane s points at (k0 + s / 4, 4 columns from
+// 4 (s % 4)) and lane i receives column i at k0 .. k0 + 3, which is the MFMA operand layout (row
+// per lane, consecutive k per register).  The permutation puts the four k rows of such a read on
+// different banks.
+template <bool A_KM, bool B_KM>
+__device__ __forceinline__ void gemm_tile(AccTile& acc, const Operand& A, const Operand& B, int64_t K, uint16_t* lds) {
     const int tid = opaque_tid();
     // the wave index as a scalar: the LDS destinations of the loads (M0) then take no VALU work
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -153,58 +193,118 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // loader side: lane -> (row, stored chunk) inside a block of 8 rows.  Addresses are a uniform
-    // 64-bit base (tile origin + k offset) plus a 32-bit byte offset per lane (rows of a tile span
-    // < 4 GB).
-    const char* a_tile = reinterpret_cast<const char*>(A + m0 * lda);
-    const char* b_tile = reinterpret_cast<const char*>(B + n0 * ldb);
-    const int a_last = (int)((M - 1 - m0) < 255 ? (M - 1 - m0) : 255);
-    const int b_last = (int)((N - 1 - n0) < 255 ? (N - 1 - n0) : 255);
-    uint32_t ao[4], bo[4];
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        const int r = wave * 32 + b * 8 + (lane >> 3);
-        const int c = (lane & 7) ^ swz(r);
-        ao[b] = (uint32_t)(r < a_last ? r : a_last) * (uint32_t)(lda * 2) + c * 16;
-        bo[b] = (uint32_t)(r < b_last ? r : b_last) * (uint32_t)(ldb * 2) + c * 16;
-    }
-    uint16_t* my_rows = lds + wave * 32 * BK;
     const int64_t ktiles = K / BK;
-    // k-tiles past the end re-read the last one into a slot nobody reads any more: the loop body
-    // stays free of branches
-    auto k_src = [&](const char* tile, int64_t kt) {
-        const uint64_t v = reinterpret_cast<uint64_t>(tile + (kt < ktiles ? kt : ktiles - 1) * (BK * 2));
+    // loader side.  Addresses are a uniform 64-bit base (tile origin + k offset) plus a 32-bit byte
+    // offset per lane; for a k-major operand the lanes' offsets of the last k-tile differ (its k
+    // rows may end early), `last` holds those.
+    struct Loader {
+        const char* tile;    // origin of the tile in global memory
+        int64_t k_step;      // bytes from one k-tile to the next
+        uint32_t off[4];     // per-lane byte offsets of the four loads
+        uint32_t last[4];    // the same for the last k-tile
+        int lds_block;       // elements between the LDS destinations of consecutive loads
+        int lds_wave;        // element offset of this wave's first load inside a slot
+    };
+    auto make_loader = [&](const Operand& op, auto km_tag) {
+        constexpr bool KM = decltype(km_tag)::value;
+        Loader L;
+        if constexpr (!KM) {
+            L.tile = reinterpret_cast<const char*>(op.p + op.r0 * op.ld);
+            L.k_step = BK * 2;
+            const int last_row = (int)((op.extent - 1 - op.r0) < 255 ? (op.extent - 1 - op.r0) : 255);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int r = wave * 32 + b * 8 + (lane >> 3);
+                const int c = (lane & 7) ^ swz(r);
+                L.off[b] = (uint32_t)(r < last_row ? r : last_row) * (uint32_t)(op.ld * 2) + c * 16;
+                L.last[b] = L.off[b];
+            }
+            L.lds_block = 8 * BK;
+            L.lds_wave = wave * 32 * BK;
+        } else {
+            L.tile = reinterpret_cast<const char*>(op.p);
+            L.k_step = BK * op.ld * 2;
+            const int last_k = (int)(op.k_valid - 1 - (ktiles - 1) * BK);  // inside the last k-tile
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int kk = wave * 8 + b * 2 + (lane >> 5);
+                const int c = (lane & 31) ^ (4 * (kk & 3));
+                int64_t col = op.r0 + c * 8;
+                col = col + 8 <= op.extent ? col : op.extent - 8;
+                L.off[b] = (uint32_t)kk * (uint32_t)(op.ld * 2) + (uint32_t)(col * 2);
+                L.last[b] = (uint32_t)(kk < last_k ? kk : last_k) * (uint32_t)(op.ld * 2) + (uint32_t)(col * 2);
+            }
+            L.lds_block = 2 * 256;
+            L.lds_wave = wave * 8 * 256;
+        }
+        return L;
+    };
+    const Loader la = make_loader(A, std::integral_constant<bool, A_KM>{});
+    const Loader lb = make_loader(B, std::integral_constant<bool, B_KM>{});
+    // k-tiles past the end are never requested by the loop below; the prologue may ask for k-tile 1
+    // of a one-k-tile product and then re-reads k-tile 0 into a slot nobody reads
+    auto k_src = [&](const Loader& L, int64_t kt) {
+        const uint64_t v = reinterpret_cast<uint64_t>(L.tile + (kt < ktiles ? kt : ktiles - 1) * L.k_step);
         const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
         const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
         return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
     };
-    // one 1 KB load: 8 rows (block b of this wave's 32) of an operand k-tile into ring slot `slot`
-    auto load_rows = [&](const char* src, uint32_t off, int slot, int b) {
-        __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(src + off), OI_LDS_PTR(my_rows + slot * TILE_ELEMS + b * 8 * BK),
-                                         16, 0, 0);
+    // one 1 KB load: block b of this wave's share of an operand k-tile into ring slot `slot`
+    auto load_block = [&](const Loader& L, const char* src, uint32_t off, int slot, int b) {
+        __builtin_amdgcn_global_load_lds(OI_GLOBAL_PTR(src + off),
+                                         OI_LDS_PTR(lds + slot * TILE_ELEMS + L.lds_wave + b * L.lds_block), 16, 0, 0);
     };
     // ring slots: A_t -> (2 t) mod 5, B_t -> (2 t + 1) mod 5
     {
-        const char* a_k0 = k_src(a_tile, 0);
-        const char* b_k0 = k_src(b_tile, 0);
-        const char* a_k1 = k_src(a_tile, 1);
-        const char* b_k1 = k_src(b_tile, 1);
+        const char* a_k0 = k_src(la, 0);
+        const char* b_k0 = k_src(lb, 0);
+        const char* a_k1 = k_src(la, 1);
+        const char* b_k1 = k_src(lb, 1);
+        const bool t0_last = ktiles == 1, t1_last = ktiles <= 2;
 #pragma unroll
-        for (int b = 0; b < 4; ++b) load_rows(a_k0, ao[b], 0, b);
+        for (int b = 0; b < 4; ++b) load_block(la, a_k0, t0_last ? la.last[b] : la.off[b], 0, b);
 #pragma unroll
-        for (int b = 0; b < 4; ++b) load_rows(b_k0, bo[b], 1, b);
+        for (int b = 0; b < 4; ++b) load_block(lb, b_k0, t0_last ? lb.last[b] : lb.off[b], 1, b);
 #pragma unroll
-        for (int b = 0; b < 4; ++b) load_rows(a_k1, ao[b], 2, b);
+        for (int b = 0; b < 4; ++b) load_block(la, a_k1, t1_last ? la.last[b] : la.off[b], 2, b);
 #pragma unroll
-        for (int b = 0; b < 3; ++b) load_rows(b_k1, bo[b], 3, b);
+        for (int b = 0; b < 3; ++b) load_block(lb, b_k1, t1_last ? lb.last[b] : lb.off[b], 3, b);
     }
 
-    // consumer side: element offsets of this lane's fragments inside a slot; k-step ks flips the
-    // stored chunk by (2 ks); rows 32 apart share the same permutation
+    // consumer side: element offsets of this lane's fragments inside a slot
     const int lr = lane & 31, h = lane >> 5;
-    const int ra = wm * 64 + lr, rb = wn * 128 + lr;
+    // k-contiguous image: k-step ks flips the stored chunk by (2 ks); rows 32 apart share the
+    // same permutation
     const int pg = h ^ swz(lr);
-    const int a_base = ra * BK + pg * 8, b_base = rb * BK + pg * 8;
+    const int a_base = (wm * 64 + lr) * BK + pg * 8, b_base = (wn * 128 + lr) * BK + pg * 8;
+    // k-major image: source lane s of a 16-lane group points at k row (s >> 2) of the lane's
+    // half-k-step and at 4 columns from 4 (s & 3) of the group's 16; one address per 32-row tile
+    // because the column permutation reaches the bits that select the tile
+    const int s16 = lane & 15, e4 = s16 >> 2, g16 = (lane >> 4) & 1;
+    int a_km[2], b_km[4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+        a_km[i] = (h * 8 + e4) * 256 + (((wm * 8 + i * 4 + g16 * 2 + ((s16 & 3) >> 1)) ^ (4 * e4)) * 8) + 4 * (s16 & 1);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        b_km[j] = (h * 8 + e4) * 256 + (((wn * 16 + j * 4 + g16 * 2 + ((s16 & 3) >> 1)) ^ (4 * e4)) * 8) + 4 * (s16 & 1);
+    auto read_tr = [&](const uint16_t* p) {
+        // rows k0 .. k0 + 3 and k0 + 4 .. k0 + 7 of the lane's half-k-step
+        const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) v4i16*)OI_LDS_PTR(const_cast<uint16_t*>(p)));
+        const v4i16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) v4i16*)OI_LDS_PTR(const_cast<uint16_t*>(p + 4 * 256)));
+        const short __attribute__((ext_vector_type(8))) both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(bf16x8, both);
+    };
+    auto read_a = [&](int slot, int ks, int i) {
+        if constexpr (A_KM) return read_tr(lds + slot * TILE_ELEMS + ks * 16 * 256 + a_km[i]);
+        else return *reinterpret_cast<const bf16x8*>(lds + slot * TILE_ELEMS + (a_base ^ (ks * 16)) + i * 32 * BK);
+    };
+    auto read_b = [&](int slot, int ks, int j) {
+        if constexpr (B_KM) return read_tr(lds + slot * TILE_ELEMS + ks * 16 * 256 + b_km[j]);
+        else return *reinterpret_cast<const bf16x8*>(lds + slot * TILE_ELEMS + (b_base ^ (ks * 16)) + j * 32 * BK);
+    };
 
     // One k-step: 8 MFMAs on (ac, bc) with the 6 fragment reads of the following k-step (from slots
     // sa_n / sb_n at k-step ks_n) and this k-step's share of the global->LDS loads placed between
@@ -215,44 +315,43 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
     bf16x8 a0[2], b0[4], a1[2], b1[4];
 #define OI_KSTEP(ac, bc, an, bn, sa_n, sb_n, ks_n, LOADS_AT)                                                     \
     {                                                                                                            \
-        const uint16_t* pa = lds + (sa_n) * TILE_ELEMS + (a_base ^ ((ks_n) * 16));                               \
-        const uint16_t* pb = lds + (sb_n) * TILE_ELEMS + (b_base ^ ((ks_n) * 16));                               \
         _Pragma("unroll") for (int q = 0; q < 8; ++q) {                                                          \
             acc[q >> 2][q & 3] =                                                                                 \
                 __builtin_amdgcn_mfma_f32_32x32x16_bf16(ac[q >> 2], bc[q & 3], acc[q >> 2][q & 3], 0, 0, 0);     \
             __builtin_amdgcn_sched_barrier(0);                                                                   \
             LOADS_AT(q)                                                                                          \
-            if (q < 2) an[q] = *reinterpret_cast<const bf16x8*>(pa + q * 32 * BK);                               \
-            else if (q < 6) bn[q - 2] = *reinterpret_cast<const bf16x8*>(pb + (q - 2) * 32 * BK);                \
+            if (q < 2) an[q] = read_a(sa_n, ks_n, q);                                                            \
+            else if (q < 6) bn[q - 2] = read_b(sb_n, ks_n, q - 2);                                               \
             __builtin_amdgcn_sched_barrier(0);                                                                   \
         }                                                                                                        \
     }
-    // the 8 loads of a k-tile iteration, as evenly spread as the slot hand-over allows
-#define OI_LOADS_KS0(q)                               \
-    if (q == 1) load_rows(b_n1, bo[3], s_b1, 3);      \
-    if (q == 5) load_rows(a_n2, ao[0], s_a2, 0);
+    // the 8 loads of a k-tile iteration, as evenly spread as the slot hand-over allows; OFF selects
+    // the lanes' offsets (off, or last when the k-tile being fetched is the last one)
+#define OI_LOADS_KS0(q)                                         \
+    if (q == 1) load_block(lb, b_n1, lb.off[3], s_b1, 3);       \
+    if (q == 5) load_block(la, a_n2, la.OFF2[0], s_a2, 0);
 #define OI_LOADS_KS1(q) \
-    if (q == 3) load_rows(a_n2, ao[1], s_a2, 1);
-#define OI_LOADS_KS2(q)                               \
-    if (q == 1) load_rows(a_n2, ao[2], s_a2, 2);      \
-    if (q == 5) load_rows(a_n2, ao[3], s_a2, 3);
-#define OI_LOADS_KS3(q)                               \
-    if (q == 0) load_rows(b_n2, bo[0], s_a, 0);       \
-    if (q == 3) load_rows(b_n2, bo[1], s_a, 1);       \
-    if (q == 6) load_rows(b_n2, bo[2], s_a, 2);
+    if (q == 3) load_block(la, a_n2, la.OFF2[1], s_a2, 1);
+#define OI_LOADS_KS2(q)                                         \
+    if (q == 1) load_block(la, a_n2, la.OFF2[2], s_a2, 2);      \
+    if (q == 5) load_block(la, a_n2, la.OFF2[3], s_a2, 3);
+#define OI_LOADS_KS3(q)                                         \
+    if (q == 0) load_block(lb, b_n2, lb.OFF2[0], s_a, 0);       \
+    if (q == 3) load_block(lb, b_n2, lb.OFF2[1], s_a, 1);       \
+    if (q == 6) load_block(lb, b_n2, lb.OFF2[2], s_a, 2);
+#define OI_LOADS_NONE(q)
+#define OI_LOADS_KS0_ONLY_B(q) \
+    if (q == 1) load_block(lb, b_n1, lb.last[3], s_b1, 3);
 
     // A_0 and B_0 must have landed.  The wait is for everything in flight, not for "all but the 7
     // younger loads": a workgroup that runs several tiles may still have the previous tile's
     // stores outstanding, and stores complete out of order with loads.
     wait_loads_and_barrier<0>();
-    {
-        const uint16_t* pa = lds + a_base;
-        const uint16_t* pb = lds + TILE_ELEMS + b_base;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) a0[i] = *reinterpret_cast<const bf16x8*>(pa + i * 32 * BK);
+    for (int i = 0; i < 2; ++i) a0[i] = read_a(0, 0, i);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) b0[j] = *reinterpret_cast<const bf16x8*>(pb + j * 32 * BK);
-    }
+    for (int j = 0; j < 4; ++j) b0[j] = read_b(1, 0, j);
+
     // One k-tile iteration.  The last two iterations have no later k-tiles to fetch: they run
     // without those loads (no wasted traffic, nothing to drain before the epilogue).
 #define OI_KTILE(L0, L1, L2, L3, PENDING)                                                                       \
@@ -260,9 +359,9 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
         const int s_a = sa, s_b = ring_slot(sa + 1);                  /* being read */                          \
         const int s_a1 = ring_slot(sa + 2), s_b1 = ring_slot(sa + 3); /* k-tile kt+1 */                         \
         const int s_a2 = ring_slot(sa + 4);                           /* free all along: takes A_(kt+2) */      \
-        const char* b_n1 = k_src(b_tile, kt + 1);                                                                \
-        const char* a_n2 = k_src(a_tile, kt + 2);                                                                \
-        const char* b_n2 = k_src(b_tile, kt + 2);                                                                \
+        const char* b_n1 = k_src(lb, kt + 1);                                                                    \
+        const char* a_n2 = k_src(la, kt + 2);                                                                    \
+        const char* b_n2 = k_src(lb, kt + 2);                                                                    \
         (void)s_a2; (void)s_b1; (void)b_n1; (void)a_n2; (void)b_n2;                                              \
         OI_KSTEP(a0, b0, a1, b1, s_a, s_b, 1, L0)                                                                \
         OI_KSTEP(a1, b1, a0, b0, s_a, s_b, 2, L1)                                                                \
@@ -276,29 +375,41 @@ __device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restri
         OI_KSTEP(a1, b1, a0, b0, s_a1, s_b1, 0, L3)                                                              \
         sa = s_a1;                                                                                               \
     }
-#define OI_LOADS_NONE(q)
-#define OI_LOADS_KS0_ONLY_B(q) \
-    if (q == 1) load_rows(b_n1, bo[3], s_b1, 3);
     int sa = 0;  // slot of A_kt
     int64_t kt = 0;
-    for (; kt + 2 < ktiles; ++kt) OI_KTILE(OI_LOADS_KS0, OI_LOADS_KS1, OI_LOADS_KS2, OI_LOADS_KS3, 4)
+#define OFF2 off
+    for (; kt + 3 < ktiles; ++kt) OI_KTILE(OI_LOADS_KS0, OI_LOADS_KS1, OI_LOADS_KS2, OI_LOADS_KS3, 4)
+#undef OFF2
+#define OFF2 last
+    if (kt + 2 < ktiles) {  // this iteration fetches the last k-tile
+        OI_KTILE(OI_LOADS_KS0, OI_LOADS_KS1, OI_LOADS_KS2, OI_LOADS_KS3, 4)
+        ++kt;
+    }
+#undef OFF2
     if (kt + 1 < ktiles) {
         OI_KTILE(OI_LOADS_KS0_ONLY_B, OI_LOADS_NONE, OI_LOADS_NONE, OI_LOADS_NONE, 0)
         ++kt;
     }
     OI_KTILE(OI_LOADS_NONE, OI_LOADS_NONE, OI_LOADS_NONE, OI_LOADS_NONE, 0)
 #undef OI_KTILE
-#undef OI_LOADS_NONE
-#undef OI_LOADS_KS0_ONLY_B
 #undef OI_KSTEP
 #undef OI_LOADS_KS0
 #undef OI_LOADS_KS1
 #undef OI_LOADS_KS2
 #undef OI_LOADS_KS3
+#undef OI_LOADS_NONE
+#undef OI_LOADS_KS0_ONLY_B
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // every wave is done reading before the caller reuses the LDS (epilogue staging, next tile)
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+}
+// both operands k-contiguous: C[m, n] = sum_k A[m0 + m, k] * B[n0 + n, k]
+__device__ __forceinline__ void gemm_tile(AccTile& acc, const uint16_t* __restrict__ A, int64_t lda, int64_t m0,
+                                          int64_t M, const uint16_t* __restrict__ B, int64_t ldb, int64_t n0,
+                                          int64_t N, int64_t K, uint16_t* lds) {
+    const Operand a = {A, lda, m0, M, K}, b = {B, ldb, n0, N, K};
+    gemm_tile<false, false>(acc, a, b, K, lds);
 }
 
 // Accumulator geometry of one wave: element (i, j, r) of lane `lane` is
@@ -486,8 +597,8 @@ __device__ __forceinline__ void lmhead_dz_tile(const uint16_t* __restrict__ W, c
                                                const int64_t* __restrict__ labels, const float* __restrict__ lse,
                                                const float* __restrict__ grad, int64_t n_tokens, int64_t hdim,
                                                int64_t vocab, float c, float inv_t, int64_t v_begin, int64_t chunk_cols,
-                                               int64_t n_pad, uint16_t* __restrict__ dz, uint16_t* __restrict__ dzt,
-                                               int64_t vt, int64_t tt, uint16_t* lds) {
+                                               int64_t n_pad, uint16_t* __restrict__ dz, int64_t vt, int64_t tt,
+                                               uint16_t* lds) {
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6, wm = wave & 3, wn = wave >> 2;
     const int64_t n0 = tt * BN, m0 = v_begin + vt * BM;
 
@@ -520,7 +631,6 @@ __device__ __forceinline__ void lmhead_dz_tile(const uint16_t* __restrict__ W, c
                         if (v == y) val += g;
                     }
                     d[e] = val;
-                    acc[i][j][r] = val;  // kept for the transposed copy below
                 }
                 const int vl = acc_row(wm, i, q * 4, lane);
                 uint2 pk = make_uint2(oi_pack_bf16x2(d[0], d[1]), oi_pack_bf16x2(d[2], d[3]));
@@ -537,39 +647,6 @@ __device__ __forceinline__ void lmhead_dz_tile(const uint16_t* __restrict__ W, c
         const oi_u32x4 v = *reinterpret_cast<const oi_u32x4*>(stage + row * STAGE_STRIDE + ch * 8);
         *reinterpret_cast<oi_u32x4*>(dz + (n0 + row) * chunk_cols + vcol0 + ch * 8) = v;
     }
-    // [vocab, token] order: second pass through the same LDS buffer, transposed.  Neighbouring lanes
-    // hold neighbouring tokens of the same vocabulary rows, so one DPP swap per pair of rows gives
-    // every lane two tokens of one row: 4-byte LDS writes, then the same coalesced 16-byte row copy
-    // as above (a row of the tile is 512 contiguous bytes of dZ^T).
-    if (dzt) {
-        __syncthreads();  // everyone is done reading the [token, vocab] image
-        const bool odd = lane & 1;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int nl = acc_col(wn, j, lane) & ~1;
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const float own0 = acc[i][j][2 * t], own1 = acc[i][j][2 * t + 1];
-                    const float send = odd ? own0 : own1;
-                    const float recv = __int_as_float(
-                        __builtin_amdgcn_mov_dpp(__float_as_int(send), 0xB1 /* quad_perm 1,0,3,2 */, 0xF, 0xF, true));
-                    // even lane: row 2t, tokens (nl, nl+1) = (own, neighbour); odd lane: row 2t+1
-                    const float lo = odd ? recv : own0, hi = odd ? own1 : recv;
-                    const int vl = acc_row(wm, i, 2 * t, lane) + (odd ? 1 : 0);
-                    *reinterpret_cast<uint32_t*>(stage + vl * STAGE_STRIDE + nl) = oi_pack_bf16x2(lo, hi);
-                }
-        }
-        __syncthreads();
-#pragma unroll 4
-        for (int it = 0; it < 16; ++it) {
-            const int cidx = tid + it * NTHREADS;
-            const int row = cidx >> 5, ch = cidx & 31;
-            const oi_u32x4 v = *reinterpret_cast<const oi_u32x4*>(stage + row * STAGE_STRIDE + ch * 8);
-            *reinterpret_cast<oi_u32x4*>(dzt + (vcol0 + row) * n_pad + n0 + ch * 8) = v;
-        }
-    }
 }
 
 __global__ void __launch_bounds__(NTHREADS)
@@ -577,11 +654,11 @@ __global__ void __launch_bounds__(NTHREADS)
                      const int64_t* __restrict__ labels, const float* __restrict__ lse,
                      const float* __restrict__ grad, int64_t n_tokens, int64_t hdim, int64_t vocab, float c,
                      float inv_t, int64_t v_begin, int64_t chunk_cols, int64_t n_pad, uint16_t* __restrict__ dz,
-                     uint16_t* __restrict__ dzt, uint32_t* __restrict__ queue) {
+                     uint32_t* __restrict__ queue) {
     __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
     for_each_tile(queue, chunk_cols / BM, n_pad / BN, lds, [&](int64_t vt, int64_t tt) {
         lmhead_dz_tile(W, hidden, labels, lse, grad, n_tokens, hdim, vocab, c, inv_t, v_begin, chunk_cols, n_pad, dz,
-                       dzt, vt, tt, lds);
+                       vt, tt, lds);
     });
 }
 
@@ -590,14 +667,18 @@ __global__ void __launch_bounds__(NTHREADS)
 // ---------------------------------------------------------------------------------------------
 // mode 0: out_f32  = acc          mode 1: out_f32 += acc
 // mode 2: out_bf16 = acc          mode 3: out_bf16 = out_f32 + acc   (last chunk of d_hidden)
-__device__ __forceinline__ void gemm_store_tile(const uint16_t* __restrict__ A, int64_t lda, int64_t M,
-                                                const uint16_t* __restrict__ B, int64_t ldb, int64_t N, int64_t K,
-                                                int mode, float* out_f32, uint16_t* out_bf16, int64_t ldo,
-                                                int64_t m_valid, int64_t tm, int64_t tn, uint16_t* lds) {
+// A, B: operands without their tile origin (r0 is filled in here); the product has M x N
+// entries, of which rows below m_valid are stored.
+template <bool A_KM, bool B_KM>
+__device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B, int64_t N, int64_t K, int mode,
+                                                float* out_f32, uint16_t* out_bf16, int64_t ldo, int64_t m_valid,
+                                                int64_t tm, int64_t tn, uint16_t* lds) {
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6, wm = wave & 3, wn = wave >> 2;
     const int64_t m0 = tm * BM, n0 = tn * BN;
+    A.r0 = m0;
+    B.r0 = n0;
     AccTile acc;
-    gemm_tile(acc, A, lda, m0, M, B, ldb, n0, N, K, lds);
+    gemm_tile<A_KM, B_KM>(acc, A, B, K, lds);
     if (mode >= 2 && (ldo & 1) == 0) {
         // bf16 output: neighbouring lanes hold neighbouring columns of the same rows; after one DPP
         // swap per pair of rows every lane stores two columns of one row as a 4-byte word (half as
@@ -654,38 +735,20 @@ __device__ __forceinline__ void gemm_store_tile(const uint16_t* __restrict__ A, 
 
 // `queue` null: one workgroup per tile id (blockIdx); otherwise a launch of resident workgroups
 // that draw their tiles from the queue
+template <bool A_KM, bool B_KM>
 __global__ void __launch_bounds__(NTHREADS)
-    gemm_store_kernel(const uint16_t* __restrict__ A, int64_t lda, int64_t M, const uint16_t* __restrict__ B,
-                      int64_t ldb, int64_t N, int64_t K, int mode, float* out_f32, uint16_t* out_bf16, int64_t ldo,
-                      int64_t m_valid, uint32_t* __restrict__ queue) {
+    gemm_store_kernel(const Operand A, int64_t M, const Operand B, int64_t N, int64_t K, int mode, float* out_f32,
+                      uint16_t* out_bf16, int64_t ldo, int64_t m_valid, uint32_t* __restrict__ queue) {
     __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (queue) {
         for_each_tile(queue, tiles_m, tiles_n, lds, [&](int64_t tm, int64_t tn) {
-            gemm_store_tile(A, lda, M, B, ldb, N, K, mode, out_f32, out_bf16, ldo, m_valid, tm, tn, lds);
+            gemm_store_tile<A_KM, B_KM>(A, M, B, N, K, mode, out_f32, out_bf16, ldo, m_valid, tm, tn, lds);
         });
     } else {
         int64_t tm, tn;
         if (tile_of_block(tiles_m, tiles_n, &tm, &tn))
-            gemm_store_tile(A, lda, M, B, ldb, N, K, mode, out_f32, out_bf16, ldo, m_valid, tm, tn, lds);
-    }
-}
-
-// out[c, r] = in[r, c] for bf16, rows of `out` padded with zeros up to ld_out columns
-__global__ void __launch_bounds__(256)
-    transpose_pad_kernel(const uint16_t* __restrict__ in, int64_t rows, int64_t cols, uint16_t* __restrict__ out,
-                         int64_t ld_out) {
-    __shared__ uint16_t tile[64][66];
-    const int64_t r0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64;
-    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    for (int k = ty; k < 64; k += 4) {
-        const int64_t r = r0 + k, cc = c0 + tx;
-        tile[k][tx] = (r < rows && cc < cols) ? in[r * cols + cc] : (uint16_t)0;
-    }
-    __syncthreads();
-    for (int k = ty; k < 64; k += 4) {
-        const int64_t cc = c0 + k, r = r0 + tx;
-        if (cc < cols && r < ld_out) out[cc * ld_out + r] = tile[tx][k];
+            gemm_store_tile<A_KM, B_KM>(A, M, B, N, K, mode, out_f32, out_bf16, ldo, m_valid, tm, tn, lds);
     }
 }
 
@@ -734,29 +797,25 @@ FwdPlan plan_fwd(int64_t n_tokens, int64_t vocab) {
 }
 
 struct BwdPlan {
-    int64_t n_pad, v_pad, chunk;
-    size_t off_wt, off_ht, off_dz, off_dzt, off_dh32, off_queues, total;
-    int64_t n_queues;
+    int64_t n_pad, v_pad, chunk, n_chunks;
+    size_t off_dz, off_dh32, off_queues, total;
 };
-BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab, int want_dw) {
+BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab) {
     BwdPlan p;
     p.n_pad = round_up(n_tokens, 256);
     p.v_pad = round_up(vocab, 256);
     p.chunk = p.v_pad < BWD_VOCAB_CHUNK ? p.v_pad : BWD_VOCAB_CHUNK;
+    p.n_chunks = (p.v_pad + p.chunk - 1) / p.chunk;
     size_t off = 0;
     auto take = [&](size_t bytes) {
         size_t o = off;
         off += (bytes + 255) / 256 * 256;
         return o;
     };
-    p.off_wt = take((size_t)hdim * p.v_pad * 2);
     p.off_dz = take((size_t)p.n_pad * p.chunk * 2);
     p.off_dh32 = take((size_t)n_tokens * hdim * 4);
-    p.off_ht = want_dw ? take((size_t)hdim * p.n_pad * 2) : 0;
-    p.off_dzt = want_dw ? take((size_t)p.chunk * p.n_pad * 2) : 0;
     // one set of work-queue counters per tile-kernel launch (three per vocabulary chunk)
-    p.n_queues = 3 * ((p.v_pad + p.chunk - 1) / p.chunk);
-    p.off_queues = take((size_t)p.n_queues * QUEUE_WORDS * sizeof(uint32_t));
+    p.off_queues = take((size_t)(3 * p.n_chunks) * QUEUE_WORDS * sizeof(uint32_t));
     p.total = off;
     return p;
 }
@@ -813,7 +872,8 @@ extern "C" int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const 
 extern "C" size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
                                                 int want_d_weight) {
     if (n_tokens <= 0 || hidden_dim <= 0 || vocab <= 0) return 0;
-    return plan_bwd(n_tokens, hidden_dim, vocab, want_d_weight).total;
+    (void)want_d_weight;
+    return plan_bwd(n_tokens, hidden_dim, vocab).total;
 }
 
 extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
@@ -826,54 +886,52 @@ extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const 
     OI_RETURN_IF(!lse || !grad_logprob || !d_hidden || !workspace, OI_ENULL);
     OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 2) || !oi_aligned(d_weight, 2), OI_EALIGN);
     const int want_dw = d_weight != nullptr;
-    const BwdPlan p = plan_bwd(n_tokens, hidden_dim, vocab, want_dw);
+    const BwdPlan p = plan_bwd(n_tokens, hidden_dim, vocab);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     hipStream_t s = static_cast<hipStream_t>(stream);
     char* ws = static_cast<char*>(workspace);
-    uint16_t* wt = reinterpret_cast<uint16_t*>(ws + p.off_wt);
     uint16_t* dz = reinterpret_cast<uint16_t*>(ws + p.off_dz);
     float* dh32 = reinterpret_cast<float*>(ws + p.off_dh32);
-    uint16_t* ht = want_dw ? reinterpret_cast<uint16_t*>(ws + p.off_ht) : nullptr;
-    uint16_t* dzt = want_dw ? reinterpret_cast<uint16_t*>(ws + p.off_dzt) : nullptr;
     const uint16_t* Wp = static_cast<const uint16_t*>(weight);
     const uint16_t* Hp = static_cast<const uint16_t*>(hidden);
     const float c = inv_temperature * OI_LOG2E;
 
-    // W^T [H, v_pad] and hidden^T [H, n_pad], zero padded (the pads are multiplied by zero dZ
-    // entries and must not hold NaN/Inf bit patterns)
-    hipLaunchKernelGGL(transpose_pad_kernel, dim3((unsigned)(p.v_pad / 64), (unsigned)(hidden_dim / 64)), dim3(256), 0,
-                       s, Wp, vocab, hidden_dim, wt, p.v_pad);
-    if (want_dw)
-        hipLaunchKernelGGL(transpose_pad_kernel, dim3((unsigned)(p.n_pad / 64), (unsigned)(hidden_dim / 64)), dim3(256),
-                           0, s, Hp, n_tokens, hidden_dim, ht, p.n_pad);
-
     uint32_t* queues = reinterpret_cast<uint32_t*>(ws + p.off_queues);
-    const int n_queue_words = (int)(p.n_queues * QUEUE_WORDS);
+    const int n_queue_words = (int)(3 * p.n_chunks * QUEUE_WORDS);
     hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_queue_words + 255) / 256)), dim3(256), 0, s, queues,
                        n_queue_words);
 
-    const int64_t n_chunks = (p.v_pad + p.chunk - 1) / p.chunk;
+    // Per vocabulary chunk: dZ [n_pad, cols] (token-major, bf16, zero in padded rows and columns),
+    // then both products straight from the caller's W and hidden, which enter as k-major operands:
+    //   d_hidden[n, h] (+)= sum_v dZ[n, v] * W[v_begin + v, h]      A k-contiguous, B k-major
+    //   d_weight[v_begin + v, h] = sum_n dZ[n, v] * hidden[n, h]    A k-major,      B k-major
+    // The sums stop at the last real vocabulary row / token (rounded up to a k-tile, whose missing
+    // rows are read from the last real one and meet zeros of dZ).
     const int64_t h_tiles = (hidden_dim + BN - 1) / BN;
-    for (int64_t ci = 0; ci < n_chunks; ++ci) {
+    for (int64_t ci = 0; ci < p.n_chunks; ++ci) {
         const int64_t v_begin = ci * p.chunk;
         const int64_t cols = (p.v_pad - v_begin) < p.chunk ? (p.v_pad - v_begin) : p.chunk;  // multiple of 256
+        const int64_t valid = vocab - v_begin < cols ? vocab - v_begin : cols;               // real rows of W
         uint32_t* q = queues + ci * 3 * QUEUE_WORDS;
         hipLaunchKernelGGL(lmhead_dz_kernel, dim3(resident_grid(cols / BM, p.n_pad / BN)), dim3(NTHREADS), 0, s, Wp,
                            Hp, labels, lse, grad_logprob, n_tokens, hidden_dim, vocab, c, inv_temperature, v_begin,
-                           cols, p.n_pad, dz, dzt, q);
-        // d_hidden[n, h] (+)= sum_v dZ[n, v] * W^T[h, v_begin + v]
-        const bool first = ci == 0, last = ci == n_chunks - 1;
+                           cols, p.n_pad, dz, q);
+        const bool first = ci == 0, last = ci == p.n_chunks - 1;
         const int mode = last ? (first ? 2 : 3) : (first ? 0 : 1);
-        hipLaunchKernelGGL(gemm_store_kernel, dim3(resident_grid(p.n_pad / BM, h_tiles)), dim3(NTHREADS), 0, s, dz,
-                           cols, p.n_pad, wt + v_begin, p.v_pad, hidden_dim, cols, mode, dh32,
-                           static_cast<uint16_t*>(d_hidden), hidden_dim, n_tokens, q + QUEUE_WORDS);
+        {
+            const Operand a = {dz, cols, 0, p.n_pad, cols};
+            const Operand b = {Wp + v_begin * hidden_dim, hidden_dim, 0, hidden_dim, valid};
+            hipLaunchKernelGGL((gemm_store_kernel<false, true>), dim3(resident_grid(p.n_pad / BM, h_tiles)),
+                               dim3(NTHREADS), 0, s, a, p.n_pad, b, hidden_dim, round_up(valid, BK), mode, dh32,
+                               static_cast<uint16_t*>(d_hidden), hidden_dim, n_tokens, q + QUEUE_WORDS);
+        }
         if (want_dw) {
-            // d_weight[v_begin + m, h] = sum_n dZ^T[m, n] * hidden^T[h, n]
-            const int64_t valid = vocab - v_begin < cols ? vocab - v_begin : cols;
-            hipLaunchKernelGGL(gemm_store_kernel, dim3(resident_grid(cols / BM, h_tiles)), dim3(NTHREADS), 0, s, dzt,
-                               p.n_pad, cols, ht, p.n_pad, hidden_dim, p.n_pad, 2, static_cast<float*>(nullptr),
-                               static_cast<uint16_t*>(d_weight) + v_begin * hidden_dim, hidden_dim, valid,
-                               q + 2 * QUEUE_WORDS);
+            const Operand a = {dz, cols, 0, cols, p.n_pad};
+            const Operand b = {Hp, hidden_dim, 0, hidden_dim, n_tokens};
+            hipLaunchKernelGGL((gemm_store_kernel<true, true>), dim3(resident_grid(cols / BM, h_tiles)),
+                               dim3(NTHREADS), 0, s, a, cols, b, hidden_dim, round_up(n_tokens, BK), 2,
+                               static_cast<float*>(nullptr), static_cast<uint16_t*>(d_weight) + v_begin * hidden_dim,
+                               hidden_dim, valid, q + 2 * QUEUE_WORDS);
         }
     }
     return oi_launch_status();
@@ -889,9 +947,10 @@ extern "C" int oi_gemm_bf16_tn(const void* A, int64_t lda, int64_t M, const void
     OI_RETURN_IF(accumulate && !out_f32, OI_EINVAL);
     OI_RETURN_IF(!oi_aligned(A, 16) || !oi_aligned(B, 16), OI_EALIGN);
     const int mode = out_f32 ? (accumulate ? 1 : 0) : 2;
-    hipLaunchKernelGGL(gemm_store_kernel, dim3(grid_for_tiles((M + BM - 1) / BM, (N + BN - 1) / BN)), dim3(NTHREADS),
-                       0, static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(A), lda, M,
-                       static_cast<const uint16_t*>(B), ldb, N, K, mode, out_f32, static_cast<uint16_t*>(out_bf16), ldo,
-                       M, static_cast<uint32_t*>(nullptr));
+    const Operand a = {static_cast<const uint16_t*>(A), lda, 0, M, K};
+    const Operand b = {static_cast<const uint16_t*>(B), ldb, 0, N, K};
+    hipLaunchKernelGGL((gemm_store_kernel<false, false>), dim3(grid_for_tiles((M + BM - 1) / BM, (N + BN - 1) / BN)),
+                       dim3(NTHREADS), 0, static_cast<hipStream_t>(stream), a, M, b, N, K, mode, out_f32,
+                       static_cast<uint16_t*>(out_bf16), ldo, M, static_cast<uint32_t*>(nullptr));
     return oi_launch_status();
 }

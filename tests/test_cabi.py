@@ -83,7 +83,9 @@ def test_rejected_arguments_return_codes_without_launching():
     assert lib.oi_logprob_diff_stats(None, None, None, -1, None, None) == -1
     assert lib.oi_masked_mean_workspace_bytes(4, 2, 3) == (4 + 1) * 2 * 1 * 4
     assert lib.oi_lmhead_fwd_workspace_bytes(0, 64, 10) == 0
-    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1) > lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 0)
+    # one dZ chunk (bf16), the fp32 d_hidden accumulator, three queues of 8 words; no transposed copies
+    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1) == 256 * 256 * 2 + 256 * 64 * 4 + 256
+    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 0) == lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1)
 
 
 def test_cpu_tensors_are_refused_loudly():

@@ -53,7 +53,20 @@ def test_forward_matches_oracle(n, h, v, temperature):
     assert none is None and torch.equal(lp2, lp)  # deterministic, run to run
 
 
-@pytest.mark.parametrize("n,h,v", [(256, 64, 256), (300, 128, 1000), (700, 256, 5000), (260, 64, 17000), (260, 64, 33000)])
+@pytest.mark.parametrize(
+    "n,h,v",
+    [
+        (256, 64, 256),
+        (300, 128, 1000),
+        (700, 256, 5000),
+        (260, 64, 17000),
+        (260, 64, 33000),  # two vocabulary chunks, the second with 232 of 256 real rows
+        (40, 64, 50),  # one k-tile in both backward products, most of its rows missing
+        (100, 64, 100),  # two k-tiles
+        (130, 128, 150),  # three k-tiles
+        (2, 64, 7),
+    ],
+)
 @pytest.mark.parametrize("want_dw", [True, False])
 def test_backward_matches_oracle(n, h, v, want_dw):
     print(f"case N={n} H={h} V={v} dW={want_dw}", flush=True)
