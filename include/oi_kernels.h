@@ -294,8 +294,10 @@ int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* la
  *   dZ[n, v] = grad_logprob[n] * inv_T * (1[v == label_n] - exp(z[n,v] * inv_T - lse[n])),
  *   d_hidden = dZ @ weight   (bf16 [n_tokens, hidden_dim]),
  *   d_weight = dZ^T @ hidden (bf16 [vocab, hidden_dim]; NULL skips it).
- * Vocabulary is processed in chunks of 32768 columns; only one chunk of dZ (bf16) lives in the
- * workspace at a time.
+ * Vocabulary is processed in chunks of 32768 columns; only one chunk of dZ (bf16, token-major)
+ * lives in the workspace at a time, next to the fp32 accumulator of d_hidden.  Both products
+ * read weight, hidden and dZ where they lie (no transposed copies), so the workspace is the same
+ * with and without d_weight.
  */
 size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int want_d_weight);
 int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
