@@ -316,6 +316,19 @@ int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* la
 int oi_gemm_bf16_tn(const void* A, int64_t lda, int64_t M, const void* B, int64_t ldb, int64_t N, int64_t K,
                     float* out_f32, void* out_bf16, int64_t ldo, int accumulate, void* stream);
 
+/*
+ * The same product with either operand in k-major order (no reference counterpart; test and timing
+ * hook of the operand layouts that the backward of the fused lm_head uses to read weight, hidden
+ * and dZ where they lie):
+ *   out[m, n] (+)= sum_k a(m, k) * b(n, k),   a(m, k) = a_k_major ? A[k * lda + m] : A[m * lda + k],
+ *                                             b(n, k) = b_k_major ? B[k * ldb + n] : B[n * ldb + k].
+ * K must be a multiple of 64; lda/ldb positive multiples of 8, at most 2^22 and at least the
+ * operand's contiguous extent; M (N) a multiple of 8 when A (B) is k-major.
+ */
+int oi_gemm_bf16_layouts(const void* A, int64_t lda, int a_k_major, const void* B, int64_t ldb, int b_k_major,
+                         int64_t M, int64_t N, int64_t K, float* out_f32, void* out_bf16, int64_t ldo,
+                         int accumulate, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

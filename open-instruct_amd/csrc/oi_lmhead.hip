@@ -954,3 +954,36 @@ extern "C" int oi_gemm_bf16_tn(const void* A, int64_t lda, int64_t M, const void
                        static_cast<uint16_t*>(out_bf16), ldo, M, static_cast<uint32_t*>(nullptr));
     return oi_launch_status();
 }
+
+extern "C" int oi_gemm_bf16_layouts(const void* A, int64_t lda, int a_k_major, const void* B, int64_t ldb,
+                                    int b_k_major, int64_t M, int64_t N, int64_t K, float* out_f32, void* out_bf16,
+                                    int64_t ldo, int accumulate, void* stream) {
+    OI_RETURN_IF(M <= 0 || N <= 0 || K <= 0 || K % 64 != 0 || ldo < N, OI_EINVAL);
+    OI_RETURN_IF(lda <= 0 || ldb <= 0 || lda % 8 != 0 || ldb % 8 != 0 || lda > MAX_LD || ldb > MAX_LD, OI_EINVAL);
+    // a k-major operand is read in 16-byte column chunks: whole chunks only
+    OI_RETURN_IF(lda < (a_k_major ? M : K) || ldb < (b_k_major ? N : K), OI_EINVAL);
+    OI_RETURN_IF((a_k_major && M % 8 != 0) || (b_k_major && N % 8 != 0), OI_EINVAL);
+    OI_RETURN_IF(!A || !B || (!out_f32 && !out_bf16) || (out_f32 && out_bf16), OI_ENULL);
+    OI_RETURN_IF(accumulate && !out_f32, OI_EINVAL);
+    OI_RETURN_IF(!oi_aligned(A, 16) || !oi_aligned(B, 16), OI_EALIGN);
+    const int mode = out_f32 ? (accumulate ? 1 : 0) : 2;
+    const Operand a = {static_cast<const uint16_t*>(A), lda, 0, M, K};
+    const Operand b = {static_cast<const uint16_t*>(B), ldb, 0, N, K};
+    const dim3 grid(grid_for_tiles((M + BM - 1) / BM, (N + BN - 1) / BN));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint16_t* o16 = static_cast<uint16_t*>(out_bf16);
+    uint32_t* no_queue = nullptr;
+    if (a_k_major && b_k_major)
+        hipLaunchKernelGGL((gemm_store_kernel<true, true>), grid, dim3(NTHREADS), 0, s, a, M, b, N, K, mode, out_f32, o16,
+                           ldo, M, no_queue);
+    else if (a_k_major)
+        hipLaunchKernelGGL((gemm_store_kernel<true, false>), grid, dim3(NTHREADS), 0, s, a, M, b, N, K, mode, out_f32,
+                           o16, ldo, M, no_queue);
+    else if (b_k_major)
+        hipLaunchKernelGGL((gemm_store_kernel<false, true>), grid, dim3(NTHREADS), 0, s, a, M, b, N, K, mode, out_f32,
+                           o16, ldo, M, no_queue);
+    else
+        hipLaunchKernelGGL((gemm_store_kernel<false, false>), grid, dim3(NTHREADS), 0, s, a, M, b, N, K, mode, out_f32,
+                           o16, ldo, M, no_queue);
+    return oi_launch_status();
+}

@@ -75,6 +75,8 @@ def test_rejected_arguments_return_codes_without_launching():
     assert lib.oi_lmhead_logp_fwd(None, None, None, big, 64, 32, 1.0, None, None, None, None, 0, None) == -1
     assert lib.oi_gemm_bf16_tn(None, big, 4, None, 64, 4, 64, None, None, 4, 0, None) == -1
     assert lib.oi_gemm_bf16_tn(None, 72, 4, None, 72, 4, 72, None, None, 4, 0, None) == -1  # K % 64
+    assert lib.oi_gemm_bf16_layouts(None, 72, 1, None, 72, 0, 4, 8, 64, None, None, 8, 0, None) == -1  # M % 8, A k-major
+    assert lib.oi_gemm_bf16_layouts(None, 72, 1, None, 72, 0, 8, 8, 64, None, None, 8, 0, None) == -2
     # packing and logprob statistics: missing pointers / sizes
     assert lib.oi_pack_sequences(*([None] * 9), -1, 0, 0, *([None] * 8)) == -1
     assert lib.oi_pack_sequences(*([None] * 9), 3, 0, 0, *([None] * 8)) == -2

@@ -164,6 +164,52 @@ def test_gemm_bf16_tn_entry_point(m, n, k):
     assert lib.oi_gemm_bf16_tn(ad.data_ptr(), k, m, bd.data_ptr(), k, n, k, None, None, n, 0, stream) != 0
 
 
+@pytest.mark.parametrize("a_km,b_km", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 64), (304, 520, 192), (8, 72, 128), (1032, 264, 1024), (64, 64, 4096)])
+def test_gemm_bf16_operand_layouts(m, n, k, a_km, b_km):
+    """Every combination of k-contiguous and k-major operands through the raw C-ABI: one, two, three
+    and many k-tiles, ragged tile edges in both dimensions, padded leading dimensions."""
+    print(f"case M={m} N={n} K={k} A k-major={a_km} B k-major={b_km}", flush=True)
+    torch.manual_seed(11)
+    a = torch.randn(m, k).bfloat16()
+    b = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    exp = o_lm.lm_head_logits(a, b, torch.float64)
+    lib = _lib.load()
+
+    def device_operand(x, k_major):
+        rows, cols = (x.shape[1], x.shape[0]) if k_major else x.shape
+        ld = cols + 16  # padded rows, filled with a value that must never be read as data
+        buf = torch.full((rows, ld), 77.0, dtype=torch.bfloat16, device=DEV)
+        buf[:, :cols] = (x.t() if k_major else x).to(DEV)
+        return buf, ld
+
+    ad, lda = device_operand(a, a_km)
+    bd, ldb = device_operand(b, b_km)
+    out32 = torch.full((m, n), -0.25, dtype=torch.float32, device=DEV)
+    out16 = torch.zeros(m, n, dtype=torch.bfloat16, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    args = (ad.data_ptr(), lda, a_km, bd.data_ptr(), ldb, b_km, m, n, k)
+    assert lib.oi_gemm_bf16_layouts(*args, out32.data_ptr(), None, n, 1, stream) == 0
+    assert lib.oi_gemm_bf16_layouts(*args, None, out16.data_ptr(), n, 0, stream) == 0
+    torch.cuda.synchronize()
+    assert (out32.cpu().double() + 0.25 - exp).abs().max().item() <= 1e-4
+    assert (out16.cpu().double() - exp).abs().max().item() <= exp.abs().max().item() * 2**-8 + 1e-4
+    # the two layouts of the same numbers give the same bits (same products, same order of summation)
+    if a_km or b_km:
+        ref32 = torch.zeros(m, n, dtype=torch.float32, device=DEV)
+        a0, b0 = a.to(DEV).contiguous(), b.to(DEV).contiguous()
+        assert lib.oi_gemm_bf16_layouts(a0.data_ptr(), k, 0, b0.data_ptr(), k, 0, m, n, k, ref32.data_ptr(), None, n, 0, stream) == 0
+        got32 = torch.zeros(m, n, dtype=torch.float32, device=DEV)
+        assert lib.oi_gemm_bf16_layouts(*args, got32.data_ptr(), None, n, 0, stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(ref32, got32)
+    # rejected arguments launch nothing
+    assert lib.oi_gemm_bf16_layouts(ad.data_ptr(), lda, a_km, bd.data_ptr(), ldb, b_km, m, n, k + 8, out32.data_ptr(), None, n, 0, stream) == -1
+    assert lib.oi_gemm_bf16_layouts(ad.data_ptr(), 4, a_km, bd.data_ptr(), ldb, b_km, m, n, k, out32.data_ptr(), None, n, 0, stream) == -1
+    if a_km:
+        assert lib.oi_gemm_bf16_layouts(ad.data_ptr(), lda, 1, bd.data_ptr(), ldb, b_km, m - 1, n, k, out32.data_ptr(), None, n, 0, stream) == -1
+
+
 def test_full_size_properties_fused_head():
     """Llama-3.1-8B head shape (H = 4096, V = 128256), 1500 rows: properties that need no oracle.
 
