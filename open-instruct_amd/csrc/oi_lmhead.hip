@@ -1,21 +1,25 @@
 // Fused lm_head projection + per-token logprob / entropy for gfx950, logits never materialised.
 //
-// One bf16 MFMA main loop (C[m, n] = sum_k A[m, k] * B[n, k], both operands row-major with k
-// contiguous) serves four kernels that differ only in what they do with the fp32 tile:
+// One bf16 MFMA main loop, C[m, n] = sum_k a(m, k) * b(n, k), serves four kernels that differ in
+// what they do with the fp32 tile and in the memory order of their operands (k-contiguous: the k
+// values of a row lie together; k-major: the rows of a k value lie together):
 //
-//   forward   A = W [V, H],  B = hidden [N, H]   -> online (max, sum-exp, sum exp*z) per token,
-//                                                    merged over the vocabulary tiles of a split
-//   dz        A = W,         B = hidden          -> dZ = g * (onehot - softmax), bf16, written in
-//                                                    both [token, vocab] and [vocab, token] order
-//   d_hidden  A = dZ [N, Vc], B = W^T [H, V]     -> fp32 accumulate over vocabulary chunks
-//   d_weight  A = dZ^T [Vc, N], B = hidden^T     -> bf16 rows of dW for the chunk
+//   forward   a = W [V, H],  b = hidden [N, H]   both k-contiguous -> online (max, sum-exp,
+//             sum exp*z) per token, merged over the vocabulary tiles of a work item
+//   dz        a = W,         b = hidden          -> dZ = g * (onehot - softmax), bf16 [N, Vc]
+//   d_hidden  a = dZ [N, Vc] k-contiguous, b = W [Vc, H] k-major -> fp32 accumulate over chunks
+//   d_weight  a = dZ [N, Vc] k-major,      b = hidden [N, H] k-major -> bf16 rows of dW
+//
+// so the backward reads W, hidden and dZ where they lie: no transposed copies.
 //
 // Tile: 256 x 256 x 64 per 512-thread workgroup, 8 waves as 4 (m) x 2 (n), each wave 64 x 128 =
 // 2 x 4 MFMA 32x32x16 accumulators.  With vocabulary as the m dim a lane's 16 accumulator
 // registers of one MFMA tile belong to ONE token (column), so the softmax statistics reduce
 // inside the lane.  LDS: a ring of five 32 KB operand slots (k-tiles of A and of B) filled by
-// direct global->LDS loads of whole 128-byte row segments; rows are unpadded and their 16-byte
-// chunks XOR-permuted so that fragment reads stay free of bank conflicts.
+// direct global->LDS loads of whole 128-byte line segments; the 16-byte chunks of a row are
+// XOR-permuted so that fragment reads (16-byte reads of a k-contiguous image, transposing 8-byte
+// reads of a k-major image) stay free of bank conflicts.  A launch is one resident workgroup per
+// CU that draws tile ids from per-XCD counters.
 #include "oi_common.h"
 
 #include <type_traits>
