@@ -65,6 +65,8 @@ def test_forward_matches_oracle(n, h, v, temperature):
         (100, 64, 100),  # two k-tiles
         (130, 128, 150),  # three k-tiles
         (2, 64, 7),
+        (300, 320, 1000),  # hidden size between one and two tiles wide: clamped column chunks
+        (130, 192, 300),
     ],
 )
 @pytest.mark.parametrize("want_dw", [True, False])
