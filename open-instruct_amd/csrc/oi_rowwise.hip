@@ -435,6 +435,9 @@ int launch_bwd(const void* logits, int64_t rows, int64_t n_inner, int64_t so, in
 // ---------------------------------------------------------------------------------------------
 constexpr int FUSED_ROW_THREADS = 1024;
 constexpr int FUSED_ROW_U = 4;
+// 16-byte pieces of a row that wait in the LDS for the second pass: 144 KB of the CU's 160 KB (the
+// kernel runs one 1024-thread workgroup per CU anyway), a whole number of sweeps of the workgroup
+constexpr int FUSED_STASH_VECS = 9 * FUSED_ROW_THREADS;
 
 template <typename R>
 __global__ void __launch_bounds__(FUSED_ROW_THREADS)
@@ -452,6 +455,8 @@ __global__ void __launch_bounds__(FUSED_ROW_THREADS)
     constexpr int64_t nthr = FUSED_ROW_THREADS;
     __shared__ float sm[3][NW];
     __shared__ float bcast[2];
+    __shared__ __align__(16) typename R::raw_t stash[FUSED_STASH_VECS];
+    static_assert(sizeof(typename R::raw_t) == 16, "row pieces are 16 bytes");
     const int64_t row = blockIdx.x;
     const typename R::elem_t* p = logits + row_offset(row, n_inner, stride_outer, stride_inner);
     typename R::elem_t* q = dlogits + row_offset(row, n_inner, out_stride_outer, out_stride_inner);
@@ -459,21 +464,38 @@ __global__ void __launch_bounds__(FUSED_ROW_THREADS)
     const int64_t nvec = vocab / VEC;
     const float c = inv_t * OI_LOG2E;
 
+    // The first FUSED_STASH_VECS 16-byte pieces of the row stay in the LDS between the two passes
+    // (every thread keeps exactly the pieces it will need again, so no barrier guards them); only
+    // the rest of the row is read a second time, from the caches.  Pieces that go into the LDS
+    // are fetched with non-temporal loads, the others with ordinary ones so that they stay cached.
     RowStat st = {OI_NEG_BIG, 0.f, 0.f};
     {
         int64_t i = tid;
         for (; i + (U - 1) * nthr < nvec; i += U * nthr) {
             typename R::raw_t raw[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) raw[u] = R::load_raw_cached(p + (i + u * nthr) * VEC);
+            for (int u = 0; u < U; ++u) {
+                const int64_t v = i + u * nthr;
+                raw[u] = (v - tid < FUSED_STASH_VECS) ? R::load_raw(p + v * VEC) : R::load_raw_cached(p + v * VEC);
+            }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
+                const int64_t v = i + u * nthr;
+                if (v - tid < FUSED_STASH_VECS) stash[v] = raw[u];
                 float z[VEC];
                 R::unpack(raw[u], z);
                 stat_update<VEC, true>(st, z, c);
             }
         }
         for (; i < nvec; i += nthr) {
+            if (i - tid < FUSED_STASH_VECS) {
+                const typename R::raw_t r = R::load_raw(p + i * VEC);
+                stash[i] = r;
+                float z[VEC];
+                R::unpack(r, z);
+                stat_update<VEC, true>(st, z, c);
+                continue;
+            }
             float z[VEC];
             R::unpack(R::load_raw_cached(p + i * VEC), z);
             stat_update<VEC, true>(st, z, c);
@@ -532,50 +554,43 @@ __global__ void __launch_bounds__(FUSED_ROW_THREADS)
         for (int64_t j = nvec * VEC + tid; j < vocab; j += nthr) R::store_one(q + j, 0.f);
         return;
     }
-    // second pass: the row was read moments ago by this workgroup
-    int64_t i = tid;
-    float z[U][VEC], zn[U][VEC];
+    // second pass.  The tail of the row (read moments ago by this workgroup) comes from the
+    // caches: its first loads are requested now and consumed after the part that waits in the LDS.
+    const int64_t head = nvec < FUSED_STASH_VECS ? nvec : (int64_t)FUSED_STASH_VECS;
+    int64_t i = FUSED_STASH_VECS + tid;
+    typename R::raw_t rz[U], rn[U];
     if (i + (U - 1) * nthr < nvec) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) R::load_vec(p + (i + u * nthr) * VEC, z[u]);
+        for (int u = 0; u < U; ++u) rz[u] = R::load_raw(p + (i + u * nthr) * VEC);
     }
+    auto emit = [&](typename R::raw_t raw, int64_t base) {
+        float w[VEC];
+        R::unpack(raw, w);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) w[j] = ng * __builtin_amdgcn_exp2f(fmaf(w[j], c, -l2));
+        if (y >= base && y < base + VEC) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                if (base + j == y) w[j] += g;
+        }
+        R::store_vec(q + base, w);
+    };
+    for (int64_t k = tid; k < head; k += nthr) emit(stash[k], k * VEC);
     for (; i + (U - 1) * nthr < nvec; i += U * nthr) {
         const int64_t nx = i + U * nthr;
         const bool more = nx + (U - 1) * nthr < nvec;
         if (more) {
 #pragma unroll
-            for (int u = 0; u < U; ++u) R::load_vec(p + (nx + u * nthr) * VEC, zn[u]);
+            for (int u = 0; u < U; ++u) rn[u] = R::load_raw(p + (nx + u * nthr) * VEC);
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int64_t base = (i + u * nthr) * VEC;
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) z[u][j] = ng * __builtin_amdgcn_exp2f(fmaf(z[u][j], c, -l2));
-            if (y >= base && y < base + VEC) {
-#pragma unroll
-                for (int j = 0; j < VEC; ++j)
-                    if (base + j == y) z[u][j] += g;
-            }
-            R::store_vec(q + base, z[u]);
-        }
+        for (int u = 0; u < U; ++u) emit(rz[u], (i + u * nthr) * VEC);
         if (more) {
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) z[u][j] = zn[u][j];
+            for (int u = 0; u < U; ++u) rz[u] = rn[u];
         }
     }
-    for (; i < nvec; i += nthr) {
-        float w[VEC];
-        const int64_t base = i * VEC;
-        R::load_vec(p + base, w);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-            w[j] = ng * __builtin_amdgcn_exp2f(fmaf(w[j], c, -l2));
-            if (base + j == y) w[j] += g;
-        }
-        R::store_vec(q + base, w);
-    }
+    for (; i < nvec; i += nthr) emit(R::load_raw(p + i * VEC), i * VEC);
     for (int64_t j = nvec * VEC + tid; j < vocab; j += nthr) {
         float d = ng * __builtin_amdgcn_exp2f(fmaf(R::load_one(p + j), c, -l2));
         if (j == y) d += g;
