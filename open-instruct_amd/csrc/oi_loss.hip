@@ -745,7 +745,7 @@ extern "C" int oi_logprob_diff_stats(const float* local_logprobs, const float* o
     return oi_launch_status();
 }
 
-extern "C" int oi_version(void) { return 1001; }
+extern "C" int oi_version(void) { return 1002; }
 
 extern "C" const char* oi_error_string(int code) {
     switch (code) {
