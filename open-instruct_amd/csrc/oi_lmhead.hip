@@ -611,15 +611,24 @@ __device__ __forceinline__ void lmhead_dz_tile(const uint16_t* __restrict__ W, c
 
     // stage[n][v]: rows = tokens of the tile, 256 (+8 pad) vocabulary columns
     uint16_t* stage = lds;
+    const int rows_left = (int)(vocab - m0 < BM ? vocab - m0 : BM);  // real vocabulary rows of the tile
+    const int wave_row0 = wm * 64;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int nl = acc_col(wn, j, lane);
         const int64_t n = n0 + nl;
         const bool live = n < n_tokens;
         const float g = live ? grad[n] * inv_t : 0.f;
-        const float l2 = live ? lse[n] * OI_LOG2E : 0.f;
+        // a token without gradient gets an exponent of -huge: every entry becomes -0 * 0
+        const float l2 = g != 0.f ? lse[n] * OI_LOG2E : 3.0e38f;
         int64_t y = live ? labels[n] : -1;
         if (live) y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
+        // the label's entry gets + g; find out whether this lane holds it and in which register
+        const int rel = (live && y >= m0 && y < m0 + BM) ? (int)(y - m0) - wave_row0 : -1;
+        const bool mine = rel >= 0 && rel < 64 && (((rel & 31) >> 2) & 1) == (lane >> 5);
+        const int target = mine ? (rel >> 5) * 16 + ((rel & 31) >> 3) * 4 + (rel & 3) : -1;
+        const float ng = -g;
+        float z_label = 0.f;
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -628,18 +637,20 @@ __device__ __forceinline__ void lmhead_dz_tile(const uint16_t* __restrict__ W, c
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int r = q * 4 + e;
-                    const int64_t v = m0 + acc_row(wm, i, r, lane);
-                    float val = 0.f;
-                    if (g != 0.f && v < vocab) {
-                        val = -g * __builtin_amdgcn_exp2f(fmaf(acc[i][j][r], c, -l2));
-                        if (v == y) val += g;
-                    }
+                    if (i * 16 + r == target) z_label = acc[i][j][r];
+                    float val = ng * __builtin_amdgcn_exp2f(fmaf(acc[i][j][r], c, -l2));
+                    if (rows_left < BM && acc_row(wm, i, r, lane) >= rows_left) val = 0.f;  // last tile only
                     d[e] = val;
                 }
                 const int vl = acc_row(wm, i, q * 4, lane);
                 uint2 pk = make_uint2(oi_pack_bf16x2(d[0], d[1]), oi_pack_bf16x2(d[2], d[3]));
                 *reinterpret_cast<uint2*>(stage + nl * STAGE_STRIDE + vl) = pk;
             }
+        if (mine) {
+            // same lane, same LDS word as the store above: program order keeps them apart
+            const float val = fmaf(ng, __builtin_amdgcn_exp2f(fmaf(z_label, c, -l2)), g);
+            stage[nl * STAGE_STRIDE + wave_row0 + rel] = (uint16_t)oi_f32_to_bf16_bits(val);
+        }
     }
     __syncthreads();
     const int64_t vcol0 = vt * BM;  // column of this tile inside the chunk
