@@ -61,6 +61,8 @@ def test_forward_matches_oracle(n, h, v, temperature):
         (700, 256, 5000),
         (260, 64, 17000),
         (260, 64, 33000),  # two vocabulary chunks, the second with 232 of 256 real rows
+        (260, 64, 70000),  # three chunks: d_hidden accumulates in fp32 over a middle chunk
+        (130, 128, 100000),  # four chunks, the last with 1696 columns
         (40, 64, 50),  # one k-tile in both backward products, most of its rows missing
         (100, 64, 100),  # two k-tiles
         (130, 128, 150),  # three k-tiles
