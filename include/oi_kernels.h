@@ -97,7 +97,7 @@ int oi_lsg_bwd(const void* logits, int dtype, int64_t n_outer, int64_t n_inner, 
  * token_coef (fp32 per row) carries the loss denominators, which depend on the mask alone:
  * scale / denominator on response tokens, 0 elsewhere (such rows get a zero gradient row).
  * Requirement: 16-byte aligned rows (pointers and strides of logits and dlogits); OI_EALIGN
- * otherwise (use the two-pass entry points).  dlogits must not alias logits.  The scalar loss and
+ * otherwise (use the two-pass entry points).  dlogits must not alias logits (OI_EINVAL).  The scalar loss and
  * its statistics come from oi_grpo_fused_fwd on `logprob`.
  */
 int oi_lsg_grpo_fwd_bwd(const void* logits, int dtype, int64_t n_outer, int64_t n_inner, int64_t stride_outer,
@@ -106,6 +106,15 @@ int oi_lsg_grpo_fwd_bwd(const void* logits, int dtype, int64_t n_outer, int64_t 
                         const float* rho_weights, const float* token_coef, int loss_fn, float ratio_lo,
                         float ratio_hi, int kl_estimator, float beta, float* logprob, float* entropy, float* lse,
                         void* dlogits, int64_t out_stride_outer, int64_t out_stride_inner, void* stream);
+
+/*
+ * data[i] *= *scale over a contiguous tensor of n elements (dtype tag as above), where `scale` is
+ * a DEVICE scalar; when it is exactly 1 the kernel leaves the data untouched.  No reference
+ * counterpart: it applies the upstream gradient of the loss to the gradient that
+ * oi_lsg_grpo_fwd_bwd stored, the step autograd performs at open_instruct/grpo_fast.py:724
+ * (`loss.backward()`), without a host read of the scalar.
+ */
+int oi_scale_by_device_scalar(void* data, int dtype, int64_t n, const float* scale, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Per-token GRPO loss terms.  Carries open_instruct/grpo_utils.py:504-538 (compute_grpo_loss)
@@ -139,16 +148,39 @@ int oi_grpo_terms_bwd(const float* new_logprobs, const float* ratio, const float
  *
  * out_stats (fp32[OI_GRPO_NUM_STATS]): [0] loss, [1] masked mean pg, [2..5] masked mean of KL
  * estimators 0..3, [6] masked mean clipfrac, [7] masked mean ratio, [8] masked mean entropy,
- * [9] mask.sum().  row_denoms (fp32[rows]) receives the reciprocal denominator applied to each
- * row's tokens, which oi_grpo_fused_bwd consumes.
+ * [9] mask.sum(), [10..12] masked means of the rho drop indicators (any / below the lower bound /
+ * above the upper bound), [13] masked mean of rho_weights, [14] masked mean of the rho clamp
+ * indicator (the five metric tensors of open_instruct/grpo_utils.py:446-452; 0 for a NULL
+ * pointer, [13] is 1 without rho_weights), [15] = [2 + kl_estimator] * beta, the "loss/kl_avg" of
+ * open_instruct/grpo_utils.py:718.  row_denoms (fp32[rows]) receives the reciprocal denominator
+ * applied to each row's tokens, which oi_grpo_fused_bwd consumes.  rows * ceil(cols / 1024) must
+ * stay below 2^31 (one block per row and 1024 columns).
  */
-#define OI_GRPO_NUM_STATS 10
+#define OI_GRPO_NUM_STATS 16
 size_t oi_grpo_fused_workspace_bytes(int64_t rows, int64_t cols);
 int oi_grpo_fused_fwd(const float* new_logprobs, const float* old_logprobs, const float* ref_logprobs,
                       const float* advantages, const uint8_t* mask, const float* rho_weights, const float* entropy,
-                      int64_t rows, int64_t cols, int loss_fn, float ratio_lo, float ratio_hi, int kl_estimator,
-                      float beta, int axis_mode, float denominator, float scale, float* out_stats,
-                      float* row_denoms, void* workspace, size_t workspace_bytes, void* stream);
+                      const float* rho_drop_any, const float* rho_drop_low, const float* rho_drop_high,
+                      const float* rho_clipped, int64_t rows, int64_t cols, int loss_fn, float ratio_lo,
+                      float ratio_hi, int kl_estimator, float beta, int axis_mode, float denominator, float scale,
+                      float* out_stats, float* row_denoms, void* workspace, size_t workspace_bytes, void* stream);
+/*
+ * The same statistics for a caller that already holds the per-token terms.  Carries
+ * open_instruct/grpo_utils.py:699-729 (populate_sample_loss_stats) in two launches: masked means
+ * of pg_loss, clipfrac, ratio, of the four KL estimators of clamp(new - ref, +-40) (zeros when
+ * ref_logprobs is NULL), of entropy and of the rho metric tensors.  Statistic q (numbering of
+ * oi_grpo_fused_fwd; [0] is the caller's own loss and is never written) goes to
+ * out_stats[q * out_stride] when bit q of write_mask is set, so one column of a
+ * [OI_GRPO_NUM_STATS, num_samples] table can be filled in place.  Workspace as for
+ * oi_grpo_fused_fwd.
+ */
+int oi_grpo_stats_from_terms(const float* pg_loss, const float* clipfrac, const float* ratio,
+                             const float* new_logprobs, const float* ref_logprobs, const uint8_t* mask,
+                             const float* entropy, const float* rho_weight, const float* rho_drop_any,
+                             const float* rho_drop_low, const float* rho_drop_high, const float* rho_clipped,
+                             int64_t rows, int64_t cols, int kl_estimator, float beta, float* out_stats,
+                             int64_t out_stride, uint32_t write_mask, void* workspace, size_t workspace_bytes,
+                             void* stream);
 /* d loss / d new_logprobs (fp32 [rows, cols]); grad_loss is a DEVICE scalar (upstream gradient). */
 int oi_grpo_fused_bwd(const float* new_logprobs, const float* old_logprobs, const float* ref_logprobs,
                       const float* advantages, const uint8_t* mask, const float* rho_weights, int64_t rows,
@@ -190,7 +222,8 @@ int oi_group_advantages(const double* scores, int64_t n_groups, int64_t group_si
 /* ------------------------------------------------------------------------------------------
  * Masked mean.  Carries open_instruct/rl_utils.py:426-448 for fp32 values [extra, rows, cols]
  * and a byte or fp32 mask [rows, cols] (mask_is_float selects).  axis_mode as above;
- * out: fp32 [extra].  row_denoms (fp32 [rows], may be NULL) as above.
+ * out: fp32 [extra].  row_denoms (fp32 [rows], may be NULL) as above.  extra <= 65535 and
+ * extra * rows * ceil(cols / 1024) < 2^31.
  * ------------------------------------------------------------------------------------------ */
 size_t oi_masked_mean_workspace_bytes(int64_t extra, int64_t rows, int64_t cols);
 int oi_masked_mean_fwd(const float* values, const void* mask, int mask_is_float, int64_t extra, int64_t rows,

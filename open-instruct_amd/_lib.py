@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_uint32, c_void_p
 
 import torch
 
@@ -35,8 +35,10 @@ SIGNATURES: dict[str, tuple] = {
     "oi_grpo_fused_workspace_bytes": (_SZ, [_I64, _I64]),
     "oi_grpo_fused_fwd": (
         _I,
-        [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I, _F, _F, _I, _F, _I, _F, _F, _P, _P, _P, _SZ, _P],
+        [_P] * 11 + [_I64, _I64, _I, _F, _F, _I, _F, _I, _F, _F, _P, _P, _P, _SZ, _P],
     ),
+    "oi_grpo_stats_from_terms": (_I, [_P] * 12 + [_I64, _I64, _I, _F, _P, _I64, c_uint32, _P, _SZ, _P]),
+    "oi_scale_by_device_scalar": (_I, [_P, _I, _I64, _P, _P]),
     "oi_grpo_fused_bwd": (_I, [_P, _P, _P, _P, _P, _P, _I64, _I64, _I, _F, _F, _I, _F, _F, _P, _P, _P, _P]),
     "oi_estimate_kl_fwd": (_I, [_P, _P, _I64, _P, _P]),
     "oi_estimate_kl_bwd": (_I, [_P, _P, _P, _I64, _P, _P, _P]),

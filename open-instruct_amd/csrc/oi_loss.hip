@@ -37,29 +37,48 @@ __global__ void grpo_terms_bwd_kernel(const float* __restrict__ nlp, const float
 constexpr int FUSED_THREADS = 256;
 constexpr int FUSED_PER_THREAD = 4;
 constexpr int FUSED_CHUNK = FUSED_THREADS * FUSED_PER_THREAD;
-constexpr int NQ = OI_GRPO_NUM_STATS;  // partial sums kept per (row, chunk)
+constexpr int NSUM = 15;  // partial sums kept per (row, chunk): entries 0..14 of the statistics vector
+static_assert(NSUM + 1 == OI_GRPO_NUM_STATS, "the last statistic is derived from the sums");
+
+// Per-token inputs of the statistics pass.  Two ways to obtain the loss terms of a token:
+//   from the logprobs (pg == nullptr): ratio = exp(new - old), terms by grpo_token_fwd;
+//   from tensors the caller already holds (pg != nullptr): pg, clipfrac and ratio are read, the
+//   four KL estimators are evaluated from new - ref and ratio.
+// The remaining pointers are optional tensors that are only averaged over the mask.
+struct StatIn {
+    const float *nlp, *old, *ref, *adv, *rho;
+    const float *pg, *clipfrac, *ratio;
+    const float *ent, *drop_any, *drop_low, *drop_high, *rho_clipped;
+    const uint8_t* mask;
+};
 
 __global__ void __launch_bounds__(FUSED_THREADS)
-    grpo_fused_partial_kernel(const float* __restrict__ nlp, const float* __restrict__ old,
-                              const float* __restrict__ ref, const float* __restrict__ adv,
-                              const uint8_t* __restrict__ mask, const float* __restrict__ rho,
-                              const float* __restrict__ ent, int64_t cols, GrpoCfg c, float beta,
+    grpo_stats_partial_kernel(StatIn in, int64_t cols, int64_t nchunks, GrpoCfg c, float beta,
                               float* __restrict__ partial) {
-    const int64_t row = blockIdx.y, chunk = blockIdx.x, nchunks = gridDim.x;
-    float acc[NQ];
+    const int64_t row = blockIdx.x / nchunks, chunk = blockIdx.x - row * nchunks;
+    float acc[NSUM];
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) acc[q] = 0.f;
+    for (int q = 0; q < NSUM; ++q) acc[q] = 0.f;
     const int64_t base = row * cols;
 #pragma unroll
     for (int k = 0; k < FUSED_PER_THREAD; ++k) {
         const int64_t col = chunk * FUSED_CHUNK + (int64_t)k * FUSED_THREADS + threadIdx.x;
         if (col < cols) {
             const int64_t i = base + col;
-            const float x = nlp[i];
-            const float ratio = old ? expf(x - old[i]) : 1.f;
-            const float w = rho ? rho[i] : 1.f;
-            const GrpoOut o = grpo_token_fwd(x, ratio, adv[i], ref != nullptr, ref ? ref[i] : 0.f, w, c);
-            const float mf = mask[i] ? 1.f : 0.f;
+            const float x = in.nlp ? in.nlp[i] : 0.f;
+            const float w = in.rho ? in.rho[i] : 1.f;
+            GrpoOut o;
+            float ratio;
+            if (in.pg) {
+                ratio = in.ratio[i];
+                o = grpo_token_fwd(x, ratio, 0.f, in.ref != nullptr, in.ref ? in.ref[i] : 0.f, 1.f, c);
+                o.pg = in.pg[i];
+                o.clipfrac = in.clipfrac[i];
+            } else {
+                ratio = in.old ? expf(x - in.old[i]) : 1.f;
+                o = grpo_token_fwd(x, ratio, in.adv[i], in.ref != nullptr, in.ref ? in.ref[i] : 0.f, w, c);
+            }
+            const float mf = in.mask[i] ? 1.f : 0.f;
             acc[0] += (o.pg + beta * o.kl[c.kl_est]) * mf;
             acc[1] += o.pg * mf;
             acc[2] += o.kl[0] * mf;
@@ -68,16 +87,29 @@ __global__ void __launch_bounds__(FUSED_THREADS)
             acc[5] += o.kl[3] * mf;
             acc[6] += o.clipfrac * mf;
             acc[7] += ratio * mf;
-            acc[8] += ent ? ent[i] * mf : 0.f;
+            acc[8] += in.ent ? in.ent[i] * mf : 0.f;
             acc[9] += mf;
+            acc[10] += in.drop_any ? in.drop_any[i] * mf : 0.f;
+            acc[11] += in.drop_low ? in.drop_low[i] * mf : 0.f;
+            acc[12] += in.drop_high ? in.drop_high[i] * mf : 0.f;
+            acc[13] += w * mf;
+            acc[14] += in.rho_clipped ? in.rho_clipped[i] * mf : 0.f;
         }
     }
-    __shared__ float scratch[16];
-    float* out = partial + (row * nchunks + chunk) * NQ;
+    // wave sums first, then one pass over the four waves: fixed order, one barrier
+    __shared__ float wave_sums[FUSED_THREADS / OI_WAVE][NSUM];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-        const float t = oi_block_sum(acc[q], scratch);
-        if (threadIdx.x == 0) out[q] = t;
+    for (int q = 0; q < NSUM; ++q) {
+        const float t = oi_wave_sum(acc[q]);
+        if (lane == 0) wave_sums[wave][q] = t;
+    }
+    __syncthreads();
+    if (threadIdx.x < NSUM) {
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < FUSED_THREADS / OI_WAVE; ++w) t += wave_sums[w][threadIdx.x];
+        partial[(size_t)blockIdx.x * NSUM + threadIdx.x] = t;
     }
 }
 
@@ -93,45 +125,52 @@ __device__ __forceinline__ double block_sum_f64(double v, double* scratch) {
 }
 
 // One workgroup: per-row totals in fp64 in chunk order, then the loss and the statistics.
+// Statistic q goes to out_stats[q * out_stride] when bit q of write_mask is set.
 __global__ void __launch_bounds__(256)
-    grpo_fused_final_kernel(const float* __restrict__ partial, int64_t rows, int64_t nchunks, int axis_mode,
-                            float denominator, float scale, float* __restrict__ out_stats,
-                            float* __restrict__ row_denoms) {
+    grpo_stats_final_kernel(const float* __restrict__ partial, int64_t rows, int64_t nchunks, int axis_mode,
+                            float denominator, float scale, float beta, int kl_est, float* __restrict__ out_stats,
+                            int64_t out_stride, uint32_t write_mask, float* __restrict__ row_denoms) {
     __shared__ double scratch[4];
-    double tot[NQ];
-    for (int q = 0; q < NQ; ++q) tot[q] = 0.0;
+    double tot[NSUM];
+    for (int q = 0; q < NSUM; ++q) tot[q] = 0.0;
     double row_mean_sum = 0.0;
     // pass 1: totals, and for axis_mode 1 the per-row means and reciprocal denominators
     for (int64_t r = threadIdx.x; r < rows; r += blockDim.x) {
-        double rt[NQ];
-        for (int q = 0; q < NQ; ++q) rt[q] = 0.0;
+        double rt[NSUM];
+        for (int q = 0; q < NSUM; ++q) rt[q] = 0.0;
         for (int64_t ch = 0; ch < nchunks; ++ch) {
-            const float* p = partial + (r * nchunks + ch) * NQ;
-            for (int q = 0; q < NQ; ++q) rt[q] += (double)p[q];
+            const float* p = partial + (r * nchunks + ch) * NSUM;
+            for (int q = 0; q < NSUM; ++q) rt[q] += (double)p[q];
         }
-        for (int q = 0; q < NQ; ++q) tot[q] += rt[q];
+        for (int q = 0; q < NSUM; ++q) tot[q] += rt[q];
         if (axis_mode == 1) {
             const double den = denominator > 0.f ? (double)denominator : rt[9];
             const double inv = den > 0.0 ? 1.0 / den : 0.0;
             row_mean_sum += rt[0] * inv;
-            row_denoms[r] = (float)(inv / (double)rows);
+            if (row_denoms) row_denoms[r] = (float)(inv / (double)rows);
         }
     }
-    double all[NQ];
-    for (int q = 0; q < NQ; ++q) all[q] = block_sum_f64(tot[q], scratch);
+    double all[NSUM];
+    for (int q = 0; q < NSUM; ++q) all[q] = block_sum_f64(tot[q], scratch);
     const double rms = block_sum_f64(row_mean_sum, scratch);
     double inv_global = 0.0;
     if (axis_mode == 0) {
         const double den = denominator > 0.f ? (double)denominator : all[9];
         inv_global = den > 0.0 ? 1.0 / den : 0.0;
-        for (int64_t r = threadIdx.x; r < rows; r += blockDim.x) row_denoms[r] = (float)inv_global;
+        if (row_denoms)
+            for (int64_t r = threadIdx.x; r < rows; r += blockDim.x) row_denoms[r] = (float)inv_global;
     }
     if (threadIdx.x == 0) {
+        float st[OI_GRPO_NUM_STATS];
         const double loss = axis_mode == 0 ? all[0] * inv_global : rms / (double)rows;
-        out_stats[0] = (float)(loss * (double)scale);
+        st[0] = (float)(loss * (double)scale);
         const double invc = all[9] > 0.0 ? 1.0 / all[9] : 0.0;
-        for (int q = 1; q < 9; ++q) out_stats[q] = (float)(all[q] * invc);
-        out_stats[9] = (float)all[9];
+        for (int q = 1; q < NSUM; ++q) st[q] = (float)(all[q] * invc);
+        st[9] = (float)all[9];
+        // the KL share of the loss, rounded as the caller's fp32 product of the mean and beta
+        st[15] = st[2 + kl_est] * beta;
+        for (int q = 0; q < OI_GRPO_NUM_STATS; ++q)
+            if ((write_mask >> q) & 1u) out_stats[q * out_stride] = st[q];
     }
 }
 
@@ -184,8 +223,10 @@ __device__ __forceinline__ float mask_at(const void* mask, int is_float, int64_t
 // partial[(e * rows + r) * nchunks + ch] = sum values*mask ; cnt[r * nchunks + ch] = sum mask
 __global__ void __launch_bounds__(FUSED_THREADS)
     masked_partial_kernel(const float* __restrict__ values, const void* __restrict__ mask, int mask_is_float,
-                          int64_t rows, int64_t cols, float* __restrict__ partial, float* __restrict__ cnt) {
-    const int64_t chunk = blockIdx.x, nchunks = gridDim.x, row = blockIdx.y, e = blockIdx.z;
+                          int64_t rows, int64_t cols, int64_t nchunks, float* __restrict__ partial,
+                          float* __restrict__ cnt) {
+    // one block per (extra, row, chunk)
+    const int64_t chunk = blockIdx.x % nchunks, er = blockIdx.x / nchunks, row = er % rows, e = er / rows;
     float num = 0.f, c = 0.f;
 #pragma unroll
     for (int k = 0; k < FUSED_PER_THREAD; ++k) {
@@ -543,31 +584,71 @@ extern "C" int oi_grpo_terms_bwd(const float* new_logprobs, const float* ratio, 
 extern "C" size_t oi_grpo_fused_workspace_bytes(int64_t rows, int64_t cols) {
     if (rows <= 0 || cols <= 0) return 0;
     const int64_t nchunks = (cols + FUSED_CHUNK - 1) / FUSED_CHUNK;
-    return (size_t)(rows * nchunks * NQ) * sizeof(float);
+    return (size_t)(rows * nchunks * NSUM) * sizeof(float);
 }
+
+namespace {
+// Shared launch sequence of the statistics entry points: one block per (row, chunk), then one
+// workgroup that adds the partial sums up in a fixed order.
+int launch_grpo_stats(const StatIn& in, int64_t rows, int64_t cols, const GrpoCfg& c, float beta, int axis_mode,
+                      float denominator, float scale, float* out_stats, int64_t out_stride, uint32_t write_mask,
+                      float* row_denoms, float* partial, hipStream_t s) {
+    const int64_t nchunks = (cols + FUSED_CHUNK - 1) / FUSED_CHUNK;
+    hipLaunchKernelGGL(grpo_stats_partial_kernel, dim3((unsigned)(rows * nchunks)), dim3(FUSED_THREADS), 0, s, in,
+                       cols, nchunks, c, beta, partial);
+    hipLaunchKernelGGL(grpo_stats_final_kernel, dim3(1), dim3(256), 0, s, partial, rows, nchunks, axis_mode,
+                       denominator, scale, beta, c.kl_est, out_stats, out_stride, write_mask, row_denoms);
+    return oi_launch_status();
+}
+
+int check_stats_shape(int64_t rows, int64_t cols) {
+    OI_RETURN_IF(rows <= 0 || cols <= 0, OI_EINVAL);
+    const int64_t nchunks = (cols + FUSED_CHUNK - 1) / FUSED_CHUNK;
+    OI_RETURN_IF(rows > 0x7fffffffLL / nchunks, OI_EINVAL);  // one block per (row, chunk)
+    return OI_OK;
+}
+}  // namespace
 
 extern "C" int oi_grpo_fused_fwd(const float* new_logprobs, const float* old_logprobs, const float* ref_logprobs,
                                  const float* advantages, const uint8_t* mask, const float* rho_weights,
-                                 const float* entropy, int64_t rows, int64_t cols, int loss_fn, float ratio_lo,
-                                 float ratio_hi, int kl_estimator, float beta, int axis_mode, float denominator,
-                                 float scale, float* out_stats, float* row_denoms, void* workspace,
-                                 size_t workspace_bytes, void* stream) {
-    OI_RETURN_IF(rows <= 0 || cols <= 0 || rows > 65535, OI_EINVAL);
+                                 const float* entropy, const float* rho_drop_any, const float* rho_drop_low,
+                                 const float* rho_drop_high, const float* rho_clipped, int64_t rows, int64_t cols,
+                                 int loss_fn, float ratio_lo, float ratio_hi, int kl_estimator, float beta,
+                                 int axis_mode, float denominator, float scale, float* out_stats, float* row_denoms,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_stats_shape(rows, cols);
+    if (rc != OI_OK) return rc;
     OI_RETURN_IF(axis_mode != 0 && axis_mode != 1, OI_EINVAL);
-    const int rc = check_cfg(loss_fn, kl_estimator);
+    rc = check_cfg(loss_fn, kl_estimator);
     if (rc != OI_OK) return rc;
     OI_RETURN_IF(!new_logprobs || !advantages || !mask || !out_stats || !row_denoms || !workspace, OI_ENULL);
     OI_RETURN_IF(workspace_bytes < oi_grpo_fused_workspace_bytes(rows, cols), OI_EWORKSPACE);
     const GrpoCfg c = {loss_fn, ratio_lo, ratio_hi, kl_estimator};
-    const int64_t nchunks = (cols + FUSED_CHUNK - 1) / FUSED_CHUNK;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    float* partial = static_cast<float*>(workspace);
-    hipLaunchKernelGGL(grpo_fused_partial_kernel, dim3((unsigned)nchunks, (unsigned)rows), dim3(FUSED_THREADS), 0, s,
-                       new_logprobs, old_logprobs, ref_logprobs, advantages, mask, rho_weights, entropy, cols, c, beta,
-                       partial);
-    hipLaunchKernelGGL(grpo_fused_final_kernel, dim3(1), dim3(256), 0, s, partial, rows, nchunks, axis_mode,
-                       denominator, scale, out_stats, row_denoms);
-    return oi_launch_status();
+    const StatIn in = {new_logprobs, old_logprobs, ref_logprobs, advantages, rho_weights, nullptr, nullptr,
+                       nullptr,      entropy,      rho_drop_any, rho_drop_low, rho_drop_high, rho_clipped, mask};
+    return launch_grpo_stats(in, rows, cols, c, beta, axis_mode, denominator, scale, out_stats, 1, 0xffffu, row_denoms,
+                             static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
+}
+
+extern "C" int oi_grpo_stats_from_terms(const float* pg_loss, const float* clipfrac, const float* ratio,
+                                        const float* new_logprobs, const float* ref_logprobs, const uint8_t* mask,
+                                        const float* entropy, const float* rho_weight, const float* rho_drop_any,
+                                        const float* rho_drop_low, const float* rho_drop_high,
+                                        const float* rho_clipped, int64_t rows, int64_t cols, int kl_estimator,
+                                        float beta, float* out_stats, int64_t out_stride, uint32_t write_mask,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_stats_shape(rows, cols);
+    if (rc != OI_OK) return rc;
+    OI_RETURN_IF(kl_estimator < 0 || kl_estimator > 3 || out_stride < 1, OI_EINVAL);
+    OI_RETURN_IF(!pg_loss || !clipfrac || !ratio || !mask || !out_stats || !workspace, OI_ENULL);
+    OI_RETURN_IF(ref_logprobs && !new_logprobs, OI_ENULL);
+    OI_RETURN_IF(workspace_bytes < oi_grpo_fused_workspace_bytes(rows, cols), OI_EWORKSPACE);
+    const GrpoCfg c = {OI_LOSS_DAPO, 0.f, 0.f, kl_estimator};
+    const StatIn in = {new_logprobs, nullptr, ref_logprobs, nullptr,      rho_weight,   pg_loss,       clipfrac,
+                       ratio,        entropy, rho_drop_any, rho_drop_low, rho_drop_high, rho_clipped, mask};
+    // the loss itself belongs to the caller here: entry 0 is never written
+    return launch_grpo_stats(in, rows, cols, c, beta, 0, 0.f, 1.f, out_stats, out_stride, write_mask & 0xfffeu,
+                             nullptr, static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
 }
 
 extern "C" int oi_grpo_fused_bwd(const float* new_logprobs, const float* old_logprobs, const float* ref_logprobs,
@@ -605,16 +686,17 @@ extern "C" size_t oi_masked_mean_workspace_bytes(int64_t extra, int64_t rows, in
 extern "C" int oi_masked_mean_fwd(const float* values, const void* mask, int mask_is_float, int64_t extra,
                                   int64_t rows, int64_t cols, int axis_mode, float denominator, float* out,
                                   float* row_denoms, void* workspace, size_t workspace_bytes, void* stream) {
-    OI_RETURN_IF(extra <= 0 || rows <= 0 || cols <= 0 || rows > 65535 || extra > 65535, OI_EINVAL);
+    OI_RETURN_IF(extra <= 0 || rows <= 0 || cols <= 0 || extra > 65535, OI_EINVAL);
     OI_RETURN_IF(axis_mode != 0 && axis_mode != 1, OI_EINVAL);
     OI_RETURN_IF(!values || !mask || !out || !workspace, OI_ENULL);
     OI_RETURN_IF(workspace_bytes < oi_masked_mean_workspace_bytes(extra, rows, cols), OI_EWORKSPACE);
     const int64_t nchunks = (cols + FUSED_CHUNK - 1) / FUSED_CHUNK;
+    OI_RETURN_IF(rows > 0x7fffffffLL / nchunks / extra, OI_EINVAL);  // one block per (extra, row, chunk)
     float* partial = static_cast<float*>(workspace);
     float* cnt = partial + extra * rows * nchunks;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(masked_partial_kernel, dim3((unsigned)nchunks, (unsigned)rows, (unsigned)extra),
-                       dim3(FUSED_THREADS), 0, s, values, mask, mask_is_float, rows, cols, partial, cnt);
+    hipLaunchKernelGGL(masked_partial_kernel, dim3((unsigned)(extra * rows * nchunks)), dim3(FUSED_THREADS), 0, s,
+                       values, mask, mask_is_float, rows, cols, nchunks, partial, cnt);
     hipLaunchKernelGGL(masked_final_kernel, dim3((unsigned)extra), dim3(256), 0, s, partial, cnt, rows, nchunks,
                        axis_mode, denominator, out, row_denoms);
     return oi_launch_status();
@@ -745,7 +827,7 @@ extern "C" int oi_logprob_diff_stats(const float* local_logprobs, const float* o
     return oi_launch_status();
 }
 
-extern "C" int oi_version(void) { return 1002; }
+extern "C" int oi_version(void) { return 1100; }
 
 extern "C" const char* oi_error_string(int code) {
     switch (code) {

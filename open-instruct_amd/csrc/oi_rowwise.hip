@@ -613,6 +613,40 @@ int launch_grpo_fused(const void* logits, int64_t rows, int64_t n_inner, int64_t
     return oi_launch_status();
 }
 
+// data[i] *= *scale for a contiguous tensor, skipped altogether when the device scalar is exactly 1
+// (the upstream gradient of a loss that is differentiated directly): every workgroup reads the
+// scalar and leaves, so the host never has to look at it.
+template <typename R>
+__global__ void __launch_bounds__(256) scale_by_scalar_kernel(typename R::elem_t* __restrict__ data, int64_t n,
+                                                              bool vectorised, const float* __restrict__ scale) {
+    const float s = *scale;
+    if (s == 1.f) return;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x, first = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (vectorised) {
+        for (int64_t v = first; v < n / R::VEC; v += stride) {
+            float z[R::VEC];
+            R::load_vec(data + v * R::VEC, z);
+#pragma unroll
+            for (int e = 0; e < R::VEC; ++e) z[e] *= s;
+            R::store_vec(data + v * R::VEC, z);
+        }
+        for (int64_t i = n / R::VEC * R::VEC + first; i < n; i += stride) R::store_one(data + i, R::load_one(data + i) * s);
+    } else {
+        for (int64_t i = first; i < n; i += stride) R::store_one(data + i, R::load_one(data + i) * s);
+    }
+}
+
+template <typename R>
+int launch_scale(void* data, int64_t n, const float* scale, hipStream_t stream) {
+    typedef typename R::elem_t E;
+    const int64_t vecs = (n + R::VEC - 1) / R::VEC;
+    const int64_t want = (vecs + 255) / 256;
+    const unsigned blocks = (unsigned)(want < 1 ? 1 : (want > 16384 ? 16384 : want));
+    hipLaunchKernelGGL((scale_by_scalar_kernel<R>), dim3(blocks), dim3(256), 0, stream, static_cast<E*>(data), n,
+                       oi_aligned(data, 16), scale);
+    return oi_launch_status();
+}
+
 int check_rows(const void* logits, int64_t n_outer, int64_t n_inner, int64_t so, int64_t si, int64_t vocab,
                const int64_t* index, float inv_t, int64_t* rows) {
     OI_RETURN_IF(n_outer < 0 || n_inner < 0 || vocab <= 0, OI_EINVAL);
@@ -700,6 +734,7 @@ extern "C" int oi_lsg_grpo_fwd_bwd(const void* logits, int dtype, int64_t n_oute
     OI_RETURN_IF(kl_estimator < 0 || kl_estimator > 3, OI_EINVAL);
     if (rows == 0) return OI_OK;
     OI_RETURN_IF(!advantages || !token_coef || !logprob || !dlogits, OI_ENULL);
+    OI_RETURN_IF(dlogits == logits, OI_EINVAL);  // a row is read again after its gradient has started to land
     OI_RETURN_IF(out_stride_outer < 0 || out_stride_inner < 0 || (out_stride_inner < vocab && n_inner > 1), OI_EINVAL);
     const GrpoCfg cfg = {loss_fn, ratio_lo, ratio_hi, kl_estimator};
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -719,5 +754,19 @@ extern "C" int oi_lsg_grpo_fwd_bwd(const void* logits, int dtype, int64_t n_oute
                                              inv_temperature, old_logprobs, ref_logprobs, advantages, rho_weights,
                                              token_coef, cfg, beta, logprob, entropy, lse, dlogits, out_stride_outer,
                                              out_stride_inner, s);
+    }
+}
+
+extern "C" int oi_scale_by_device_scalar(void* data, int dtype, int64_t n, const float* scale, void* stream) {
+    OI_RETURN_IF(n < 0, OI_EINVAL);
+    OI_RETURN_IF(dtype != OI_DTYPE_F32 && dtype != OI_DTYPE_BF16 && dtype != OI_DTYPE_F16, OI_EDTYPE);
+    if (n == 0) return OI_OK;
+    OI_RETURN_IF(!data || !scale, OI_ENULL);
+    OI_RETURN_IF(!oi_aligned(data, dtype == OI_DTYPE_F32 ? 4 : 2), OI_EALIGN);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case OI_DTYPE_F32: return launch_scale<F32Row>(data, n, scale, s);
+        case OI_DTYPE_BF16: return launch_scale<BF16Row>(data, n, scale, s);
+        default: return launch_scale<F16Row>(data, n, scale, s);
     }
 }

@@ -71,6 +71,16 @@ class RhoCorrection:
     histogram_metrics: dict[str, torch.Tensor] = field(default_factory=dict)
 
 
+def _expand_to(t: torch.Tensor, shape: tuple[int, ...], name: str) -> torch.Tensor:
+    """``t`` broadcast to ``shape`` (a view), ``ValueError`` when it does not broadcast."""
+    if tuple(t.shape) == tuple(shape):
+        return t
+    try:
+        return t.expand(shape)
+    except RuntimeError:
+        raise ValueError(f"{name} of shape {tuple(t.shape)} does not broadcast to {tuple(shape)}") from None
+
+
 def compute_rho_correction(
     old_logprob: torch.Tensor,
     vllm_logprobs: torch.Tensor,
@@ -82,11 +92,15 @@ def compute_rho_correction(
 
     Stop-gradient by construction (the reference's inputs carry no grad either).
     """
+    shape = tuple(old_logprob.shape)
+    # the kernel indexes every side tensor per token: broadcastable inputs are expanded first
+    vllm_logprobs = _expand_to(vllm_logprobs.detach(), shape, "vllm_logprobs")
+    advantages = _expand_to(advantages.detach(), shape, "advantages")
+    response_mask = _expand_to(response_mask, shape, "response_mask")
     dev = _lib.require_gpu(old_logprob, vllm_logprobs, response_mask, advantages)
     with torch.no_grad():
-        old, vl, adv = _lib.f32c(old_logprob.detach()), _lib.f32c(vllm_logprobs.detach()), _lib.f32c(advantages)
+        old, vl, adv = _lib.f32c(old_logprob.detach()), _lib.f32c(vllm_logprobs), _lib.f32c(advantages)
         m = _lib.mask_u8(response_mask)
-        shape = tuple(old.shape)
         cols = shape[-1] if shape else 1
         rows = old.numel() // max(cols, 1)
         bufs = torch.empty((6,) + shape, dtype=torch.float32, device=dev)
@@ -131,16 +145,20 @@ def resolve_old_logprob(
     vllm_logprobs: torch.Tensor,
     new_logprobs: torch.Tensor,
 ) -> torch.Tensor:
-    """Pick the baseline logprobs of a sample; host-side bookkeeping only (open_instruct/grpo_utils.py:475-501)."""
-    if num_mini_batches > 1:
-        result = old_logprobs_cache[sample_idx]
-    else:
-        with torch.no_grad():
-            if epoch_idx == 0:
-                old_logprobs_cache[sample_idx] = vllm_logprobs if use_vllm_logprobs else new_logprobs.detach()
-            result = old_logprobs_cache[sample_idx]
-    assert result is not None
-    return result
+    """Baseline ("old") logprobs of one sample; host bookkeeping of open_instruct/grpo_utils.py:475-501.
+
+    With several mini-batches the cache was filled by a separate no-grad pass and is only read.
+    With a single mini-batch the first epoch's own logprobs (detached), or the sampler's when
+    ``use_vllm_logprobs``, become the baseline of the later epochs, so the first epoch runs at
+    ratio 1.
+    """
+    fills_cache = num_mini_batches <= 1 and epoch_idx == 0
+    if fills_cache:
+        old_logprobs_cache[sample_idx] = vllm_logprobs if use_vllm_logprobs else new_logprobs.detach()
+    baseline = old_logprobs_cache[sample_idx]
+    if baseline is None:
+        raise AssertionError(f"no old logprobs cached for sample {sample_idx}")
+    return baseline
 
 
 # ----------------------------------------------------------------------------------------------
@@ -225,6 +243,7 @@ def compute_grpo_loss(
 # ----------------------------------------------------------------------------------------------
 # fused scalar loss (+ statistics) of one micro-batch
 # ----------------------------------------------------------------------------------------------
+# entry q of the kernels' statistics vector (OI_GRPO_NUM_STATS entries)
 GRPO_STAT_NAMES = (
     "loss/total_avg",
     "loss/policy_avg",
@@ -236,12 +255,33 @@ GRPO_STAT_NAMES = (
     "val/ratio",
     "policy/entropy_avg",
     "num_response_tokens",
+    "val/rho_drop_frac",
+    "val/rho_drop_low_frac",
+    "val/rho_drop_high_frac",
+    "val/rho_weight",
+    "val/rho_clipfrac",
+    "loss/kl_avg",
 )
+_STAT_ROW = {name: i for i, name in enumerate(GRPO_STAT_NAMES)}
+# per-token indicator tensors of compute_rho_correction that the statistics kernels only average
+_RHO_INDICATOR_KEYS = ("val/rho_drop_frac", "val/rho_drop_low_frac", "val/rho_drop_high_frac", "val/rho_clipfrac")
+
+
+def _rho_indicator_ptrs(rho_metrics: dict[str, torch.Tensor] | None, shape) -> tuple[list, list]:
+    """Device pointers (or None) of the four indicator tensors in the kernels' argument order, and the
+    tensors that must stay alive for the duration of the call."""
+    if not rho_metrics:
+        return [None] * 4, []
+    keep = [
+        _lib.f32c(_expand_to(rho_metrics[k].detach(), shape, k)) if k in rho_metrics else None
+        for k in _RHO_INDICATOR_KEYS
+    ]
+    return [_lib.ptr(t) for t in keep], keep
 
 
 class _GrpoFused(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, new_logprobs, old, ref, adv, mask, rho, entropy, cfg):
+    def forward(ctx, new_logprobs, old, ref, adv, mask, rho, entropy, cfg, rho_metrics=None):
         dev = _lib.require_gpu(new_logprobs, old, ref, adv, mask, rho, entropy)
         loss_fn, lo, hi, kl_estimator, beta, axis_mode, denominator, scale = cfg
         nl = _lib.f32c(new_logprobs)
@@ -255,10 +295,11 @@ class _GrpoFused(torch.autograd.Function):
         row_denoms = torch.empty(rows, dtype=torch.float32, device=dev)
         ws_bytes = _lib.load().oi_grpo_fused_workspace_bytes(rows, cols)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        rho_ptrs, _alive = _rho_indicator_ptrs(rho_metrics, (rows, cols))
         _lib.call(
             "oi_grpo_fused_fwd", nl.data_ptr(), _lib.ptr(old_c), _lib.ptr(ref_c), adv_c.data_ptr(), m.data_ptr(),
-            _lib.ptr(rho_c), _lib.ptr(ent_c), rows, cols, loss_fn, lo, hi, kl_estimator, beta, axis_mode, denominator,
-            scale, stats.data_ptr(), row_denoms.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(nl),
+            _lib.ptr(rho_c), _lib.ptr(ent_c), *rho_ptrs, rows, cols, loss_fn, lo, hi, kl_estimator, beta, axis_mode,
+            denominator, scale, stats.data_ptr(), row_denoms.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(nl),
         )  # fmt: skip
         ctx.save_for_backward(nl, old_c, ref_c, adv_c, m, rho_c, row_denoms)
         ctx.cfg = cfg
@@ -279,7 +320,7 @@ class _GrpoFused(torch.autograd.Function):
             _lib.ptr(rho_c), rows, cols, loss_fn, lo, hi, kl_estimator, beta, scale, row_denoms.data_ptr(),
             g.data_ptr(), d_new.data_ptr(), _lib.stream_of(nl),
         )  # fmt: skip
-        return d_new.to(ctx.in_dtype), None, None, None, None, None, None, None
+        return d_new.to(ctx.in_dtype), None, None, None, None, None, None, None, None
 
 
 def grpo_loss_fused(
@@ -294,6 +335,7 @@ def grpo_loss_fused(
     loss_denominator: float | None = None,
     axis: int | None = None,
     dp_scale: float = 1.0,
+    rho_metrics: dict[str, torch.Tensor] | None = None,
 ) -> tuple[torch.Tensor, dict[str, torch.Tensor]]:
     """Scalar GRPO loss of a ``[B, T]`` micro-batch and its statistics in two launches.
 
@@ -303,8 +345,10 @@ def grpo_loss_fused(
     ``populate_sample_loss_stats`` records (open_instruct/grpo_utils.py:699-729).
     ``old_logprobs=None`` means ``old = new.detach()`` (ratio 1 with a live gradient).
     Differentiable with respect to ``new_logprobs`` only; ``old``/``ref``/``advantages``/``rho`` are
-    constants, as in the reference.  Returns ``(loss, stats)`` with ``stats`` keyed by
-    ``GRPO_STAT_NAMES`` (0-dim views of one device vector, no host sync).
+    constants, as in the reference.  ``rho_metrics`` (the ``metrics`` of
+    :func:`compute_rho_correction`) adds the masked means of the rho indicators to the same pass.
+    Returns ``(loss, stats)`` with ``stats`` keyed by ``GRPO_STAT_NAMES`` (0-dim views of one device
+    vector, no host sync); ``populate_sample_loss_stats(..., fused_stats=stats)`` records them.
     """
     if axis not in (None, 1, -1):
         raise ValueError("axis must be None or the token axis (1)")
@@ -318,9 +362,18 @@ def grpo_loss_fused(
     detach = lambda t: None if t is None else t.detach()  # noqa: E731
     loss, stats = _GrpoFused.apply(
         new_logprobs, detach(old_logprobs), detach(ref_logprobs), advantages.detach(), response_mask,
-        detach(rho_weights), detach(entropy), cfg,
+        detach(rho_weights), detach(entropy), cfg, rho_metrics,
     )  # fmt: skip
-    return loss, {name: stats[i] for i, name in enumerate(GRPO_STAT_NAMES)}
+    return loss, _StatsView(stats)
+
+
+class _StatsView(dict):
+    """The statistics of one micro-batch keyed by ``GRPO_STAT_NAMES``; ``vector`` is the device
+    vector the 0-dim entries are views of."""
+
+    def __init__(self, vector: torch.Tensor):
+        super().__init__((name, vector[i]) for i, name in enumerate(GRPO_STAT_NAMES))
+        self.vector = vector
 
 
 # ----------------------------------------------------------------------------------------------
@@ -375,15 +428,23 @@ class _AttachLogitsGrad(torch.autograd.Function):
     @staticmethod
     def forward(ctx, loss, logits, dlogits):
         ctx.save_for_backward(dlogits)
+        ctx.handed_out = False
         return loss.clone()
 
     @staticmethod
     def backward(ctx, grad_loss):
         (dlogits,) = ctx.saved_tensors
-        # the usual upstream gradient of a loss is exactly 1: then the stored tensor is the answer
-        # as it is; anything else costs one more pass over it (and one host synchronisation here)
-        if float(grad_loss) != 1.0:
-            dlogits = dlogits * grad_loss.to(dlogits.dtype)
+        if ctx.handed_out:  # a second backward over a retained graph must not scale the same memory twice
+            dlogits = dlogits.clone()
+        ctx.handed_out = True
+        # The usual upstream gradient of a loss is exactly 1 and the stored tensor is the answer as it
+        # is.  The kernel reads the device scalar and returns at once in that case; anything else is
+        # applied in place.  The host never looks at the value.
+        g = _lib.f32c(grad_loss.detach()).reshape(1)
+        _lib.call(
+            "oi_scale_by_device_scalar", dlogits.data_ptr(), _lib.DTYPE_TAGS[dlogits.dtype], dlogits.numel(),
+            g.data_ptr(), _lib.stream_of(dlogits),
+        )  # fmt: skip
         return None, dlogits, None
 
 
@@ -412,9 +473,11 @@ def grpo_loss_on_logits(
     forward call and stored (one tensor of the logits' shape and dtype, which the backward pass
     would allocate anyway).  ``logits`` is ``[B, T, V]`` (``[B, T + 1, V]`` with ``drop_last``),
     ``labels`` and the side tensors ``[B, T]``.  ``old_logprobs=None`` means ``old =
-    new.detach()``.  ``logprobs`` and ``entropy`` are returned detached, for logging.  Rows that do
-    not fit the single-pass kernel (vocabulary not a multiple of the 16-byte vector, more than
-    16384 vectors, unaligned views) go through the two-pass kernels with identical results.
+    new.detach()``.  ``logprobs`` and ``entropy`` are returned detached, for logging.  Side tensors
+    may be anything that broadcasts to ``labels.shape`` (``[B, 1]`` advantages, a 0-dim weight).
+    Rows that do not fit the single-pass kernel (vocabulary not a multiple of the 16-byte vector,
+    unaligned views), and calls that need no gradient (``torch.no_grad()``, logits without
+    ``requires_grad``), go through the two-pass kernels with identical results.
     """
     if axis not in (None, 1, -1):
         raise ValueError("axis must be None or the token axis (1)")
@@ -427,7 +490,8 @@ def grpo_loss_on_logits(
     if tuple(view.shape[:-1]) != tuple(labels.shape):
         raise ValueError(f"labels {tuple(labels.shape)} do not match logits rows {tuple(view.shape[:-1])}")
     layout_view, _, _, so, si = model_utils._row_layout(view)
-    if not logits.requires_grad or not _single_pass_ok(layout_view, so, si) or logits.dtype not in _lib.DTYPE_TAGS:
+    wants_grad = torch.is_grad_enabled() and logits.requires_grad
+    if not wants_grad or not _single_pass_ok(layout_view, so, si) or logits.dtype not in _lib.DTYPE_TAGS:
         logprob, entropy = model_utils.logprob_and_entropy(logits, labels, temperature=temperature, drop_last=drop_last)
         loss, stats = grpo_loss_fused(
             logprob, old_logprobs, ref_logprobs, advantages, response_mask, config, rho_weights=rho_weights,
@@ -438,11 +502,14 @@ def grpo_loss_on_logits(
     cfg = (_loss_fn_tag(config), lo, hi, int(config.kl_estimator), float(config.beta))
     mask = response_mask if response_mask.dtype == torch.bool else response_mask != 0
     coef = _token_coef(mask, None if axis is None else 1, loss_denominator, dp_scale).contiguous()
-    f32 = lambda t: None if t is None else _lib.f32c(t.detach())  # noqa: E731
+    shape = tuple(labels.shape)
+    # the kernel indexes every side tensor per token: broadcastable inputs are expanded first
+    f32 = lambda t, name: None if t is None else _lib.f32c(_expand_to(t.detach(), shape, name))  # noqa: E731
     with torch.no_grad():
         logprob, entropy, dlogits = _grpo_on_logits_launch(
-            logits.detach(), labels.long().contiguous(), f32(old_logprobs), f32(ref_logprobs), f32(advantages),
-            f32(rho_weights), coef, inv_t, cfg, drop_last,
+            logits.detach(), labels.long().contiguous(), f32(old_logprobs, "old_logprobs"),
+            f32(ref_logprobs, "ref_logprobs"), f32(advantages, "advantages"), f32(rho_weights, "rho_weights"), coef,
+            inv_t, cfg, drop_last,
         )  # fmt: skip
         loss, stats = grpo_loss_fused(
             logprob, old_logprobs, ref_logprobs, advantages, response_mask, config, rho_weights=rho_weights,
@@ -603,6 +670,7 @@ def calculate_token_counts(
 # ----------------------------------------------------------------------------------------------
 # loss statistics (open_instruct/grpo_utils.py:674-742)
 # ----------------------------------------------------------------------------------------------
+# the keys the reference's training loops read back (open_instruct/grpo_utils.py:674-689)
 _SCALAR_LOSS_STAT_KEYS = [
     "loss/kl_avg",
     "loss/policy_avg",
@@ -619,21 +687,65 @@ _SCALAR_LOSS_STAT_KEYS = [
     "val/rho_drop_low_frac",
     "val/rho_drop_high_frac",
 ]
+_KL_ROWS = [_STAT_ROW[f"objective/kl{j}_avg"] for j in range(4)] + [_STAT_ROW["loss/kl_avg"]]
+_RHO_ROWS = [_STAT_ROW[k] for k in _RHO_INDICATOR_KEYS] + [_STAT_ROW["val/rho_weight"]]
+_ALWAYS_ROWS = [_STAT_ROW[k] for k in ("loss/policy_avg", "policy/clipfrac_avg", "val/ratio")]
+
+
+class LossStats(dict):
+    """Per-sample loss statistics: the reference's ``dict[key -> tensor[num_samples]]`` whose entries
+    are the rows of ONE ``[len(GRPO_STAT_NAMES), num_samples]`` device table (``self.table``), laid
+    out like the statistics vector of the kernels.  A sample's column is then filled by the
+    kernel itself, and the epoch summary is one reduction over the table."""
+
+    def __init__(self, num_samples: int, device, record_entropy: bool):
+        self.table = torch.zeros(len(GRPO_STAT_NAMES), num_samples, dtype=torch.float32, device=device)
+        keys = list(_SCALAR_LOSS_STAT_KEYS) + (["policy/entropy_avg"] if record_entropy else [])
+        super().__init__((key, self.table[_STAT_ROW[key]]) for key in keys)
+
+    def is_intact(self) -> bool:
+        """True while every entry is still the table row it was created as."""
+        base = self.table.data_ptr()
+        width = self.table.shape[1]
+        return all(
+            key in _STAT_ROW and t.data_ptr() == base + 4 * width * _STAT_ROW[key] and t.shape == (width,)
+            for key, t in self.items()
+        )
 
 
 def create_loss_stats(num_samples: int, device: torch.device, record_entropy: bool = False) -> dict[str, torch.Tensor]:
-    stats = {key: torch.zeros(num_samples, device=device) for key in _SCALAR_LOSS_STAT_KEYS}
-    if record_entropy:
-        stats["policy/entropy_avg"] = torch.zeros(num_samples, device=device)
-    return stats
+    """Zeroed per-sample statistics with the keys of open_instruct/grpo_utils.py:692-696."""
+    return LossStats(num_samples, device, record_entropy)
+
+
+_ROW_SELECTORS: dict[tuple, torch.Tensor] = {}
+
+
+def _row_selector(rows: tuple[int, ...], device) -> torch.Tensor:
+    """Index tensor of the table rows to record, made once per combination and device."""
+    key = (rows, str(device))
+    if key not in _ROW_SELECTORS:
+        _ROW_SELECTORS[key] = torch.tensor(rows, dtype=torch.int64, device=device)
+    return _ROW_SELECTORS[key]
+
+
+def _rows_to_record(config, ref_logprobs, entropy, rho_metrics) -> list[int]:
+    rows = list(_ALWAYS_ROWS)
+    if config.load_ref_policy and ref_logprobs is not None:
+        rows += _KL_ROWS
+    if rho_metrics is not None:
+        rows += [_STAT_ROW[k] for k in rho_metrics if k in _STAT_ROW]
+    if entropy is not None:
+        rows.append(_STAT_ROW["policy/entropy_avg"])
+    return sorted(set(rows))
 
 
 def populate_sample_loss_stats(
     loss_stats_B: dict[str, torch.Tensor],
     sample_idx: int,
-    pg_loss: torch.Tensor,
-    clipfrac: torch.Tensor,
-    ratio: torch.Tensor,
+    pg_loss: torch.Tensor | None,
+    clipfrac: torch.Tensor | None,
+    ratio: torch.Tensor | None,
     loss: torch.Tensor,
     response_mask: torch.Tensor,
     new_logprobs: torch.Tensor,
@@ -641,34 +753,79 @@ def populate_sample_loss_stats(
     entropy: torch.Tensor | None,
     config,
     rho_metrics: dict[str, torch.Tensor] | None = None,
+    fused_stats: dict | torch.Tensor | None = None,
 ) -> None:
-    """Record the masked means of one sample; open_instruct/grpo_utils.py:699-729."""
+    """Record the masked means of one sample; same arguments and recorded keys as
+    open_instruct/grpo_utils.py:699-729.
+
+    With the per-token tensors (the reference's call) all means come from one pass over them
+    (``oi_grpo_stats_from_terms``), written straight into the sample's column when ``loss_stats_B``
+    is the table made by :func:`create_loss_stats`.  With ``fused_stats`` (the statistics that
+    :func:`grpo_loss_fused` returned for this sample) nothing is recomputed: the entries are
+    copied, and ``pg_loss`` / ``clipfrac`` / ``ratio`` may be None.  No host synchronisation either
+    way.
+    """
+    rows = _rows_to_record(config, ref_logprobs, entropy, rho_metrics)
+    table = loss_stats_B.table if isinstance(loss_stats_B, LossStats) and loss_stats_B.is_intact() else None
     with torch.no_grad():
-        if config.load_ref_policy and ref_logprobs is not None:
-            diff = (new_logprobs - ref_logprobs).clamp(-40.0, 40.0)
-            kl_values = masked_mean(model_utils.estimate_kl(diff, ratio), response_mask).float()
-            for j in range(4):
-                loss_stats_B[f"objective/kl{j}_avg"][sample_idx] = kl_values[j]
-            loss_stats_B["loss/kl_avg"][sample_idx] = kl_values[config.kl_estimator] * config.beta
-        if rho_metrics is not None:
-            for key, value in rho_metrics.items():
-                loss_stats_B[key][sample_idx] = masked_mean(value, response_mask)
-        loss_stats_B["policy/clipfrac_avg"][sample_idx] = masked_mean(clipfrac, response_mask)
-        loss_stats_B["loss/policy_avg"][sample_idx] = masked_mean(pg_loss, response_mask)
-        loss_stats_B["loss/total_avg"][sample_idx] = loss
-        loss_stats_B["val/ratio"][sample_idx] = masked_mean(ratio, response_mask)
-        if entropy is not None:
-            loss_stats_B["policy/entropy_avg"][sample_idx] = masked_mean(entropy, response_mask).float()
+        if fused_stats is not None:
+            vec = getattr(fused_stats, "vector", fused_stats)
+            if isinstance(vec, dict):
+                vec = torch.stack([vec[name].float() for name in GRPO_STAT_NAMES])
+        else:
+            dev = _lib.require_gpu(pg_loss, clipfrac, ratio, response_mask)
+            shape = tuple(pg_loss.shape)
+            cols = shape[-1] if shape else 1
+            n_rows = pg_loss.numel() // max(cols, 1)
+            f32 = lambda t, name: None if t is None else _lib.f32c(_expand_to(t.detach(), shape, name))  # noqa: E731
+            pg_c, cf_c, rt_c = f32(pg_loss, "pg_loss"), f32(clipfrac, "clipfrac"), f32(ratio, "ratio")
+            with_kl = config.load_ref_policy and ref_logprobs is not None
+            nl_c = f32(new_logprobs, "new_logprobs") if with_kl else None
+            ref_c = f32(ref_logprobs, "ref_logprobs") if with_kl else None
+            ent_c = f32(entropy, "entropy")
+            m = _lib.mask_u8(_expand_to(response_mask, shape, "response_mask"))
+            w_c = f32(rho_metrics.get("val/rho_weight"), "val/rho_weight") if rho_metrics else None
+            rho_ptrs, _alive = _rho_indicator_ptrs(rho_metrics, shape)
+            write_mask = sum(1 << r for r in rows)
+            ws_bytes = _lib.load().oi_grpo_fused_workspace_bytes(n_rows, cols)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            if table is not None:
+                out_ptr, out_stride, vec = table.data_ptr() + 4 * sample_idx, table.shape[1], None
+            else:
+                vec = torch.zeros(len(GRPO_STAT_NAMES), dtype=torch.float32, device=dev)
+                out_ptr, out_stride = vec.data_ptr(), 1
+            _lib.call(
+                "oi_grpo_stats_from_terms", pg_c.data_ptr(), cf_c.data_ptr(), rt_c.data_ptr(), _lib.ptr(nl_c),
+                _lib.ptr(ref_c), m.data_ptr(), _lib.ptr(ent_c), _lib.ptr(w_c), *rho_ptrs, n_rows, cols,
+                int(config.kl_estimator), float(config.beta), out_ptr, out_stride, write_mask, ws.data_ptr(), ws_bytes,
+                _lib.stream_of(pg_c),
+            )  # fmt: skip
+        if vec is not None:
+            if table is not None:
+                sel = _row_selector(tuple(rows), table.device)
+                table[:, sample_idx].index_copy_(0, sel, vec.to(table.device).index_select(0, sel))
+            else:
+                for r in rows:
+                    name = GRPO_STAT_NAMES[r]
+                    if name in loss_stats_B:
+                        loss_stats_B[name][sample_idx] = vec[r]
+        loss_stats_B["loss/total_avg"][sample_idx] = loss.detach() if torch.is_tensor(loss) else loss
 
 
 def compute_metrics_from_loss_stats(
     loss_stats_B: dict[str, torch.Tensor], token_counts: torch.Tensor
 ) -> dict[str, float]:
-    """Token-weighted averages over samples + ratio variance; open_instruct/grpo_utils.py:732-742."""
-    total = token_counts.sum()
-    weights = token_counts / total if total > 0 else torch.zeros_like(token_counts)
-    metrics: dict[str, float] = {}
-    for key, value in loss_stats_B.items():
-        metrics[key] = (value * weights).sum().item()
-    metrics["val/ratio_var"] = (weights * (loss_stats_B["val/ratio"] - metrics["val/ratio"]) ** 2).sum().item()
+    """Token-weighted averages over the samples plus the weighted variance of ``val/ratio``;
+    open_instruct/grpo_utils.py:732-742.  One reduction over the stacked statistics and one
+    device-to-host copy for all keys (the reference reads every key back on its own)."""
+    keys = list(loss_stats_B)
+    counts = token_counts.to(torch.float32)
+    stacked = torch.stack([loss_stats_B[k].to(torch.float32) for k in keys])  # [keys, samples]
+    total = counts.sum()
+    weights = torch.where(total > 0, counts / total.clamp(min=1e-30), torch.zeros_like(counts))
+    means = stacked @ weights
+    spread = (weights * (loss_stats_B["val/ratio"].to(torch.float32) - means[keys.index("val/ratio")]) ** 2).sum()
+    values = torch.cat([means, spread.reshape(1)]).tolist()
+    metrics = dict(zip(keys, values[:-1]))
+    metrics["val/ratio_var"] = values[-1]
     return metrics

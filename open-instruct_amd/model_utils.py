@@ -11,38 +11,50 @@ to the logits' dtype) - pass ``out_dtype=logits.dtype`` to get the reference's d
 
 from __future__ import annotations
 
+import os
 import pathlib
-import tempfile
-from dataclasses import dataclass
 
 import torch
 
 from . import _lib
 
 
-@dataclass
 class TensorCache:
-    """Tensors indexed by dataset index (the reference-logprob cache of DPO); same fields and
-    methods as open_instruct/model_utils.py:92-115."""
+    """Device-resident tables with one row per dataset sample (the reference-logprob cache of DPO).
 
-    tensors: dict[str, torch.Tensor]
+    Same constructor, attribute and methods as open_instruct/model_utils.py:92-115:
+    ``TensorCache(tensors={...})``, ``cache[indices]`` gathers the rows of every table, ``to_disk`` /
+    ``from_disk`` move the whole cache through one ``torch.save`` file (readable by the reference).
+    """
+
+    def __init__(self, tensors: dict[str, torch.Tensor]):
+        self.tensors = dict(tensors)
 
     def __getitem__(self, indices: torch.Tensor) -> dict[str, torch.Tensor]:
-        return {k: v[indices.long()] for k, v in self.tensors.items()}
+        out = {}
+        for name, table in self.tensors.items():
+            idx = indices.to(device=table.device, dtype=torch.int64)
+            out[name] = table.index_select(0, idx.reshape(-1)).reshape(idx.shape + table.shape[1:])
+        return out
+
+    def __eq__(self, other) -> bool:
+        return isinstance(other, TensorCache) and self.tensors.keys() == other.tensors.keys() and all(
+            torch.equal(v, other.tensors[k]) for k, v in self.tensors.items()
+        )
 
     def to_disk(self, path: str | pathlib.Path) -> None:
-        """Write atomically: temporary file in the target directory, then rename."""
-        path = pathlib.Path(path)
-        path.parent.mkdir(parents=True, exist_ok=True)
-        cpu_tensors = {k: v.cpu() for k, v in self.tensors.items()}
-        with tempfile.NamedTemporaryFile(dir=path.parent, delete=False, suffix=".tmp") as tmp:
-            tmp_path = pathlib.Path(tmp.name)
-            torch.save(cpu_tensors, tmp_path)
-        tmp_path.rename(path)
+        """The file appears under its final name only when it is complete (written next to it under
+        a process-private name, then moved over)."""
+        target = pathlib.Path(path)
+        target.parent.mkdir(parents=True, exist_ok=True)
+        partial = target.with_name(f".{target.name}.{os.getpid()}.partial")
+        torch.save({name: table.detach().to("cpu") for name, table in self.tensors.items()}, partial)
+        os.replace(partial, target)
 
     @classmethod
     def from_disk(cls, path: str | pathlib.Path, device: torch.device) -> "TensorCache":
-        return cls(tensors=torch.load(path, weights_only=True, map_location=device))
+        """Tensors only: the file is read with ``weights_only=True``."""
+        return cls(tensors=torch.load(pathlib.Path(path), weights_only=True, map_location=device))
 
 
 def _row_layout(logits: torch.Tensor) -> tuple[torch.Tensor, int, int, int, int]:

@@ -27,6 +27,7 @@ dpo.dpo_loss                   open_instruct/dpo_utils.py:523-563               
 dpo.simpo_loss / dpo.wpo_loss  open_instruct/dpo_utils.py:566-642                     closed forms only (no reference known-answer vector)
 lm_head.lm_head_logprobs       HF nn.Linear lm_head + padding_free_collator.py:10-16  textbook F.linear in fp32/fp64 (the GEMM itself lives in third-party code; no reference vector)
 lm_head.linear_cross_entropy   open_instruct/finetune.py:818-824 (HF ForCausalLMLoss)    transformers.loss.loss_utils.ForCausalLMLoss itself (the third-party routine the reference calls), brute force
+grpo.populate_sample_loss_stats  open_instruct/grpo_utils.py:674-742                   hand-computed table (tests/test_oracle_pins.py): means of three tokens by hand, untouched keys stay 0, weighted mean / variance by hand
 grpo.compute_vllm_local_debug_metrics  open_instruct/grpo_utils.py:345-369             pure-Python math / statistics.stdev brute force; empty and single-token masks
 packing.pack_sequences         open_instruct/rl_utils.py:215-375                      reference known-answer vectors (test_rl_utils.py:125-158), reference test properties (test_rl_utils.py:98-123,299-334)
 packing.broadcast_advantages   open_instruct/data_loader.py:1509-1514                 hand-written example

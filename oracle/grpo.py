@@ -195,3 +195,51 @@ def compute_vllm_local_debug_metrics(
         "debug/vllm_vs_local_logprob_diff_std": float(diff[valid].std() if count > 1 else zero),
         "debug/vllm_local_reverse_kl": float(rkl.sum() / count if count > 0 else zero),
     }
+
+
+LOSS_STAT_KEYS = (
+    "loss/kl_avg", "loss/policy_avg", "loss/total_avg", "objective/kl0_avg", "objective/kl1_avg",
+    "objective/kl2_avg", "objective/kl3_avg", "policy/clipfrac_avg", "val/ratio", "val/rho_clipfrac",
+    "val/rho_weight", "val/rho_drop_frac", "val/rho_drop_low_frac", "val/rho_drop_high_frac",
+)  # fmt: skip
+
+
+def create_loss_stats(num_samples: int, record_entropy: bool = False) -> dict[str, torch.Tensor]:
+    """One zero vector per key; restates open_instruct/grpo_utils.py:674-696."""
+    keys = LOSS_STAT_KEYS + (("policy/entropy_avg",) if record_entropy else ())
+    return {k: torch.zeros(num_samples) for k in keys}
+
+
+def populate_sample_loss_stats(
+    stats, sample_idx, pg_loss, clipfrac, ratio, loss, response_mask, new_logprobs, ref_logprobs, entropy, config,
+    rho_metrics=None,
+) -> None:  # fmt: skip
+    """Masked means of one sample written at ``sample_idx``; restates open_instruct/grpo_utils.py:699-729.
+
+    KL entries only with ``config.load_ref_policy`` and reference logprobs (the four estimators of
+    ``clamp(new - ref, +-40)`` and ``beta`` times the selected one); rho entries only when the
+    metric tensors are given; entropy only when given; the loss is stored as passed."""
+    mm = lambda t: reductions.masked_mean(t, response_mask)  # noqa: E731
+    if config.load_ref_policy and ref_logprobs is not None:
+        kls = mm(logprob.estimate_kl((new_logprobs - ref_logprobs).clamp(-40.0, 40.0), ratio)).float()
+        for j in range(4):
+            stats[f"objective/kl{j}_avg"][sample_idx] = kls[j]
+        stats["loss/kl_avg"][sample_idx] = kls[config.kl_estimator] * config.beta
+    for key, value in (rho_metrics or {}).items():
+        stats[key][sample_idx] = mm(value)
+    stats["policy/clipfrac_avg"][sample_idx] = mm(clipfrac)
+    stats["loss/policy_avg"][sample_idx] = mm(pg_loss)
+    stats["loss/total_avg"][sample_idx] = loss
+    stats["val/ratio"][sample_idx] = mm(ratio)
+    if entropy is not None:
+        stats["policy/entropy_avg"][sample_idx] = mm(entropy).float()
+
+
+def compute_metrics_from_loss_stats(stats: dict[str, torch.Tensor], token_counts: torch.Tensor) -> dict[str, float]:
+    """Token-weighted average of every key over the samples and the weighted variance of
+    ``val/ratio``; restates open_instruct/grpo_utils.py:732-742."""
+    total = token_counts.sum()
+    w = token_counts / total if total > 0 else torch.zeros_like(token_counts)
+    out = {k: float((v * w).sum()) for k, v in stats.items()}
+    out["val/ratio_var"] = float((w * (stats["val/ratio"] - out["val/ratio"]) ** 2).sum())
+    return out

@@ -249,6 +249,64 @@ def test_grpo_loss_fused_empty_mask_is_zero():
     assert loss.item() == 0.0 and (dn.grad == 0).all() and stats["num_response_tokens"].item() == 0.0
 
 
+@pytest.mark.parametrize("load_ref,with_rho,with_entropy", [(True, True, True), (False, True, False), (True, False, False)])
+@pytest.mark.parametrize("route", ["tensors", "fused", "plain_dict"])
+def test_populate_sample_loss_stats_parity(load_ref, with_rho, with_entropy, route):
+    """open_instruct/grpo_utils.py:674-742 on the device against the oracle's restatement: from the
+    per-token tensors (the reference's call; one pass, written into the table column), from the
+    statistics of the fused loss kernels (nothing recomputed) and into a plain dict of tensors."""
+    new, old, ref, adv, mask, _ = _grpo_inputs(16, shape=(5, 1300), edge=True)
+    cfg = make_grpo_config(
+        loss_fn="dapo", clip_higher=0.28, beta=0.05, kl_estimator=2, load_ref_policy=load_ref, use_rho_correction=True,
+        rho_mask_lower_bound=0.7, rho_mask_upper_bound=1.4, rho_clamp_lower_bound=0.8, rho_clamp_upper_bound=1.2,
+    )  # fmt: skip
+    g = torch.Generator().manual_seed(17)
+    vllm = old + 0.3 * torch.randn(old.shape, generator=g)
+    ent = torch.rand(new.shape, generator=g) * 3 if with_entropy else None
+    o_rho = o_grpo.compute_rho_correction(old, vllm, mask, adv, cfg)
+    e_loss, e_pg, e_cf, _, e_ratio = o_grpo.grpo_token_loss(new, old, ref, adv, mask, cfg, o_rho.weights)
+    exp = o_grpo.create_loss_stats(3, record_entropy=with_entropy)
+    o_grpo.populate_sample_loss_stats(
+        exp, 1, e_pg, e_cf, e_ratio, e_loss, mask, new, ref, ent, cfg, o_rho.metrics if with_rho else None
+    )
+
+    d = lambda t: None if t is None else t.to(DEV)  # noqa: E731
+    rho = grpo_utils.compute_rho_correction(d(old), d(vllm), d(mask), d(adv), cfg)
+    stats = grpo_utils.create_loss_stats(3, torch.device(DEV), record_entropy=with_entropy)
+    assert set(stats) == set(exp) and all(v.shape == (3,) and v.is_cuda for v in stats.values())
+    if route == "plain_dict":
+        stats = {k: torch.zeros(3, device=DEV) for k in stats}
+    rho_metrics = rho.metrics if with_rho else None
+    if route == "fused":
+        loss, fused = grpo_utils.grpo_loss_fused(
+            d(new), d(old), d(ref), d(adv), d(mask), cfg, rho.weights, d(ent), rho_metrics=rho_metrics
+        )
+        grpo_utils.populate_sample_loss_stats(
+            stats, 1, None, None, None, loss, d(mask), d(new), d(ref), d(ent), cfg, rho_metrics, fused_stats=fused
+        )
+    else:
+        ratio = torch.exp(d(new) - d(old))
+        pg, cf, _ = grpo_utils.compute_grpo_loss(d(new), ratio, d(adv), d(ref), cfg, rho.weights)
+        loss = d(e_loss)
+        grpo_utils.populate_sample_loss_stats(stats, 1, pg, cf, ratio, loss, d(mask), d(new), d(ref), d(ent), cfg, rho_metrics)
+    for key, value in exp.items():
+        got = stats[key].cpu()
+        assert got[0].item() == 0.0 and got[2].item() == 0.0, key  # other samples untouched
+        tol = 2e-5 * max(1.0, abs(value[1].item()))
+        assert abs(got[1].item() - value[1].item()) <= tol, (key, got[1].item(), value[1].item())
+    # the epoch summary: token-weighted means and the weighted variance of val/ratio
+    counts = torch.tensor([3.0, 5.0, 0.0])
+    for k in stats:
+        stats[k][0] = 0.25
+    exp_summary = o_grpo.compute_metrics_from_loss_stats({k: v.cpu() for k, v in stats.items()}, counts)
+    summary = grpo_utils.compute_metrics_from_loss_stats(stats, counts.to(DEV))
+    assert set(summary) == set(exp_summary)
+    for k, v in exp_summary.items():
+        assert summary[k] == pytest.approx(v, rel=1e-5, abs=1e-7), k
+    zero = grpo_utils.compute_metrics_from_loss_stats(stats, torch.zeros(3, device=DEV))
+    assert all(v == 0.0 for v in zero.values())
+
+
 def test_group_advantages_on_device():
     rng = np.random.default_rng(0)
     scores = (rng.random(64) < 0.3).astype(np.float64)
@@ -599,3 +657,52 @@ def test_grpo_loss_on_logits_full_vocabulary_rows():
     assert ga.sum(-1).abs().max().item() <= 0.05 * ga.abs().max().item() * 8
     for k in stats_c:
         assert abs(stats_a[k].item() - stats_c[k].item()) <= 1e-5 * max(1.0, abs(stats_c[k].item())), k
+
+
+def test_grpo_loss_on_logits_broadcast_side_tensors():
+    """Side tensors that only broadcast to [B, T] ([B, 1] advantages, a 0-dim rho weight, [1, T] old
+    logprobs) are accepted by the reference's elementwise code; the single-launch route must expand
+    them like the two-pass route does and give the same loss and gradient."""
+    g = torch.Generator().manual_seed(51)
+    b, t, vocab = 4, 9, 4096
+    logits = (torch.randn(b, t, vocab, generator=g) * 2.0).bfloat16()
+    labels = torch.randint(0, vocab, (b, t), generator=g)
+    mask = torch.rand(b, t, generator=g) > 0.2
+    adv = torch.randn(b, 1, generator=g)
+    rho = torch.tensor(0.75)
+    ref = -10.3 + 0.5 * torch.randn(1, t, generator=g)  # near the logprobs of N(0, 2) logits at this vocabulary
+    cfg = make_grpo_config(loss_fn="dapo", beta=0.05, kl_estimator=2, clip_higher=0.28)
+    d = lambda x: x.to(DEV)  # noqa: E731
+    one = d(logits).requires_grad_(True)
+    loss1, _, lp1, _ = grpo_utils.grpo_loss_on_logits(one, d(labels), None, d(ref), d(adv), d(mask), cfg, rho_weights=d(rho))
+    loss1.backward()
+    two = d(logits).requires_grad_(True)
+    lp2, ent2 = model_utils.logprob_and_entropy(two, d(labels))
+    loss2, _ = grpo_utils.grpo_loss_fused(lp2, None, d(ref), d(adv), d(mask), cfg, rho_weights=d(rho), entropy=ent2)
+    loss2.backward()
+    rl = logits.float().requires_grad_(True)
+    lp_o = o_logprob.log_softmax_and_gather(rl, labels, None)
+    loss_o, *_ = o_grpo.grpo_token_loss(
+        lp_o, lp_o.detach(), ref.expand(b, t), adv.expand(b, t), mask.float(), cfg, rho_weights=rho.expand(b, t)
+    )
+    loss_o.backward()
+    assert abs(loss1.item() - loss2.item()) <= 1e-5 and abs(loss1.item() - loss_o.item()) <= 2e-3
+    assert (one.grad.float() - two.grad.float()).abs().max().item() <= 2.0**-7 * two.grad.float().abs().max().item()
+    assert (one.grad.float().cpu() - rl.grad).abs().max().item() <= 2e-3 + 2.0**-7 * rl.grad.abs().max().item()
+    with pytest.raises(ValueError, match="does not broadcast"):
+        grpo_utils.grpo_loss_on_logits(one, d(labels), None, None, d(adv.reshape(1, b)), d(mask), cfg)
+    # an evaluation call builds no gradient tensor and still returns the loss
+    with torch.no_grad():
+        loss3, _, lp3, _ = grpo_utils.grpo_loss_on_logits(one, d(labels), None, d(ref), d(adv), d(mask), cfg, rho_weights=d(rho))
+    assert not loss3.requires_grad and abs(loss3.item() - loss1.item()) <= 1e-5
+
+
+def test_rho_correction_broadcast_advantages():
+    new, old, _, _, mask, _ = _grpo_inputs(23, shape=(4, 60))
+    adv = torch.randn(4, 1, generator=torch.Generator().manual_seed(3))
+    cfg = make_grpo_config(use_rho_correction=True, rho_mask_tv_divergence=True, rho_mask_lower_bound=0.05, rho_mask_upper_bound=0.2)
+    exp = o_grpo.compute_rho_correction(old, new, mask, adv.expand(4, 60), cfg)
+    got = grpo_utils.compute_rho_correction(old.to(DEV), new.to(DEV), mask.to(DEV), adv.to(DEV), cfg)
+    _close(got.weights, exp.weights)
+    for k, v in exp.metrics.items():
+        _close(got.metrics[k], v)

@@ -194,3 +194,14 @@ def test_collation_of_packed_rows_for_workers():
     single = data_loader.prepare_collated_data_for_workers(packed, 1, 1, pad_token_id=0)
     assert len(single) == 1 and len(single[0]) == 5 and all(t.shape[0] == 1 for t in single[0].query_responses)
     assert data_loader.collate_fn([torch.tensor([1, 2, 3])], 0).shape == (1, 3)
+
+
+def test_side_tensors_that_do_not_broadcast_are_rejected_before_any_kernel():
+    cfg = make_grpo_config()
+    logits = torch.randn(2, 3, 16).requires_grad_(True)
+    labels = torch.zeros(2, 3, dtype=torch.int64)
+    mask = torch.ones(2, 3, dtype=torch.bool)
+    with pytest.raises(ValueError, match="advantages of shape"):
+        grpo_utils.grpo_loss_on_logits(logits, labels, None, None, torch.zeros(3, 2), mask, cfg)
+    with pytest.raises(ValueError, match="advantages of shape"):
+        grpo_utils.compute_rho_correction(torch.zeros(2, 3), torch.zeros(2, 3), mask, torch.zeros(5), cfg)

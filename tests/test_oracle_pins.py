@@ -6,6 +6,7 @@ the reference's own test data (tests/golden/reference_known_answers.json).
 """
 
 import math
+import types
 
 import numpy as np
 import pytest
@@ -414,18 +415,64 @@ def test_dpo_loss_reference_test_properties():
     assert not cr.requires_grad and not rj.requires_grad
 
 
+def _py_pair_loss(x: float, beta: float, ls: float) -> float:
+    """-(1 - ls) log sigmoid(beta x) - ls log sigmoid(-beta x) on Python floats."""
+    neg_log_sigmoid = lambda u: math.log1p(math.exp(-u)) if u > 0 else -u + math.log1p(math.exp(u))  # noqa: E731
+    return (1 - ls) * neg_log_sigmoid(beta * x) + ls * neg_log_sigmoid(-beta * x)
+
+
 def test_simpo_and_wpo_closed_forms():
     pc, pr = torch.tensor([-2.0, -1.0]), torch.tensor([-3.0, -4.0])
     out, cr, rj = dpo.simpo_loss(pc, pr, beta=2.0, gamma_beta_ratio=1.0)
     assert out[0].item() == pytest.approx(math.log(2.0), rel=1e-6)  # margin exactly cancels: x = 0
     assert torch.allclose(cr, 2.0 * pc) and torch.allclose(rj, 2.0 * pr)
-    # the reference broadcasts the [bs] logps against the [bs, T] token masks, which only works
-    # for bs == 1 (its shipped configs); there the "average" is logp * count / count = logp
-    pc1, pr1 = pc[:1], pr[:1]
-    mask = torch.tensor([[True, True, False, True]])
-    base, _, _ = dpo.dpo_loss(pc1, pr1, pc1 + 0.5, pr1, beta=0.3)
-    out, _, _ = dpo.wpo_loss(pc1, pr1, pc1 + 0.5, pr1, 0.3, mask, mask)
-    assert torch.allclose(out, base * torch.exp(pc1 + pr1).clamp(max=1))
+    assert not cr.requires_grad and not rj.requires_grad
+
+
+@pytest.mark.parametrize("label_smoothing", [0.0, 0.1, 0.5])
+def test_simpo_loss_against_python_floats(label_smoothing):
+    """open_instruct/dpo_utils.py:617-642 away from x = 0, with label smoothing, on both sides of the
+    margin: every pair against a ``math.log1p`` evaluation on Python floats."""
+    pc = [-2.0, -1.0, -30.0, -0.25, -7.5]
+    pr = [-3.0, -4.0, -2.0, -0.75, -7.5]
+    beta, gbr = 2.5, 0.6
+    out, cr, rj = dpo.simpo_loss(torch.tensor(pc), torch.tensor(pr), beta, gbr, label_smoothing)
+    for i in range(len(pc)):
+        exp = _py_pair_loss(pc[i] - pr[i] - gbr, beta, label_smoothing)
+        assert out[i].item() == pytest.approx(exp, rel=2e-6, abs=1e-6), i
+        assert cr[i].item() == pytest.approx(beta * pc[i]) and rj[i].item() == pytest.approx(beta * pr[i])
+    # the margin enters as a plain shift of the log-ratio
+    shifted, _, _ = dpo.simpo_loss(torch.tensor(pc) - gbr, torch.tensor(pr), beta, 0.0, label_smoothing)
+    assert torch.allclose(out, shifted, atol=1e-6)
+
+
+@pytest.mark.parametrize("label_smoothing", [0.0, 0.2])
+def test_wpo_loss_against_python_floats(label_smoothing):
+    """open_instruct/dpo_utils.py:566-613 for one pair (the reference broadcasts the [bs] logps against
+    the [bs, T] token masks, which only works for bs == 1, its shipped setting; there the "average"
+    is logp * count / count = logp).  Cases on both sides of the clamp: exp(avg_c + avg_r) below 1
+    (negative logps) and above 1 (a positive sum, where the weight must stop at 1); expected values
+    from Python floats."""
+    mask_c = torch.tensor([[True, True, False, True]])
+    mask_r = torch.tensor([[True, False, False, False]])
+    beta = 0.3
+    for pc, pr, rc, rr in [(-0.2, -0.5, -0.4, -0.1), (0.9, -0.3, 0.1, -0.2), (1.5, 2.0, 1.0, 0.0), (-6.0, -9.0, -5.0, -5.0)]:
+        out, cr, rj = dpo.wpo_loss(
+            torch.tensor([pc]), torch.tensor([pr]), torch.tensor([rc]), torch.tensor([rr]), beta, mask_c, mask_r,
+            label_smoothing,
+        )  # fmt: skip
+        weight = min(1.0, math.exp(pc + pr))
+        exp = _py_pair_loss((pc - pr) - (rc - rr), beta, label_smoothing) * weight
+        assert out.shape == (1,) and out.item() == pytest.approx(exp, rel=2e-6, abs=1e-7), (pc, pr)
+        assert cr.item() == pytest.approx(beta * (pc - rc), abs=1e-6) and rj.item() == pytest.approx(beta * (pr - rr), abs=1e-6)
+    # the weight is not detached in the reference: its gradient reaches the policy logps
+    pc_t = torch.tensor([-0.2], requires_grad=True)
+    out, _, _ = dpo.wpo_loss(pc_t, torch.tensor([-0.5]), torch.tensor([-0.4]), torch.tensor([-0.1]), beta, mask_c, mask_r)
+    out.sum().backward()
+    x = (-0.2 + 0.5) - (-0.4 + 0.1)
+    w = math.exp(-0.7)
+    d_loss_dx = -beta / (1 + math.exp(beta * x))
+    assert pc_t.grad.item() == pytest.approx(w * d_loss_dx + w * _py_pair_loss(x, beta, 0.0), rel=1e-5)
 
 
 # ---------------------------------------------------------------- lm_head
@@ -563,3 +610,44 @@ def test_pack_sequences_reference_vectors_and_properties(golden):
     assert packing.broadcast_advantages([0.5, -1.5, 2.0], out["response_masks"]) == [
         [0, 0, 0, 0, 0.5, 0.5, 0.5, 0, 0, 0, -1.5], [0, 0, 2.0, 2.0, 2.0, 2.0],
     ]  # fmt: skip
+
+
+def test_loss_stat_helpers_by_hand():
+    """open_instruct/grpo_utils.py:674-742 on numbers small enough to average by hand: three kept
+    tokens, KL entries only with a reference policy, rho entries only when given, weighted summary."""
+    cfg = types.SimpleNamespace(load_ref_policy=True, kl_estimator=1, beta=0.5)
+    mask = torch.tensor([[True, True, False, True]])
+    pg = torch.tensor([[1.0, 2.0, 100.0, 6.0]])
+    clip = torch.tensor([[1.0, 0.0, 1.0, 0.0]])
+    ratio = torch.tensor([[1.0, 2.0, 50.0, 3.0]])
+    new = torch.tensor([[0.0, -1.0, 0.0, -2.0]])
+    ref = torch.tensor([[-1.0, -1.0, 5.0, 0.0]])  # d = [1, 0, ., -2]
+    ent = torch.tensor([[3.0, 3.0, 9.0, 6.0]])
+    stats = grpo.create_loss_stats(2, record_entropy=True)
+    assert set(stats) == set(grpo.LOSS_STAT_KEYS) | {"policy/entropy_avg"} and len(stats) == 15
+    grpo.populate_sample_loss_stats(stats, 1, pg, clip, ratio, torch.tensor(7.5), mask, new, ref, ent, cfg)
+    exp = {
+        "loss/policy_avg": 3.0, "policy/clipfrac_avg": 1 / 3, "val/ratio": 2.0, "loss/total_avg": 7.5,
+        "policy/entropy_avg": 4.0, "objective/kl0_avg": (1 + 0 - 2) / 3, "objective/kl1_avg": (0.5 + 0 + 2.0) / 3,
+        "objective/kl2_avg": (math.expm1(-1) + 1 + 0 + math.expm1(2) - 2) / 3,
+        "objective/kl3_avg": (1 * 1 + 2 * 0 + 3 * -2) / 3, "loss/kl_avg": 0.5 * (0.5 + 0 + 2.0) / 3,
+    }  # fmt: skip
+    for key, value in stats.items():
+        assert value[0].item() == 0.0, key  # the other sample is untouched
+        assert value[1].item() == pytest.approx(exp.get(key, 0.0), rel=1e-6, abs=1e-7), key
+    # without a reference policy the KL entries stay zero even when reference logprobs are passed
+    cfg2 = types.SimpleNamespace(load_ref_policy=False, kl_estimator=1, beta=0.5)
+    stats2 = grpo.create_loss_stats(1)
+    rho = {"val/rho_weight": torch.tensor([[2.0, 0.0, 9.0, 1.0]]), "val/rho_drop_frac": torch.tensor([[0.0, 1.0, 1.0, 0.0]])}
+    grpo.populate_sample_loss_stats(stats2, 0, pg, clip, ratio, torch.tensor(1.0), mask, new, ref, None, cfg2, rho)
+    assert stats2["objective/kl1_avg"][0].item() == 0.0 and stats2["loss/kl_avg"][0].item() == 0.0
+    assert "policy/entropy_avg" not in stats2
+    assert stats2["val/rho_weight"][0].item() == pytest.approx(1.0)
+    assert stats2["val/rho_drop_frac"][0].item() == pytest.approx(1 / 3)
+    assert stats2["val/rho_clipfrac"][0].item() == 0.0
+    summary = grpo.compute_metrics_from_loss_stats(
+        {"val/ratio": torch.tensor([1.0, 3.0]), "loss/total_avg": torch.tensor([2.0, 4.0])}, torch.tensor([1.0, 3.0])
+    )
+    assert summary["val/ratio"] == pytest.approx(2.5) and summary["loss/total_avg"] == pytest.approx(3.5)
+    assert summary["val/ratio_var"] == pytest.approx(0.25 * 1.5**2 + 0.75 * 0.5**2)
+    assert grpo.compute_metrics_from_loss_stats({"val/ratio": torch.ones(2)}, torch.zeros(2))["val/ratio"] == 0.0
