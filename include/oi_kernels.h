@@ -14,7 +14,10 @@
  *    call returns without waiting for it.
  *  - Return value: 0 on success, a negative OI_E* code for a rejected argument (nothing was
  *    launched), a positive value = the hipError_t of a failed launch.
- *  - The library keeps no mutable global state; calls are re-entrant.
+ *  - Calls are re-entrant.  The only state the library keeps between calls is looked up once per
+ *    device under a lock and never changes afterwards: the CU count, and the device address of the
+ *    static scratch array of oi_grpo_fused_fwd_static (the one entry point that shares memory
+ *    between calls; see there).
  *  - Row-major everywhere; strides are in ELEMENTS, not bytes.
  *  - Token ids / labels are int64, sequence boundaries int32, masks one byte per token (0 / 1).
  */
@@ -34,6 +37,7 @@ extern "C" {
 #define OI_EALIGN (-3)     /* pointer/stride alignment the kernel needs is not met  */
 #define OI_EDTYPE (-4)     /* unknown or unsupported dtype tag                      */
 #define OI_EWORKSPACE (-5) /* workspace_bytes is smaller than the op needs          */
+#define OI_ETOOLARGE (-6)  /* larger than the static scratch of a *_static entry    */
 
 #define OI_DTYPE_F32 0
 #define OI_DTYPE_BF16 1
@@ -164,6 +168,26 @@ int oi_grpo_fused_fwd(const float* new_logprobs, const float* old_logprobs, cons
                       const float* rho_clipped, int64_t rows, int64_t cols, int loss_fn, float ratio_lo,
                       float ratio_hi, int kl_estimator, float beta, int axis_mode, float denominator, float scale,
                       float* out_stats, float* row_denoms, void* workspace, size_t workspace_bytes, void* stream);
+/*
+ * oi_grpo_fused_fwd for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments, results and kernels as oi_grpo_fused_fwd, without the workspace: the partial
+ * sums live in a file-scope device array of the library (OI_GRPO_STATIC_MAX_BLOCKS * 15 floats =
+ * 480 KB, held on every GPU the library runs on until the process ends).  The call allocates and
+ * frees nothing.  Limit: rows * ceil(cols / 1024) <= OI_GRPO_STATIC_MAX_BLOCKS, OI_ETOOLARGE
+ * beyond it (nothing is launched).  The first call on a device looks up the array's address on
+ * that device (hipGetSymbolAddress); make it before a stream capture starts.  All calls on one GPU
+ * share the array: calls that overlap in time on one GPU (two streams, two threads) race; calls
+ * in stream order do not, and nothing has to be cleared between them.
+ */
+#define OI_GRPO_STATIC_MAX_BLOCKS 8192
+int oi_grpo_fused_fwd_static(const float* new_logprobs, const float* old_logprobs, const float* ref_logprobs,
+                             const float* advantages, const uint8_t* mask, const float* rho_weights,
+                             const float* entropy, const float* rho_drop_any, const float* rho_drop_low,
+                             const float* rho_drop_high, const float* rho_clipped, int64_t rows, int64_t cols,
+                             int loss_fn, float ratio_lo, float ratio_hi, int kl_estimator, float beta, int axis_mode,
+                             float denominator, float scale, float* out_stats, float* row_denoms, void* stream);
+
 /*
  * The same statistics for a caller that already holds the per-token terms.  Carries
  * open_instruct/grpo_utils.py:699-729 (populate_sample_loss_stats) in two launches: masked means

@@ -37,6 +37,10 @@ SIGNATURES: dict[str, tuple] = {
         _I,
         [_P] * 11 + [_I64, _I64, _I, _F, _F, _I, _F, _I, _F, _F, _P, _P, _P, _SZ, _P],
     ),
+    "oi_grpo_fused_fwd_static": (
+        _I,
+        [_P] * 11 + [_I64, _I64, _I, _F, _F, _I, _F, _I, _F, _F, _P, _P, _P],
+    ),
     "oi_grpo_stats_from_terms": (_I, [_P] * 12 + [_I64, _I64, _I, _F, _P, _I64, c_uint32, _P, _SZ, _P]),
     "oi_scale_by_device_scalar": (_I, [_P, _I, _I64, _P, _P]),
     "oi_grpo_fused_bwd": (_I, [_P, _P, _P, _P, _P, _P, _I64, _I64, _I, _F, _F, _I, _F, _F, _P, _P, _P, _P]),

@@ -6,6 +6,14 @@
 #include "oi_common.h"
 #include "oi_grpo_math.h"
 
+#include <mutex>
+
+// Partial sums of oi_grpo_fused_fwd_static, the entry point for callers that cannot allocate.
+// Every GPU the library runs on holds its own copy of this array at its own address until the
+// process ends.  In host code the name is only a handle for hipGetSymbolAddress: kernels are given
+// the per-device address that static_scratch_ptr() looked up, never the name.
+static __device__ __align__(256) float oi_static_scratch[OI_GRPO_STATIC_MAX_BLOCKS * 15];
+
 namespace {
 
 __global__ void grpo_terms_fwd_kernel(const float* __restrict__ nlp, const float* __restrict__ ratio,
@@ -630,6 +638,58 @@ extern "C" int oi_grpo_fused_fwd(const float* new_logprobs, const float* old_log
                              static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
 }
 
+namespace {
+std::mutex static_scratch_mutex;
+float* static_scratch_of_device[64] = {};
+
+// Address of oi_static_scratch on the current device, looked up once per device.
+int static_scratch_ptr(float** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    OI_RETURN_IF(dev < 0 || dev >= 64, OI_EINVAL);
+    std::lock_guard<std::mutex> lock(static_scratch_mutex);
+    if (!static_scratch_of_device[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(oi_static_scratch));
+        if (e != hipSuccess) return (int)e;
+        OI_RETURN_IF(!p, OI_ENULL);
+        static_scratch_of_device[dev] = static_cast<float*>(p);
+    }
+    *out = static_scratch_of_device[dev];
+    return OI_OK;
+}
+}  // namespace
+
+extern "C" int oi_grpo_fused_fwd_static(const float* new_logprobs, const float* old_logprobs,
+                                        const float* ref_logprobs, const float* advantages, const uint8_t* mask,
+                                        const float* rho_weights, const float* entropy, const float* rho_drop_any,
+                                        const float* rho_drop_low, const float* rho_drop_high,
+                                        const float* rho_clipped, int64_t rows, int64_t cols, int loss_fn,
+                                        float ratio_lo, float ratio_hi, int kl_estimator, float beta, int axis_mode,
+                                        float denominator, float scale, float* out_stats, float* row_denoms,
+                                        void* stream) {
+    static_assert(sizeof(oi_static_scratch) == sizeof(float) * OI_GRPO_STATIC_MAX_BLOCKS * NSUM, "scratch size");
+    int rc = check_stats_shape(rows, cols);
+    if (rc != OI_OK) return rc;
+    OI_RETURN_IF(axis_mode != 0 && axis_mode != 1, OI_EINVAL);
+    rc = check_cfg(loss_fn, kl_estimator);
+    if (rc != OI_OK) return rc;
+    OI_RETURN_IF(!new_logprobs || !advantages || !mask || !out_stats || !row_denoms, OI_ENULL);
+    const int64_t nchunks = (cols + FUSED_CHUNK - 1) / FUSED_CHUNK;
+    OI_RETURN_IF(rows * nchunks > OI_GRPO_STATIC_MAX_BLOCKS, OI_ETOOLARGE);
+    float* partial = nullptr;
+    rc = static_scratch_ptr(&partial);
+    if (rc != OI_OK) return rc;
+    // nothing in the array has to start at zero: the first kernel writes every partial sum that the
+    // second one reads (rows * nchunks * NSUM floats), whatever an earlier call left there
+    const GrpoCfg c = {loss_fn, ratio_lo, ratio_hi, kl_estimator};
+    const StatIn in = {new_logprobs, old_logprobs, ref_logprobs, advantages, rho_weights, nullptr, nullptr,
+                       nullptr,      entropy,      rho_drop_any, rho_drop_low, rho_drop_high, rho_clipped, mask};
+    return launch_grpo_stats(in, rows, cols, c, beta, axis_mode, denominator, scale, out_stats, 1, 0xffffu, row_denoms,
+                             partial, static_cast<hipStream_t>(stream));
+}
+
 extern "C" int oi_grpo_stats_from_terms(const float* pg_loss, const float* clipfrac, const float* ratio,
                                         const float* new_logprobs, const float* ref_logprobs, const uint8_t* mask,
                                         const float* entropy, const float* rho_weight, const float* rho_drop_any,
@@ -837,6 +897,7 @@ extern "C" const char* oi_error_string(int code) {
         case OI_EALIGN: return "pointer or stride alignment is not met";
         case OI_EDTYPE: return "unknown or unsupported dtype tag";
         case OI_EWORKSPACE: return "workspace is too small";
+        case OI_ETOOLARGE: return "problem is larger than the static scratch of this entry point";
         default: return code > 0 ? "HIP launch error (value is a hipError_t)" : "unknown error code";
     }
 }

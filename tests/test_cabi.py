@@ -84,6 +84,13 @@ def test_rejected_arguments_return_codes_without_launching():
     assert lib.oi_logprob_diff_stats(None, None, None, 4, None, None) == -2
     assert lib.oi_logprob_diff_stats(None, None, None, -1, None, None) == -1
     assert lib.oi_masked_mean_workspace_bytes(4, 2, 3) == (4 + 1) * 2 * 1 * 4
+    # the entry point without a workspace refuses what its static scratch cannot hold (the pointers
+    # are never dereferenced: the call is rejected before anything touches the GPU)
+    fake = [8] * 11
+    assert lib.oi_grpo_fused_fwd_static(*fake, 8193, 10, 0, 0.8, 1.2, 2, 0.05, 0, 0.0, 1.0, 8, 8, None) == -6
+    assert lib.oi_grpo_fused_fwd_static(*fake, 9, 1024 * 1024, 0, 0.8, 1.2, 2, 0.05, 0, 0.0, 1.0, 8, 8, None) == -6
+    assert lib.oi_grpo_fused_fwd_static(*fake, 4, 10, 5, 0.8, 1.2, 2, 0.05, 0, 0.0, 1.0, 8, 8, None) == -1
+    assert lib.oi_grpo_fused_fwd_static(*([None] * 11), 4, 10, 0, 0.8, 1.2, 2, 0.05, 0, 0.0, 1.0, 8, 8, None) == -2
     assert lib.oi_lmhead_fwd_workspace_bytes(0, 64, 10) == 0
     # one dZ chunk (bf16), the fp32 d_hidden accumulator, three queues of 8 words; no transposed copies
     assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1) == 256 * 256 * 2 + 256 * 64 * 4 + 256
