@@ -340,11 +340,18 @@ int oi_pack_sequences(const int64_t* q_tokens, const int64_t* q_offsets, const i
  * labels are scored as token 0 (clamp(min=0) at open_instruct/padding_free_collator.py:15).
  *
  *   z = hidden @ weight^T (bf16 MFMA, fp32 accumulate), logprob/entropy/lse as for oi_lsg_*.
+ *
+ * row_mask (one byte per token, may be NULL = every row): rows whose byte is 0 are not multiplied
+ * and their outputs are 0 (prompt and padding positions, whose results the reference masks out
+ * afterwards: open_instruct/grpo_utils.py:340-344, open_instruct/dpo_utils.py:689-712).  The
+ * selection is made on the device: a row index is built from the mask and the selected rows are
+ * gathered into the workspace, every kernel reads the selected count from device memory, the host
+ * never waits.  The workspace is sized for all n_tokens rows either way.
  * ------------------------------------------------------------------------------------------ */
-size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab);
-int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
-                       int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob, float* entropy,
-                       float* lse, void* workspace, size_t workspace_bytes, void* stream);
+size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int with_row_mask);
+int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* labels, const uint8_t* row_mask,
+                       int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob,
+                       float* entropy, float* lse, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Backward: recomputes the logits tile by tile,
@@ -354,13 +361,16 @@ int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* la
  * Vocabulary is processed in chunks of 32768 columns; only one chunk of dZ (bf16, token-major)
  * lives in the workspace at a time, next to the fp32 accumulator of d_hidden.  Both products
  * read weight, hidden and dZ where they lie (no transposed copies), so the workspace is the same
- * with and without d_weight.
+ * with and without d_weight.  row_mask as in the forward (rows left out get a zero d_hidden row
+ * and add nothing to d_weight); skip_zero_grad_rows != 0 also leaves out rows whose grad_logprob is
+ * exactly 0, which changes no result.  d_hidden and d_weight must be 4-byte aligned.
  */
-size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int want_d_weight);
+size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int want_d_weight,
+                                     int with_row_selection);
 int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
-                       const float* grad_logprob, int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
-                       float inv_temperature, void* d_hidden, void* d_weight, void* workspace,
-                       size_t workspace_bytes, void* stream);
+                       const float* grad_logprob, const uint8_t* row_mask, int skip_zero_grad_rows, int64_t n_tokens,
+                       int64_t hidden_dim, int64_t vocab, float inv_temperature, void* d_hidden, void* d_weight,
+                       void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * The bf16 MFMA main loop of the lm_head kernels as a plain product (no reference counterpart;

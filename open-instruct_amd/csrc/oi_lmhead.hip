@@ -22,6 +22,7 @@
 // CU that draws tile ids from per-XCD counters.
 #include "oi_common.h"
 
+#include <atomic>
 #include <type_traits>
 
 namespace {
@@ -564,10 +565,11 @@ __device__ __forceinline__ void lmhead_fwd_item(const uint16_t* __restrict__ W, 
 
 __global__ void __launch_bounds__(NTHREADS)
     lmhead_fwd_kernel(const uint16_t* __restrict__ W, const uint16_t* __restrict__ hidden,
-                      const int64_t* __restrict__ labels, int64_t n_tokens, int64_t hdim, int64_t vocab, float c,
-                      int64_t n_splits, int64_t tiles_per_split, int64_t n_pad, float4* __restrict__ partial,
-                      float* __restrict__ zy, uint32_t* __restrict__ queue) {
+                      const int64_t* __restrict__ labels, int64_t n_tokens, const int32_t* __restrict__ n_dev,
+                      int64_t hdim, int64_t vocab, float c, int64_t n_splits, int64_t tiles_per_split, int64_t n_pad,
+                      float4* __restrict__ partial, float* __restrict__ zy, uint32_t* __restrict__ queue) {
     __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
+    if (n_dev) n_tokens = *n_dev;  // rows selected on the device: the host only knows an upper bound
     const int64_t token_tiles = (n_tokens + BN - 1) / BN;
     for_each_tile(queue, n_splits, token_tiles, lds, [&](int64_t split, int64_t tt) {
         lmhead_fwd_item(W, hidden, labels, n_tokens, hdim, vocab, c, tiles_per_split, n_pad, partial, zy, split, tt,
@@ -575,11 +577,23 @@ __global__ void __launch_bounds__(NTHREADS)
     });
 }
 
+// Merges the partial statistics of token n over the vocabulary splits.  With a row selection
+// (`rows` non-null) token n of the compacted batch is row rows[n] of the caller's tensors, the count
+// comes from the device, and the rows that were left out are written as zeros: the grid covers
+// n_total rows, thread i handles compacted token i and caller row i.
 __global__ void lmhead_fwd_combine_kernel(const float4* __restrict__ partial, const float* __restrict__ zy,
-                                          int64_t n_tokens, int64_t n_splits, int64_t n_pad, float inv_t,
+                                          int64_t n_tokens, const int32_t* __restrict__ n_dev,
+                                          const int32_t* __restrict__ rows, const uint8_t* __restrict__ row_mask,
+                                          int64_t n_total, int64_t n_splits, int64_t n_pad, float inv_t,
                                           float* __restrict__ logprob, float* __restrict__ entropy,
                                           float* __restrict__ lse_out) {
     const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (n_dev) n_tokens = *n_dev;
+    if (row_mask && n < n_total && !row_mask[n]) {
+        logprob[n] = 0.f;
+        if (entropy) entropy[n] = 0.f;
+        if (lse_out) lse_out[n] = 0.f;
+    }
     if (n >= n_tokens) return;
     float m = OI_NEG_BIG, s = 0.f, t = 0.f;
     for (int64_t sp = 0; sp < n_splits; ++sp) {
@@ -589,9 +603,10 @@ __global__ void lmhead_fwd_combine_kernel(const float4* __restrict__ partial, co
     const double ln2 = 0.69314718055994530942;
     const double log2s = log2((double)s);
     const double lse = ((double)m + log2s) * ln2;
-    logprob[n] = (float)((double)zy[n] * (double)inv_t - lse);
-    if (entropy) entropy[n] = (float)((log2s - (double)t / (double)s) * ln2);
-    if (lse_out) lse_out[n] = (float)lse;
+    const int64_t o = rows ? rows[n] : n;
+    logprob[o] = (float)((double)zy[n] * (double)inv_t - lse);
+    if (entropy) entropy[o] = (float)((log2s - (double)t / (double)s) * ln2);
+    if (lse_out) lse_out[o] = (float)lse;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -667,10 +682,14 @@ __device__ __forceinline__ void lmhead_dz_tile(const uint16_t* __restrict__ W, c
 __global__ void __launch_bounds__(NTHREADS)
     lmhead_dz_kernel(const uint16_t* __restrict__ W, const uint16_t* __restrict__ hidden,
                      const int64_t* __restrict__ labels, const float* __restrict__ lse,
-                     const float* __restrict__ grad, int64_t n_tokens, int64_t hdim, int64_t vocab, float c,
-                     float inv_t, int64_t v_begin, int64_t chunk_cols, int64_t n_pad, uint16_t* __restrict__ dz,
-                     uint32_t* __restrict__ queue) {
+                     const float* __restrict__ grad, int64_t n_tokens, const int32_t* __restrict__ n_dev,
+                     int64_t hdim, int64_t vocab, float c, float inv_t, int64_t v_begin, int64_t chunk_cols,
+                     int64_t n_pad, uint16_t* __restrict__ dz, uint32_t* __restrict__ queue) {
     __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
+    if (n_dev) {
+        n_tokens = *n_dev;
+        n_pad = (n_tokens + BN - 1) / BN * BN;
+    }
     for_each_tile(queue, chunk_cols / BM, n_pad / BN, lds, [&](int64_t vt, int64_t tt) {
         lmhead_dz_tile(W, hidden, labels, lse, grad, n_tokens, hdim, vocab, c, inv_t, v_begin, chunk_cols, n_pad, dz,
                        vt, tt, lds);
@@ -683,17 +702,28 @@ __global__ void __launch_bounds__(NTHREADS)
 // mode 0: out_f32  = acc          mode 1: out_f32 += acc
 // mode 2: out_bf16 = acc          mode 3: out_bf16 = out_f32 + acc   (last chunk of d_hidden)
 // A, B: operands without their tile origin (r0 is filled in here); the product has M x N
-// entries, of which rows below m_valid are stored.
+// entries, of which rows below m_valid are stored.  K == 0 stores zeros.  With `out_rows`, row r
+// of a bf16 result goes to row out_rows[r] of out_bf16 (the fp32 accumulator stays compact).
 template <bool A_KM, bool B_KM>
 __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B, int64_t N, int64_t K, int mode,
                                                 float* out_f32, uint16_t* out_bf16, int64_t ldo, int64_t m_valid,
-                                                int64_t tm, int64_t tn, uint16_t* lds) {
+                                                const int32_t* __restrict__ out_rows, int64_t tm, int64_t tn,
+                                                uint16_t* lds) {
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6, wm = wave & 3, wn = wave >> 2;
     const int64_t m0 = tm * BM, n0 = tn * BN;
     A.r0 = m0;
     B.r0 = n0;
     AccTile acc;
-    gemm_tile<A_KM, B_KM>(acc, A, B, K, lds);
+    if (K > 0) {
+        gemm_tile<A_KM, B_KM>(acc, A, B, K, lds);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    }
     if (mode >= 2 && (ldo & 1) == 0) {
         // bf16 output: neighbouring lanes hold neighbouring columns of the same rows; after one DPP
         // swap per pair of rows every lane stores two columns of one row as a 4-byte word (half as
@@ -702,28 +732,32 @@ __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B,
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int64_t col = n0 + (acc_col(wn, j, lane) & ~1);
+            for (int t = 0; t < 8; ++t) {
+                const int64_t row = m0 + acc_row(wm, i, 2 * t, lane) + (odd ? 1 : 0);
+                // a lane past the last row still takes part in the exchange below: its neighbour
+                // holds the row before it and needs this lane's half of that row
+                const bool row_ok = row < m_valid;
+                const int64_t dst_row = (row_ok && out_rows) ? (int64_t)out_rows[row] : row;
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
+                for (int j = 0; j < 4; ++j) {
+                    const int64_t col = n0 + (acc_col(wn, j, lane) & ~1);
                     const float own0 = acc[i][j][2 * t], own1 = acc[i][j][2 * t + 1];
                     const float send = odd ? own0 : own1;
                     const float recv = __int_as_float(
                         __builtin_amdgcn_mov_dpp(__float_as_int(send), 0xB1 /* quad_perm 1,0,3,2 */, 0xF, 0xF, true));
                     float lo = odd ? recv : own0, hi = odd ? own1 : recv;
-                    const int64_t row = m0 + acc_row(wm, i, 2 * t, lane) + (odd ? 1 : 0);
-                    if (row >= m_valid || col >= N) continue;
-                    const int64_t o = row * ldo + col;
+                    if (!row_ok || col >= N) continue;
+                    const int64_t o = row * ldo + col, d = dst_row * ldo + col;
                     if (col + 1 < N) {
                         if (mode == 3) {
                             const float2 part = *reinterpret_cast<const float2*>(out_f32 + o);
                             lo += part.x;
                             hi += part.y;
                         }
-                        *reinterpret_cast<uint32_t*>(out_bf16 + o) = oi_pack_bf16x2(lo, hi);
+                        *reinterpret_cast<uint32_t*>(out_bf16 + d) = oi_pack_bf16x2(lo, hi);
                     } else {
                         if (mode == 3) lo += out_f32[o];
-                        out_bf16[o] = (uint16_t)oi_f32_to_bf16_bits(lo);
+                        out_bf16[d] = (uint16_t)oi_f32_to_bf16_bits(lo);
                     }
                 }
             }
@@ -743,27 +777,48 @@ __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B,
                 float v = acc[i][j][r];
                 if (mode == 1 || mode == 3) v += out_f32[o];
                 if (mode <= 1) out_f32[o] = v;
-                else out_bf16[o] = (uint16_t)oi_f32_to_bf16_bits(v);
+                else out_bf16[(out_rows ? (int64_t)out_rows[row] : row) * ldo + col] = (uint16_t)oi_f32_to_bf16_bits(v);
             }
         }
 }
+
+// Sizes that depend on a row count which only the device knows (rows selected by a mask).
+//   role 1 (d_hidden = dZ * W, rows of the product are tokens):  M, m_valid and A's extent follow n
+//   role 2 (d_weight = dZ^T * hidden, the k dimension is tokens): K and the operands' k extents follow n
+struct DynRows {
+    const int32_t* n_dev;
+    int role;
+    const int32_t* out_rows;
+};
 
 // `queue` null: one workgroup per tile id (blockIdx); otherwise a launch of resident workgroups
 // that draw their tiles from the queue
 template <bool A_KM, bool B_KM>
 __global__ void __launch_bounds__(NTHREADS)
-    gemm_store_kernel(const Operand A, int64_t M, const Operand B, int64_t N, int64_t K, int mode, float* out_f32,
-                      uint16_t* out_bf16, int64_t ldo, int64_t m_valid, uint32_t* __restrict__ queue) {
+    gemm_store_kernel(Operand A, int64_t M, Operand B, int64_t N, int64_t K, int mode, float* out_f32,
+                      uint16_t* out_bf16, int64_t ldo, int64_t m_valid, DynRows dyn, uint32_t* __restrict__ queue) {
     __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
+    if (dyn.n_dev) {
+        const int64_t n = *dyn.n_dev;
+        if (dyn.role == 1) {
+            M = (n + BM - 1) / BM * BM;
+            m_valid = n;
+            A.extent = M;
+        } else if (dyn.role == 2) {
+            K = (n + BK - 1) / BK * BK;
+            A.k_valid = (n + BM - 1) / BM * BM;
+            B.k_valid = n;
+        }
+    }
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (queue) {
         for_each_tile(queue, tiles_m, tiles_n, lds, [&](int64_t tm, int64_t tn) {
-            gemm_store_tile<A_KM, B_KM>(A, M, B, N, K, mode, out_f32, out_bf16, ldo, m_valid, tm, tn, lds);
+            gemm_store_tile<A_KM, B_KM>(A, M, B, N, K, mode, out_f32, out_bf16, ldo, m_valid, dyn.out_rows, tm, tn, lds);
         });
     } else {
         int64_t tm, tn;
         if (tile_of_block(tiles_m, tiles_n, &tm, &tn))
-            gemm_store_tile<A_KM, B_KM>(A, M, B, N, K, mode, out_f32, out_bf16, ldo, m_valid, tm, tn, lds);
+            gemm_store_tile<A_KM, B_KM>(A, M, B, N, K, mode, out_f32, out_bf16, ldo, m_valid, dyn.out_rows, tm, tn, lds);
     }
 }
 
@@ -774,28 +829,128 @@ __global__ void zero_words_kernel(uint32_t* __restrict__ p, int n) {
     if (i < n) p[i] = 0u;
 }
 
+// ---------------------------------------------------------------------------------------------
+// row selection: which token rows are multiplied at all
+// ---------------------------------------------------------------------------------------------
+// Row i takes part when its mask byte is set (no mask: every row) and, in the backward pass when
+// asked for, when its upstream gradient is not exactly zero.  The selection is made on the device
+// and stays there: the host sizes grids and buffers for all n rows and every kernel reads the
+// selected count from memory, so no call ever waits for the GPU.
+__device__ __forceinline__ bool row_selected(const uint8_t* __restrict__ mask, const float* __restrict__ grad,
+                                             int64_t i) {
+    return (!mask || mask[i] != 0) && (!grad || grad[i] != 0.f);
+}
+
+constexpr int SELECT_THREADS = 1024;
+// One workgroup: rows[0 .. count) = positions of the selected rows in ascending order (a stable
+// compaction: count per thread segment, block scan, write).  Also clears `n_zero` (<= 1024) queue
+// words for the launches that follow.
+__global__ void __launch_bounds__(SELECT_THREADS)
+    select_rows_kernel(const uint8_t* __restrict__ mask, const float* __restrict__ grad, int64_t n,
+                       int32_t* __restrict__ rows, int32_t* __restrict__ count, uint32_t* __restrict__ zero_words,
+                       int n_zero) {
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int64_t per = (n + SELECT_THREADS - 1) / SELECT_THREADS;
+    const int64_t b = t * per, e = b + per < n ? b + per : n;
+    int c = 0;
+    for (int64_t i = b; i < e; ++i) c += row_selected(mask, grad, i) ? 1 : 0;
+    int incl = c;
+#pragma unroll
+    for (int off = 1; off < OI_WAVE; off <<= 1) {
+        const int o = __shfl_up(incl, off, OI_WAVE);
+        if (lane >= off) incl += o;
+    }
+    __shared__ int wave_total[SELECT_THREADS / OI_WAVE];
+    if (lane == OI_WAVE - 1) wave_total[wave] = incl;
+    __syncthreads();
+    int base = 0;
+    for (int w = 0; w < wave; ++w) base += wave_total[w];
+    int pos = base + incl - c;
+    for (int64_t i = b; i < e; ++i)
+        if (row_selected(mask, grad, i)) rows[pos++] = (int32_t)i;
+    if (t == SELECT_THREADS - 1) *count = base + incl;
+    if (t < n_zero) zero_words[t] = 0u;
+}
+
+// Workgroup j copies selected row j: the hidden-state row (hdim bf16, 16-byte pieces), its label
+// and, for the backward pass, its logsumexp and upstream gradient.
+__global__ void __launch_bounds__(256)
+    gather_rows_kernel(const uint16_t* __restrict__ hidden, const int64_t* __restrict__ labels,
+                       const float* __restrict__ lse, const float* __restrict__ grad,
+                       const int32_t* __restrict__ rows, const int32_t* __restrict__ count, int64_t hdim,
+                       uint16_t* __restrict__ hidden_c, int64_t* __restrict__ labels_c, float* __restrict__ lse_c,
+                       float* __restrict__ grad_c) {
+    const int64_t j = blockIdx.x;
+    if (j >= *count) return;
+    const int64_t src = rows[j];
+    const oi_u32x4* from = reinterpret_cast<const oi_u32x4*>(hidden + src * hdim);
+    oi_u32x4* to = reinterpret_cast<oi_u32x4*>(hidden_c + j * hdim);
+    for (int64_t c = threadIdx.x; c < hdim / 8; c += blockDim.x) to[c] = from[c];
+    if (threadIdx.x == 0) {
+        labels_c[j] = labels[src];
+        if (lse_c) lse_c[j] = lse[src];
+        if (grad_c) grad_c[j] = grad[src];
+    }
+}
+
+// d_hidden rows of tokens that took no part are zero
+__global__ void __launch_bounds__(256)
+    zero_unselected_rows_kernel(const uint8_t* __restrict__ mask, const float* __restrict__ grad, int64_t hdim,
+                                uint16_t* __restrict__ out) {
+    const int64_t i = blockIdx.x;
+    if (row_selected(mask, grad, i)) return;
+    uint32_t* row = reinterpret_cast<uint32_t*>(out + i * hdim);  // hdim is a multiple of 64
+    for (int64_t c = threadIdx.x; c < hdim / 2; c += blockDim.x) row[c] = 0u;
+}
+
 // Workgroups of a queue-driven launch: one per CU of the current device (each takes a whole CU's
 // LDS), a multiple of 8 so that every XCD gets the same number, and no more than there are tiles.
 unsigned resident_grid(int64_t tiles_m, int64_t tiles_n) {
-    static int cus_of_device[64] = {0};
+    static std::atomic<int> cus_of_device[64];  // 0 = not looked up yet; the value never changes afterwards
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-    if (cus_of_device[dev] == 0) {
-        int cus = 0;
+    int cus = cus_of_device[dev].load(std::memory_order_relaxed);
+    if (cus == 0) {
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-        cus_of_device[dev] = cus;
+        cus_of_device[dev].store(cus, std::memory_order_relaxed);
     }
-    const int64_t cus = (cus_of_device[dev] + 7) / 8 * 8;
+    const int64_t grid = (cus + 7) / 8 * 8;
     const int64_t pids = pids_for_tiles(tiles_m, tiles_n);
-    return (unsigned)(pids < cus ? pids : cus);
+    return (unsigned)(pids < grid ? pids : grid);
 }
 
 constexpr int64_t BWD_VOCAB_CHUNK = 32768;
 
+struct Carver {
+    size_t off = 0;
+    size_t take(size_t bytes) {
+        const size_t o = off;
+        off += (bytes + 255) / 256 * 256;
+        return o;
+    }
+};
+
+// buffers of a row selection: the row index, the selected count and the compacted per-row inputs
+struct SelectionPlan {
+    size_t off_rows, off_count, off_hidden, off_labels, off_lse, off_grad;
+};
+SelectionPlan plan_selection(Carver& cv, int64_t n_pad, int64_t hdim, bool backward) {
+    SelectionPlan p;
+    p.off_rows = cv.take((size_t)n_pad * sizeof(int32_t));
+    p.off_count = cv.take(sizeof(int32_t));
+    p.off_hidden = cv.take((size_t)n_pad * hdim * 2);
+    p.off_labels = cv.take((size_t)n_pad * sizeof(int64_t));
+    p.off_lse = backward ? cv.take((size_t)n_pad * sizeof(float)) : 0;
+    p.off_grad = backward ? cv.take((size_t)n_pad * sizeof(float)) : 0;
+    return p;
+}
+
 struct FwdPlan {
     int64_t token_tiles, vocab_tiles, n_splits, tiles_per_split, n_pad;
+    size_t off_partial, off_zy, off_queue, total;
+    SelectionPlan sel;
 };
-FwdPlan plan_fwd(int64_t n_tokens, int64_t vocab) {
+FwdPlan plan_fwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_selection) {
     FwdPlan p;
     p.token_tiles = (n_tokens + BN - 1) / BN;
     p.vocab_tiles = (vocab + BM - 1) / BM;
@@ -808,30 +963,33 @@ FwdPlan plan_fwd(int64_t n_tokens, int64_t vocab) {
     while (tps > 1 && ((p.vocab_tiles + tps - 1) / tps) * p.token_tiles < 512) tps /= 2;
     p.tiles_per_split = tps;
     p.n_splits = (p.vocab_tiles + p.tiles_per_split - 1) / p.tiles_per_split;
+    Carver cv;
+    p.off_partial = cv.take((size_t)p.n_splits * p.n_pad * sizeof(float4));
+    p.off_zy = cv.take((size_t)p.n_pad * sizeof(float));
+    p.off_queue = cv.take(QUEUE_WORDS * sizeof(uint32_t));
+    if (with_selection) p.sel = plan_selection(cv, p.n_pad, hdim, false);
+    p.total = cv.off;
     return p;
 }
 
 struct BwdPlan {
     int64_t n_pad, v_pad, chunk, n_chunks;
     size_t off_dz, off_dh32, off_queues, total;
+    SelectionPlan sel;
 };
-BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab) {
+BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_selection) {
     BwdPlan p;
     p.n_pad = round_up(n_tokens, 256);
     p.v_pad = round_up(vocab, 256);
     p.chunk = p.v_pad < BWD_VOCAB_CHUNK ? p.v_pad : BWD_VOCAB_CHUNK;
     p.n_chunks = (p.v_pad + p.chunk - 1) / p.chunk;
-    size_t off = 0;
-    auto take = [&](size_t bytes) {
-        size_t o = off;
-        off += (bytes + 255) / 256 * 256;
-        return o;
-    };
-    p.off_dz = take((size_t)p.n_pad * p.chunk * 2);
-    p.off_dh32 = take((size_t)n_tokens * hdim * 4);
+    Carver cv;
+    p.off_dz = cv.take((size_t)p.n_pad * p.chunk * 2);
+    p.off_dh32 = cv.take((size_t)n_tokens * hdim * 4);
     // one set of work-queue counters per tile-kernel launch (three per vocabulary chunk)
-    p.off_queues = take((size_t)(3 * p.n_chunks) * QUEUE_WORDS * sizeof(uint32_t));
-    p.total = off;
+    p.off_queues = cv.take((size_t)(3 * p.n_chunks) * QUEUE_WORDS * sizeof(uint32_t));
+    if (with_selection) p.sel = plan_selection(cv, p.n_pad, hdim, true);
+    p.total = cv.off;
     return p;
 }
 
@@ -849,75 +1007,122 @@ int check_lmhead(const void* hidden, const void* weight, const int64_t* labels, 
     return OI_OK;
 }
 
+// The per-row inputs the tile kernels read: the caller's own, or their compacted copies
+struct RowInputs {
+    const uint16_t* hidden;
+    const int64_t* labels;
+    const float *lse, *grad;
+    const int32_t *rows, *n_dev;  // null without a selection
+};
+
+// select + gather on `s`; clears `n_zero` queue words on the way
+RowInputs launch_selection(const SelectionPlan& sp, char* ws, const void* hidden, const int64_t* labels,
+                           const float* lse, const float* grad, const uint8_t* row_mask, bool skip_zero_grad,
+                           int64_t n_tokens, int64_t hdim, uint32_t* zero_words, int n_zero, hipStream_t s) {
+    int32_t* rows = reinterpret_cast<int32_t*>(ws + sp.off_rows);
+    int32_t* count = reinterpret_cast<int32_t*>(ws + sp.off_count);
+    uint16_t* hidden_c = reinterpret_cast<uint16_t*>(ws + sp.off_hidden);
+    int64_t* labels_c = reinterpret_cast<int64_t*>(ws + sp.off_labels);
+    float* lse_c = lse ? reinterpret_cast<float*>(ws + sp.off_lse) : nullptr;
+    float* grad_c = grad ? reinterpret_cast<float*>(ws + sp.off_grad) : nullptr;
+    hipLaunchKernelGGL(select_rows_kernel, dim3(1), dim3(SELECT_THREADS), 0, s, row_mask,
+                       skip_zero_grad ? grad : static_cast<const float*>(nullptr), n_tokens, rows, count, zero_words,
+                       n_zero);
+    hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s,
+                       static_cast<const uint16_t*>(hidden), labels, lse, grad, rows, count, hdim, hidden_c, labels_c,
+                       lse_c, grad_c);
+    return RowInputs{hidden_c, labels_c, lse_c, grad_c, rows, count};
+}
+
 }  // namespace
 
-extern "C" size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab) {
-    (void)hidden_dim;
-    if (n_tokens <= 0 || vocab <= 0) return 0;
-    const FwdPlan p = plan_fwd(n_tokens, vocab);
-    // partial statistics, target logits, the work-queue counters
-    return (size_t)p.n_splits * p.n_pad * sizeof(float4) + (size_t)p.n_pad * sizeof(float) +
-           QUEUE_WORDS * sizeof(uint32_t);
+extern "C" size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
+                                                int with_row_mask) {
+    if (n_tokens <= 0 || vocab <= 0 || hidden_dim <= 0) return 0;
+    return plan_fwd(n_tokens, hidden_dim, vocab, with_row_mask != 0).total;
 }
 
-extern "C" int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
-                                  int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob,
-                                  float* entropy, float* lse, void* workspace, size_t workspace_bytes, void* stream) {
-    const int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
-    if (rc != OI_OK) return rc;
-    if (n_tokens == 0) return OI_OK;
-    OI_RETURN_IF(!logprob || !workspace, OI_ENULL);
-    OI_RETURN_IF(!oi_aligned(workspace, 16), OI_EALIGN);
-    OI_RETURN_IF(workspace_bytes < oi_lmhead_fwd_workspace_bytes(n_tokens, hidden_dim, vocab), OI_EWORKSPACE);
-    const FwdPlan p = plan_fwd(n_tokens, vocab);
-    float4* partial = static_cast<float4*>(workspace);
-    float* zy = reinterpret_cast<float*>(partial + p.n_splits * p.n_pad);
-    uint32_t* queue = reinterpret_cast<uint32_t*>(zy + p.n_pad);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const float c = inv_temperature * OI_LOG2E;
-    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, queue, QUEUE_WORDS);
-    hipLaunchKernelGGL(lmhead_fwd_kernel, dim3(resident_grid(p.n_splits, p.token_tiles)), dim3(NTHREADS), 0, s,
-                       static_cast<const uint16_t*>(weight), static_cast<const uint16_t*>(hidden), labels, n_tokens,
-                       hidden_dim, vocab, c, p.n_splits, p.tiles_per_split, p.n_pad, partial, zy, queue);
-    hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
-                       zy, n_tokens, p.n_splits, p.n_pad, inv_temperature, logprob, entropy, lse);
-    return oi_launch_status();
-}
-
-extern "C" size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
-                                                int want_d_weight) {
-    if (n_tokens <= 0 || hidden_dim <= 0 || vocab <= 0) return 0;
-    (void)want_d_weight;
-    return plan_bwd(n_tokens, hidden_dim, vocab).total;
-}
-
-extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
-                                  const float* grad_logprob, int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
-                                  float inv_temperature, void* d_hidden, void* d_weight, void* workspace,
+extern "C" int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* labels,
+                                  const uint8_t* row_mask, int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
+                                  float inv_temperature, float* logprob, float* entropy, float* lse, void* workspace,
                                   size_t workspace_bytes, void* stream) {
     const int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
     if (rc != OI_OK) return rc;
     if (n_tokens == 0) return OI_OK;
+    OI_RETURN_IF(!logprob || !workspace, OI_ENULL);
+    OI_RETURN_IF(!oi_aligned(workspace, 256), OI_EALIGN);
+    const FwdPlan p = plan_fwd(n_tokens, hidden_dim, vocab, row_mask != nullptr);
+    OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
+    char* ws = static_cast<char*>(workspace);
+    float4* partial = reinterpret_cast<float4*>(ws + p.off_partial);
+    float* zy = reinterpret_cast<float*>(ws + p.off_zy);
+    uint32_t* queue = reinterpret_cast<uint32_t*>(ws + p.off_queue);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const float c = inv_temperature * OI_LOG2E;
+    RowInputs in = {static_cast<const uint16_t*>(hidden), labels, nullptr, nullptr, nullptr, nullptr};
+    if (row_mask)
+        in = launch_selection(p.sel, ws, hidden, labels, nullptr, nullptr, row_mask, false, n_tokens, hidden_dim, queue,
+                              QUEUE_WORDS, s);
+    else
+        hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, queue, QUEUE_WORDS);
+    hipLaunchKernelGGL(lmhead_fwd_kernel, dim3(resident_grid(p.n_splits, p.token_tiles)), dim3(NTHREADS), 0, s,
+                       static_cast<const uint16_t*>(weight), in.hidden, in.labels, n_tokens, in.n_dev, hidden_dim, vocab,
+                       c, p.n_splits, p.tiles_per_split, p.n_pad, partial, zy, queue);
+    hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
+                       zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, logprob,
+                       entropy, lse);
+    return oi_launch_status();
+}
+
+extern "C" size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
+                                                int want_d_weight, int with_row_selection) {
+    if (n_tokens <= 0 || hidden_dim <= 0 || vocab <= 0) return 0;
+    (void)want_d_weight;
+    return plan_bwd(n_tokens, hidden_dim, vocab, with_row_selection != 0).total;
+}
+
+extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
+                                  const float* grad_logprob, const uint8_t* row_mask, int skip_zero_grad_rows,
+                                  int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature,
+                                  void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes,
+                                  void* stream) {
+    const int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
+    if (rc != OI_OK) return rc;
+    if (n_tokens == 0) return OI_OK;
     OI_RETURN_IF(!lse || !grad_logprob || !d_hidden || !workspace, OI_ENULL);
-    OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 2) || !oi_aligned(d_weight, 2), OI_EALIGN);
+    // bf16 results are stored as pairs (4-byte words)
+    OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 4) || !oi_aligned(d_weight, 4), OI_EALIGN);
     const int want_dw = d_weight != nullptr;
-    const BwdPlan p = plan_bwd(n_tokens, hidden_dim, vocab);
+    const bool selecting = row_mask != nullptr || skip_zero_grad_rows != 0;
+    const BwdPlan p = plan_bwd(n_tokens, hidden_dim, vocab, selecting);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     hipStream_t s = static_cast<hipStream_t>(stream);
     char* ws = static_cast<char*>(workspace);
     uint16_t* dz = reinterpret_cast<uint16_t*>(ws + p.off_dz);
     float* dh32 = reinterpret_cast<float*>(ws + p.off_dh32);
     const uint16_t* Wp = static_cast<const uint16_t*>(weight);
-    const uint16_t* Hp = static_cast<const uint16_t*>(hidden);
     const float c = inv_temperature * OI_LOG2E;
 
     uint32_t* queues = reinterpret_cast<uint32_t*>(ws + p.off_queues);
     const int n_queue_words = (int)(3 * p.n_chunks * QUEUE_WORDS);
-    hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_queue_words + 255) / 256)), dim3(256), 0, s, queues,
-                       n_queue_words);
+    RowInputs in = {static_cast<const uint16_t*>(hidden), labels, lse, grad_logprob, nullptr, nullptr};
+    if (selecting && n_queue_words <= SELECT_THREADS) {
+        in = launch_selection(p.sel, ws, hidden, labels, lse, grad_logprob, row_mask, skip_zero_grad_rows != 0, n_tokens,
+                              hidden_dim, queues, n_queue_words, s);
+    } else {
+        hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_queue_words + 255) / 256)), dim3(256), 0, s, queues,
+                           n_queue_words);
+        if (selecting)
+            in = launch_selection(p.sel, ws, hidden, labels, lse, grad_logprob, row_mask, skip_zero_grad_rows != 0,
+                                  n_tokens, hidden_dim, queues, 0, s);
+    }
+    if (selecting)
+        hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, row_mask,
+                           skip_zero_grad_rows ? grad_logprob : static_cast<const float*>(nullptr), hidden_dim,
+                           static_cast<uint16_t*>(d_hidden));
 
     // Per vocabulary chunk: dZ [n_pad, cols] (token-major, bf16, zero in padded rows and columns),
-    // then both products straight from the caller's W and hidden, which enter as k-major operands:
+    // then both products straight from W and the (selected) hidden rows, which enter as k-major operands:
     //   d_hidden[n, h] (+)= sum_v dZ[n, v] * W[v_begin + v, h]      A k-contiguous, B k-major
     //   d_weight[v_begin + v, h] = sum_n dZ[n, v] * hidden[n, h]    A k-major,      B k-major
     // The sums stop at the last real vocabulary row / token (rounded up to a k-tile, whose missing
@@ -929,24 +1134,26 @@ extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const 
         const int64_t valid = vocab - v_begin < cols ? vocab - v_begin : cols;               // real rows of W
         uint32_t* q = queues + ci * 3 * QUEUE_WORDS;
         hipLaunchKernelGGL(lmhead_dz_kernel, dim3(resident_grid(cols / BM, p.n_pad / BN)), dim3(NTHREADS), 0, s, Wp,
-                           Hp, labels, lse, grad_logprob, n_tokens, hidden_dim, vocab, c, inv_temperature, v_begin,
-                           cols, p.n_pad, dz, q);
+                           in.hidden, in.labels, in.lse, in.grad, n_tokens, in.n_dev, hidden_dim, vocab, c,
+                           inv_temperature, v_begin, cols, p.n_pad, dz, q);
         const bool first = ci == 0, last = ci == p.n_chunks - 1;
         const int mode = last ? (first ? 2 : 3) : (first ? 0 : 1);
         {
             const Operand a = {dz, cols, 0, p.n_pad, cols};
             const Operand b = {Wp + v_begin * hidden_dim, hidden_dim, 0, hidden_dim, valid};
+            const DynRows dyn = {in.n_dev, 1, in.rows};
             hipLaunchKernelGGL((gemm_store_kernel<false, true>), dim3(resident_grid(p.n_pad / BM, h_tiles)),
                                dim3(NTHREADS), 0, s, a, p.n_pad, b, hidden_dim, round_up(valid, BK), mode, dh32,
-                               static_cast<uint16_t*>(d_hidden), hidden_dim, n_tokens, q + QUEUE_WORDS);
+                               static_cast<uint16_t*>(d_hidden), hidden_dim, n_tokens, dyn, q + QUEUE_WORDS);
         }
         if (want_dw) {
             const Operand a = {dz, cols, 0, cols, p.n_pad};
-            const Operand b = {Hp, hidden_dim, 0, hidden_dim, n_tokens};
+            const Operand b = {in.hidden, hidden_dim, 0, hidden_dim, n_tokens};
+            const DynRows dyn = {in.n_dev, 2, nullptr};
             hipLaunchKernelGGL((gemm_store_kernel<true, true>), dim3(resident_grid(cols / BM, h_tiles)),
                                dim3(NTHREADS), 0, s, a, cols, b, hidden_dim, round_up(n_tokens, BK), 2,
                                static_cast<float*>(nullptr), static_cast<uint16_t*>(d_weight) + v_begin * hidden_dim,
-                               hidden_dim, valid, q + 2 * QUEUE_WORDS);
+                               hidden_dim, valid, dyn, q + 2 * QUEUE_WORDS);
         }
     }
     return oi_launch_status();
@@ -966,7 +1173,7 @@ extern "C" int oi_gemm_bf16_tn(const void* A, int64_t lda, int64_t M, const void
     const Operand b = {static_cast<const uint16_t*>(B), ldb, 0, N, K};
     hipLaunchKernelGGL((gemm_store_kernel<false, false>), dim3(grid_for_tiles((M + BM - 1) / BM, (N + BN - 1) / BN)),
                        dim3(NTHREADS), 0, static_cast<hipStream_t>(stream), a, M, b, N, K, mode, out_f32,
-                       static_cast<uint16_t*>(out_bf16), ldo, M, static_cast<uint32_t*>(nullptr));
+                       static_cast<uint16_t*>(out_bf16), ldo, M, DynRows{nullptr, 0, nullptr}, static_cast<uint32_t*>(nullptr));
     return oi_launch_status();
 }
 
@@ -988,17 +1195,18 @@ extern "C" int oi_gemm_bf16_layouts(const void* A, int64_t lda, int a_k_major, c
     hipStream_t s = static_cast<hipStream_t>(stream);
     uint16_t* o16 = static_cast<uint16_t*>(out_bf16);
     uint32_t* no_queue = nullptr;
+    const DynRows fixed = {nullptr, 0, nullptr};
     if (a_k_major && b_k_major)
         hipLaunchKernelGGL((gemm_store_kernel<true, true>), grid, dim3(NTHREADS), 0, s, a, M, b, N, K, mode, out_f32, o16,
-                           ldo, M, no_queue);
+                           ldo, M, fixed, no_queue);
     else if (a_k_major)
         hipLaunchKernelGGL((gemm_store_kernel<true, false>), grid, dim3(NTHREADS), 0, s, a, M, b, N, K, mode, out_f32,
-                           o16, ldo, M, no_queue);
+                           o16, ldo, M, fixed, no_queue);
     else if (b_k_major)
         hipLaunchKernelGGL((gemm_store_kernel<false, true>), grid, dim3(NTHREADS), 0, s, a, M, b, N, K, mode, out_f32,
-                           o16, ldo, M, no_queue);
+                           o16, ldo, M, fixed, no_queue);
     else
         hipLaunchKernelGGL((gemm_store_kernel<false, false>), grid, dim3(NTHREADS), 0, s, a, M, b, N, K, mode, out_f32,
-                           o16, ldo, M, no_queue);
+                           o16, ldo, M, fixed, no_queue);
     return oi_launch_status();
 }

@@ -19,8 +19,8 @@ from . import _lib
 
 class _FusedLMHead(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, labels, inv_temperature, want_entropy, compact_backward=False):
-        dev = _lib.require_gpu(hidden, weight, labels)
+    def forward(ctx, hidden, weight, labels, mask, inv_temperature, want_entropy, compact_backward=False):
+        dev = _lib.require_gpu(hidden, weight, labels, mask)
         if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
             raise ValueError("fused lm_head expects bf16 hidden states and weight")
         if hidden.ndim != 2 or weight.ndim != 2 or hidden.shape[1] != weight.shape[1]:
@@ -33,17 +33,23 @@ class _FusedLMHead(torch.autograd.Function):
         lab = labels.reshape(-1).to(torch.int64).contiguous()
         if lab.numel() != n:
             raise ValueError(f"{lab.numel()} labels for {n} hidden rows")
+        m = None
+        if mask is not None:
+            m = _lib.mask_u8(mask.reshape(-1))
+            if m.numel() != n:
+                raise ValueError(f"mask of {m.numel()} entries for {n} hidden rows")
         logprob = torch.empty(n, dtype=torch.float32, device=dev)
         entropy = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
         lse = torch.empty(n, dtype=torch.float32, device=dev)
         if n > 0:
-            ws_bytes = _lib.load().oi_lmhead_fwd_workspace_bytes(n, h, v)
+            ws_bytes = _lib.load().oi_lmhead_fwd_workspace_bytes(n, h, v, int(m is not None))
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
             _lib.call(
-                "oi_lmhead_logp_fwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), n, h, v, inv_temperature,
-                logprob.data_ptr(), _lib.ptr(entropy), lse.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
+                "oi_lmhead_logp_fwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), _lib.ptr(m), n, h, v,
+                inv_temperature, logprob.data_ptr(), _lib.ptr(entropy), lse.data_ptr(), ws.data_ptr(), ws_bytes,
+                _lib.stream_of(hid),
             )  # fmt: skip
-        ctx.save_for_backward(hid, w, lab, lse)
+        ctx.save_for_backward(hid, w, lab, lse, m)
         ctx.inv_temperature = inv_temperature
         ctx.compact_backward = bool(compact_backward)
         if want_entropy:
@@ -52,38 +58,27 @@ class _FusedLMHead(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_logprob, _grad_entropy):
-        hid, w, lab, lse = ctx.saved_tensors
+        hid, w, lab, lse, m = ctx.saved_tensors
         n, h = hid.shape
         v = w.shape[0]
         need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if grad_logprob is None or not (need_h or need_w):
-            return None, None, None, None, None, None
+            return None, None, None, None, None, None, None
         g = _lib.f32c(grad_logprob)
-        keep = None
-        if ctx.compact_backward and n > 0:
-            # rows whose upstream gradient is exactly zero (zero advantage, clipped ratio with no KL
-            # term) contribute nothing to either gradient: leave them out of the three products.
-            # torch.nonzero synchronises with the host, which is why this is opt-in.
-            nz = torch.nonzero(g != 0, as_tuple=False).squeeze(1)
-            if nz.numel() < n:
-                keep, full_n = nz, n
-                hid, lab, lse, g = hid.index_select(0, nz), lab.index_select(0, nz), lse.index_select(0, nz), g.index_select(0, nz)
-                n = nz.numel()
         d_hidden = torch.empty_like(hid)
         d_weight = torch.empty_like(w) if need_w else None
         if n > 0:
-            ws_bytes = _lib.load().oi_lmhead_bwd_workspace_bytes(n, h, v, int(need_w))
+            selecting = m is not None or ctx.compact_backward
+            ws_bytes = _lib.load().oi_lmhead_bwd_workspace_bytes(n, h, v, int(need_w), int(selecting))
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=hid.device)
             _lib.call(
-                "oi_lmhead_logp_bwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), lse.data_ptr(), g.data_ptr(), n, h,
-                v, ctx.inv_temperature, d_hidden.data_ptr(), _lib.ptr(d_weight), ws.data_ptr(), ws_bytes,
-                _lib.stream_of(hid),
+                "oi_lmhead_logp_bwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), lse.data_ptr(), g.data_ptr(),
+                _lib.ptr(m), int(ctx.compact_backward), n, h, v, ctx.inv_temperature, d_hidden.data_ptr(),
+                _lib.ptr(d_weight), ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
             )  # fmt: skip
         elif d_weight is not None:
             d_weight.zero_()
-        if keep is not None:
-            d_hidden = torch.zeros(full_n, h, dtype=d_hidden.dtype, device=d_hidden.device).index_copy_(0, keep, d_hidden)
-        return (d_hidden if need_h else None), d_weight, None, None, None, None
+        return (d_hidden if need_h else None), d_weight, None, None, None, None, None
 
 
 def fused_lm_head_logprobs(
@@ -101,11 +96,12 @@ def fused_lm_head_logprobs(
     ``labels`` int64 with the leading shape of ``hidden``; negative labels are scored as token 0
     (the reference's ``clamp(min=0)``, open_instruct/padding_free_collator.py:15).  ``mask`` (bool,
     same leading shape) selects the rows that are computed at all: masked-out rows cost nothing,
-    return 0 and receive a zero gradient.  Differentiable with respect to ``hidden`` and
-    ``weight``; the entropy carries no gradient, as in the reference.  ``compact_backward=True``
-    additionally drops rows whose upstream gradient is exactly zero from the backward products
-    (zero-advantage completions, clipped ratios without a KL term); it costs one host
-    synchronisation in the backward pass and changes no result.
+    return 0 and receive a zero gradient.  The selection is made on the device (a row index built
+    from the mask, the selected rows gathered into the workspace), so neither pass waits for the
+    GPU.  Differentiable with respect to ``hidden`` and ``weight``; the entropy carries no
+    gradient, as in the reference.  ``compact_backward=True`` additionally leaves rows whose
+    upstream gradient is exactly zero (zero-advantage completions, clipped ratios without a KL
+    term) out of the backward products; it changes no result.
     """
     lead = hidden.shape[:-1]
     hid2 = hidden.reshape(-1, hidden.shape[-1])
@@ -113,20 +109,10 @@ def fused_lm_head_logprobs(
     inv_t = 1.0 / float(temperature)
     if not float(temperature) > 0.0:
         raise ValueError(f"temperature must be positive, got {temperature}")
-    if mask is None:
-        lp, ent = _FusedLMHead.apply(hid2, weight, lab1, inv_t, return_entropy, compact_backward)
-        return lp.reshape(lead), (ent.reshape(lead) if ent is not None else None)
-    keep = mask.reshape(-1).bool()
-    idx = torch.nonzero(keep, as_tuple=False).squeeze(1)
-    lp_c, ent_c = _FusedLMHead.apply(
-        hid2.index_select(0, idx), weight, lab1.index_select(0, idx), inv_t, return_entropy, compact_backward
-    )
-    lp = torch.zeros(hid2.shape[0], dtype=torch.float32, device=hidden.device).index_copy(0, idx, lp_c)
-    ent = None
-    if ent_c is not None:
-        ent = torch.zeros(hid2.shape[0], dtype=torch.float32, device=hidden.device).index_copy(0, idx, ent_c)
-        ent = ent.reshape(lead)
-    return lp.reshape(lead), ent
+    if mask is not None and tuple(mask.shape) != tuple(lead):
+        raise ValueError(f"mask {tuple(mask.shape)} does not match the rows of hidden {tuple(lead)}")
+    lp, ent = _FusedLMHead.apply(hid2, weight, lab1, mask, inv_t, return_entropy, compact_backward)
+    return lp.reshape(lead), (ent.reshape(lead) if ent is not None else None)
 
 
 def fused_linear_cross_entropy(

@@ -219,3 +219,68 @@ def test_compact_backward_leaves_gradients_unchanged():
     out, _ = lm_head.fused_lm_head_logprobs(dh, dw, labels.to(DEV), compact_backward=True)
     out.backward(torch.zeros(600, device=DEV))
     assert not dh.grad.any() and not dw.grad.any()
+
+
+@pytest.mark.parametrize("keep", ["none", "one", "all", "random", "last_tile_only"])
+@pytest.mark.parametrize("want_dw", [True, False])
+def test_row_selection_on_device(keep, want_dw):
+    """The mask is turned into a row index on the device (no host read of the count): forward and
+    backward against the oracle for an empty selection, a single row, every row, a random subset and a
+    subset that lives in the last token tile; rows left out return 0 and get a zero gradient, and an
+    upstream gradient on a row that was left out must be ignored."""
+    n, h, v = 700, 128, 3000
+    hidden, weight, labels = _case(n, h, v, seed=21, w_scale=3.0 / math.sqrt(h))
+    g = torch.Generator().manual_seed(22)
+    mask = {
+        "none": torch.zeros(n, dtype=torch.bool),
+        "one": torch.arange(n) == 377,
+        "all": torch.ones(n, dtype=torch.bool),
+        "random": torch.rand(n, generator=g) < 0.6,
+        "last_tile_only": torch.arange(n) >= 690,
+    }[keep]
+    upstream = torch.randn(n, generator=g)  # non-zero also on the rows that are left out
+    rh = hidden.float().requires_grad_(True)
+    rw = weight.float().requires_grad_(True)
+    lp_o, ent_o = o_lm.lm_head_logprobs(rh, rw, labels, 0.9, True)
+    (lp_o * mask).backward(upstream)
+    dh = hidden.to(DEV).requires_grad_(True)
+    dw = weight.to(DEV).requires_grad_(want_dw)
+    lp, ent = lm_head.fused_lm_head_logprobs(dh, dw, labels.to(DEV), 0.9, mask=mask.to(DEV), return_entropy=True)
+    lp.backward(upstream.to(DEV))
+    assert ((lp.detach().cpu() - lp_o.detach()) * mask).abs().max().item() <= TOL
+    assert ((ent.cpu() - ent_o) * mask).abs().max().item() <= TOL
+    assert (lp.detach().cpu()[~mask] == 0).all() and (ent.cpu()[~mask] == 0).all()
+    assert (dh.grad.cpu()[~mask] == 0).all()
+    assert (dh.grad.float().cpu() - rh.grad).abs().max().item() <= TOL + rh.grad.abs().max().item() * 2**-7
+    if mask.any():
+        assert ((dh.grad.float().cpu() - rh.grad).norm() / rh.grad.norm()).item() <= 2e-2
+    if want_dw:
+        assert (dw.grad.float().cpu() - rw.grad).abs().max().item() <= TOL + rw.grad.abs().max().item() * 2**-7
+        if mask.any():
+            assert ((dw.grad.float().cpu() - rw.grad).norm() / rw.grad.norm()).item() <= 2e-2
+        else:
+            assert not dw.grad.any()
+
+
+def test_row_selection_with_compact_backward_and_mask():
+    """Mask and zero-gradient rows together: the backward selects rows that are in the mask AND carry
+    a gradient."""
+    n, h, v = 900, 64, 40000  # two vocabulary chunks
+    hidden, weight, labels = _case(n, h, v, seed=23, w_scale=3.0 / math.sqrt(h))
+    g = torch.Generator().manual_seed(24)
+    mask = torch.rand(n, generator=g) < 0.7
+    upstream = torch.randn(n, generator=g)
+    upstream[torch.rand(n, generator=g) < 0.5] = 0.0
+    rh = hidden.float().requires_grad_(True)
+    rw = weight.float().requires_grad_(True)
+    lp_o, _ = o_lm.lm_head_logprobs(rh, rw, labels, 1.0)
+    (lp_o * mask).backward(upstream)
+    dh = hidden.to(DEV).requires_grad_(True)
+    dw = weight.to(DEV).requires_grad_(True)
+    lp, _ = lm_head.fused_lm_head_logprobs(dh, dw, labels.to(DEV), mask=mask.to(DEV), compact_backward=True)
+    lp.backward(upstream.to(DEV))
+    dead = ~mask | (upstream == 0)
+    assert (dh.grad.cpu()[dead] == 0).all()
+    assert ((dh.grad.float().cpu() - rh.grad).norm() / rh.grad.norm()).item() <= 2e-2
+    assert ((dw.grad.float().cpu() - rw.grad).norm() / rw.grad.norm()).item() <= 2e-2
+    assert (dw.grad.float().cpu() - rw.grad).abs().max().item() <= TOL + rw.grad.abs().max().item() * 2**-7
