@@ -16,6 +16,7 @@ from . import (  # noqa: F401
     lm_head,
     model_utils,
     olmo_core_train_modules,
+    olmo_core_utils,
     padding_free_collator,
     rl_utils,
 )

@@ -17,7 +17,7 @@ from dataclasses import dataclass, field
 
 import torch
 
-from . import _lib, model_utils
+from . import _lib, model_utils, olmo_core_utils
 from .rl_utils import masked_mean
 
 INVALID_LOGPROB = 1.0  # open_instruct/utils.py:83
@@ -592,13 +592,18 @@ def forward_for_logprobs(
     Differences from the reference that do not change results: the temperature is applied inside
     the kernel instead of through a scaled copy of the logits, the ``[:, :-1]`` slice is an
     argument of the kernel instead of a view, and entropy comes out of the same pass over the
-    logits as the logprob.  ``pass_olmo_core_doc_lens`` needs ``doc_lens`` derived from the
-    attention mask, which lives in the model-plumbing layer outside this package: pass a model
-    whose forward accepts ``attention_mask`` instead.
+    logits as the logprob.  With ``pass_olmo_core_doc_lens`` the integer-coded attention mask is
+    turned into ``doc_lens`` / ``max_doc_lens`` for models with the olmo-core interface and no
+    attention mask is passed, as in the reference.
     """
+    extra_kwargs = {}
     if pass_olmo_core_doc_lens:
-        raise NotImplementedError("doc_lens plumbing for olmo-core models is outside this package")
-    output = model(input_ids=query_responses, attention_mask=attention_mask, position_ids=position_ids)
+        if attention_mask is None:
+            raise AssertionError("pass_olmo_core_doc_lens needs the integer-coded attention mask")
+        doc_lens, max_doc_lens = olmo_core_utils.doc_lens_from_attention_mask(attention_mask)
+        extra_kwargs = {"doc_lens": doc_lens, "max_doc_lens": max_doc_lens}
+        attention_mask = None
+    output = model(input_ids=query_responses, attention_mask=attention_mask, position_ids=position_ids, **extra_kwargs)
     logits = getattr(output, "logits", output)
     labels = query_responses[:, 1:].clone().to(logits.device)
     labels[labels == pad_token_id] = 0

@@ -32,7 +32,16 @@ class DPOLMHead(torch.nn.Module):
     ``output.loss[b, i] = log p(labels[b, i+1] | x[b, i])`` with the label shift done internally,
     as ``calculate_per_token_logps`` does (open_instruct/padding_free_collator.py:10-16).  The
     ``[B, T, V]`` logits are never formed when labels are given.
+
+    Positions whose next label is ``ignore_index`` (prompt and padding tokens, the last position)
+    are not multiplied at all: their entry of ``output.loss`` is 0 and they receive no gradient.
+    The reference scores token 0 there (its ``clamp(min=0)``) and throws the number away when the
+    per-sequence sums mask those positions (open_instruct/dpo_utils.py:689-712,
+    open_instruct/padding_free_collator.py:202-229), so every result downstream is the same; set
+    ``score_ignored_positions = True`` on the module to reproduce the discarded numbers too.
     """
+
+    score_ignored_positions = False
 
     def __init__(self, d_model: int, vocab_size: int, bias: bool = False, norm: torch.nn.Module | None = None,
                  dtype: torch.dtype = torch.bfloat16, device=None):  # fmt: skip
@@ -60,7 +69,8 @@ class DPOLMHead(torch.nn.Module):
             # no labels: the parent class returns plain logits (library GEMM; not the fused path)
             return self.w_out(h)
         shifted = padding_free_collator.shift_labels(labels)
-        per_token_logps, _ = lm_head.fused_lm_head_logprobs(h, self.w_out.weight, shifted)
+        keep = None if self.score_ignored_positions else shifted != ignore_index
+        per_token_logps, _ = lm_head.fused_lm_head_logprobs(h, self.w_out.weight, shifted, mask=keep)
         return LMOutputWithLoss(
             logits=None, loss=per_token_logps, ce_loss=per_token_logps.detach().clone(), z_loss=None
         )

@@ -136,7 +136,13 @@ def test_dpo_lm_head_matches_calculate_per_token_logps():
     )
     assert output.logits is None and output.z_loss is None
     assert output.loss.shape == (batch, seq) and output.loss.requires_grad and not output.ce_loss.requires_grad
-    assert (output.loss.detach().cpu() - expected).abs().max().item() <= TOL
+    # positions whose next label is ignored are not multiplied: 0 there, the reference's value elsewhere
+    kept = (o_logprob.shift_labels(labels.cpu()) != -100)
+    assert ((output.loss.detach().cpu() - expected) * kept).abs().max().item() <= TOL
+    assert (output.loss.detach().cpu()[~kept] == 0).all() and (~kept).sum() == 2 + batch
+    head.score_ignored_positions = True  # the reference's numbers at the ignored positions too
+    assert (head(x, labels=labels).loss.detach().cpu() - expected).abs().max().item() <= TOL
+    head.score_ignored_positions = False
     logits = head(x[:1], labels=None)
     assert isinstance(logits, torch.Tensor) and logits.shape == (1, seq, vocab) and torch.equal(logits, raw[:1])
 

@@ -485,6 +485,62 @@ def test_forward_for_logprobs_and_compute_logprobs_with_mock_model():
     counts = grpo_utils.calculate_token_counts(1, data, torch.device(DEV))
     assert counts == {0: float(mask[:, 1:].sum()), 1: 0.0}
 
+    # models with the olmo-core interface get doc_lens / max_doc_lens instead of the attention mask
+    seen = {}
+
+    class OlmoModel(Model):
+        def forward(self, input_ids, attention_mask=None, position_ids=None, doc_lens=None, max_doc_lens=None):
+            seen.update(attention_mask=attention_mask, doc_lens=doc_lens, max_doc_lens=max_doc_lens)
+            return self.z[: input_ids.shape[0]]
+
+    att = torch.tensor([[1, 1, 2, 2, 0], [1, 2, 2, 2, 2]], device=DEV)
+    lp3, _ = grpo_utils.forward_for_logprobs(OlmoModel(), qr.to(DEV), att, pos.to(DEV), 0, 1.0, pass_olmo_core_doc_lens=True)
+    assert seen["attention_mask"] is None and seen["doc_lens"].tolist() == [[2, 2, 1], [1, 4, 0]] and seen["max_doc_lens"] == [2, 4]
+    assert torch.equal(lp3, lp1)
+    data.attention_masks[:] = [att, att]
+    out3 = grpo_utils.compute_logprobs(OlmoModel(), data, pad_token_id=0, temperature=1.0, pass_olmo_core_doc_lens=True)
+    assert torch.equal(out3[0], out[0].detach()) and seen["doc_lens"].shape[0] == b
+
+
+def test_separate_and_concatenated_forward_agree_and_pass_aux_loss():
+    """open_instruct/dpo_utils.py:826-956: two forwards or one give the same per-sequence logps; with
+    output_router_logits the model's aux_loss is handed on (concatenated: as is, separate: both sides
+    concatenated)."""
+    torch.manual_seed(5)
+    vocab = 50
+    table = torch.randn(vocab, vocab, device=DEV)
+
+    class Out:
+        def __init__(self, logits, aux):
+            self.logits, self.aux_loss = logits, aux
+
+    class Model(torch.nn.Module):
+        def forward(self, input_ids, attention_mask=None, output_router_logits=False):
+            return Out(table[input_ids], torch.tensor([0.25], device=DEV) if output_router_logits else None)
+
+    batch = {
+        "chosen_input_ids": torch.randint(1, vocab, (3, 9), device=DEV), "rejected_input_ids": torch.randint(1, vocab, (3, 6), device=DEV),
+        "chosen_attention_mask": torch.ones(3, 9, dtype=torch.long, device=DEV),
+        "rejected_attention_mask": torch.ones(3, 6, dtype=torch.long, device=DEV),
+    }  # fmt: skip
+    batch["chosen_labels"] = batch["chosen_input_ids"].clone()
+    batch["rejected_labels"] = batch["rejected_input_ids"].clone()
+    batch["chosen_labels"][:, :3] = -100
+    batch["rejected_labels"][:, :2] = -100
+    for average in (False, True):
+        c1, r1, aux1 = dpo_utils.concatenated_forward(Model(), batch, average_log_prob=average)
+        c2, r2, aux2 = dpo_utils.separate_forward(Model(), batch, average_log_prob=average)
+        assert aux1 is None and aux2 is None
+        _close(c1, c2)
+        _close(r1, r2)
+        for side, got in (("chosen", c1), ("rejected", r1)):
+            per_token = o_logprob.calculate_per_token_logps(table[batch[f"{side}_input_ids"]].cpu(), batch[f"{side}_labels"].cpu())
+            _close(got, o_red.get_batch_logps_padded(per_token, batch[f"{side}_labels"].cpu(), average), 1e-5)
+    _, _, aux = dpo_utils.concatenated_forward(Model(), batch, output_router_logits=True)
+    assert aux.tolist() == [0.25]
+    _, _, aux = dpo_utils.separate_forward(Model(), batch, output_router_logits=True)
+    assert aux.tolist() == [0.25, 0.25]
+
 
 @pytest.mark.parametrize("shape", [(3, 9), (1, 1), (4, 5000)])
 def test_vllm_local_debug_metrics_parity(shape):

@@ -267,3 +267,95 @@ def test_full_size_properties_fused_head():
     # of dZ is off by up to one bf16 rounding of g: |dHidden| <= 2^-8 |g| max|w|
     bound = 2**-8 * up[:300].abs().max().item() * same.float().abs().max().item() + 1e-6
     assert dh2.grad.float().abs().max().item() <= bound
+
+
+@pytest.mark.parametrize("packing", [False, True])
+@pytest.mark.parametrize("average_log_prob", [False, True])
+def test_concatenated_forward_olmo_through_dpo_lm_head(packing, average_log_prob):
+    """Call stack of the olmo-core DPO trainer (open_instruct/olmo_core_train_modules.py:190-207):
+    concatenated_forward_olmo (open_instruct/dpo_utils.py:959-1019) -> model(ids, labels=...) whose LM
+    head is DPOLMHead (open_instruct/olmo_core_train_modules.py:48-85) -> per-sequence logps -> dpo_loss,
+    forward and backward, against the oracle chain on materialised fp32 logits."""
+    from open_instruct_amd.olmo_core_train_modules import DPOLMHead
+
+    torch.manual_seed(31)
+    d_model, vocab, pairs = 64, 1500, 2
+
+    class TinyOlmo(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.embed = torch.nn.Embedding(vocab, d_model, dtype=torch.bfloat16)
+            self.lm_head = DPOLMHead(d_model=d_model, vocab_size=vocab)
+            self.seen = {}
+
+        def forward(self, input_ids, labels=None, position_ids=None, doc_lens=None, max_doc_lens=None):
+            self.seen = {"doc_lens": doc_lens, "max_doc_lens": max_doc_lens, "position_ids": position_ids}
+            return self.lm_head(self.embed(input_ids), labels=labels)
+
+    model = TinyOlmo().to(DEV)
+    with torch.no_grad():
+        model.lm_head.w_out.weight.mul_(6.0)
+
+    def side(lengths, prompt):
+        ids = [torch.randint(1, vocab, (n,)) for n in lengths]
+        labs = [t.clone() for t in ids]
+        for lab in labs:
+            lab[:prompt] = -100
+        return ids, labs
+
+    c_ids, c_labs = side([11, 17], 4)
+    r_ids, r_labs = side([9, 23], 4)
+    if packing:
+        def pack(ids, labs):
+            lens = torch.tensor([len(t) for t in ids])
+            cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32)
+            pos = torch.cat([torch.arange(n) for n in lens.tolist()])
+            return {"input_ids": torch.cat(ids)[None], "labels": torch.cat(labs)[None], "cu_seq_lens_q": cu,
+                    "cu_seq_lens_k": cu, "max_length_q": int(lens.max()), "max_length_k": int(lens.max()),
+                    "position_ids": pos[None]}  # fmt: skip
+
+        batch = {f"chosen_{k}": v for k, v in pack(c_ids, c_labs).items()}
+        batch |= {f"rejected_{k}": v for k, v in pack(r_ids, r_labs).items()}
+    else:
+        def pad(seqs, value):
+            width = max(len(t) for t in seqs)
+            return torch.stack([torch.cat([t, torch.full((width - len(t),), value)]) for t in seqs])
+
+        batch = {"chosen_input_ids": pad(c_ids, 0), "chosen_labels": pad(c_labs, -100),
+                 "rejected_input_ids": pad(r_ids, 0), "rejected_labels": pad(r_labs, -100)}  # fmt: skip
+    batch = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in batch.items()}
+    ref_c, ref_r = -torch.rand(pairs) * 30, -torch.rand(pairs) * 30
+    beta = 0.1
+
+    chosen, rejected, aux = dpo_utils.concatenated_forward_olmo(model, batch, average_log_prob=average_log_prob, packing=packing)
+    assert aux is None and chosen.shape == (pairs,) and rejected.shape == (pairs,)
+    if packing:
+        assert model.seen["doc_lens"].tolist() == [[11, 17, 9, 23]] and model.seen["max_doc_lens"] == [23]
+        assert model.seen["position_ids"].shape == (1, 60)
+    losses, _, _ = dpo_utils.dpo_loss(chosen, rejected, ref_c.to(DEV), ref_r.to(DEV), beta)
+    losses.mean().backward()
+
+    # oracle: the same embedding rows and head weights in fp32, logits materialised
+    emb = model.embed.weight.detach().float().cpu().requires_grad_(True)
+    w = model.lm_head.w_out.weight.detach().float().cpu().requires_grad_(True)
+    if packing:
+        concat, _ = padding_free_collator.concatenated_inputs({k: (v.cpu() if torch.is_tensor(v) else v) for k, v in batch.items()})
+    else:
+        concat = dpo_utils.concatenated_inputs({k: v.cpu() for k, v in batch.items()})
+    ids, labels = concat["concatenated_input_ids"], concat["concatenated_labels"]
+    logits = torch.nn.functional.linear(emb[ids], w)
+    per_token = o_logprob.calculate_per_token_logps(logits, labels)
+    if packing:
+        seq_o = o_red.get_batch_logps_packed(per_token, labels, concat["concatenated_cu_seq_lens_k"], average_log_prob)
+    else:
+        seq_o = o_red.get_batch_logps_padded(per_token, labels, average_log_prob)
+    losses_o, _, _ = o_dpo.dpo_loss(seq_o[:pairs], seq_o[pairs:], ref_c, ref_r, beta)
+    losses_o.mean().backward()
+
+    n_kept = 1.0 if average_log_prob else 23.0
+    assert (torch.cat([chosen, rejected]).detach().cpu() - seq_o.detach()).abs().max().item() <= TOL * n_kept
+    assert (losses.detach().cpu() - losses_o.detach()).abs().max().item() <= TOL * beta * 2 * n_kept + 1e-5
+    for got, exp in ((model.lm_head.w_out.weight.grad, w.grad), (model.embed.weight.grad, emb.grad)):
+        got = got.float().cpu()
+        assert (got - exp).abs().max().item() <= _bf16_tol(exp)
+        assert ((got - exp).norm() / exp.norm()).item() <= 2e-2

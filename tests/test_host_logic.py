@@ -205,3 +205,85 @@ def test_side_tensors_that_do_not_broadcast_are_rejected_before_any_kernel():
         grpo_utils.grpo_loss_on_logits(logits, labels, None, None, torch.zeros(3, 2), mask, cfg)
     with pytest.raises(ValueError, match="advantages of shape"):
         grpo_utils.compute_rho_correction(torch.zeros(2, 3), torch.zeros(2, 3), mask, torch.zeros(5), cfg)
+
+
+def test_doc_lens_from_attention_mask_reference_vectors(golden):
+    """open_instruct/test_grpo_utils.py:9-48: run lengths per row, padding runs kept as segments, rows
+    padded with zeros to the widest row, row sums equal the sequence length."""
+    from open_instruct_amd import olmo_core_utils
+
+    for case in golden["doc_lens_from_attention_mask"]["cases"]:
+        mask = torch.tensor(case["attention_mask"], dtype=torch.long)
+        doc_lens, max_doc_lens = olmo_core_utils.doc_lens_from_attention_mask(mask)
+        assert doc_lens.dtype == torch.int32, case["name"]
+        assert doc_lens.tolist() == case["doc_lens"], case["name"]
+        assert max_doc_lens == case["max_doc_lens"], case["name"]
+        assert doc_lens.sum(dim=1).tolist() == [mask.shape[1]] * mask.shape[0]
+    # against a plain Python run-length encoding on random masks with non-monotonic ids
+    g = torch.Generator().manual_seed(0)
+    mask = torch.randint(0, 3, (5, 40), generator=g).sort(dim=1).values.roll(7, dims=1)
+    doc_lens, max_doc_lens = olmo_core_utils.doc_lens_from_attention_mask(mask)
+    for row, got, longest in zip(mask.tolist(), doc_lens.tolist(), max_doc_lens):
+        runs, prev = [], object()
+        for v in row:
+            if v == prev:
+                runs[-1] += 1
+            else:
+                runs.append(1)
+                prev = v
+        assert got[: len(runs)] == runs and not any(got[len(runs) :]) and longest == max(runs)
+
+
+def test_doc_lens_from_cu_seq_lens():
+    """open_instruct/olmo_core_utils.py:650-665: differences of the offsets; a padded tail becomes a
+    segment of its own so the lengths cover the whole row (the reference holds no vector for it;
+    expected values follow from the definition)."""
+    from open_instruct_amd import olmo_core_utils
+
+    cu = torch.tensor([0, 50, 100, 550, 600], dtype=torch.int32)  # open_instruct/test_padding_free_collator.py:348-363
+    doc_lens, longest = olmo_core_utils.doc_lens_from_cu_seq_lens(cu, seq_len=600)
+    assert doc_lens.dtype == torch.int32 and doc_lens.tolist() == [[50, 50, 450, 50]] and longest == [450]
+    doc_lens, longest = olmo_core_utils.doc_lens_from_cu_seq_lens(cu, seq_len=1000)
+    assert doc_lens.tolist() == [[50, 50, 450, 50, 400]] and longest == [450]
+    doc_lens, longest = olmo_core_utils.doc_lens_from_cu_seq_lens(torch.tensor([0, 3]), seq_len=10)
+    assert doc_lens.tolist() == [[3, 7]] and longest == [7]
+
+
+def test_olmo_forward_plumbing_passes_labels_and_doc_lens():
+    """concatenated_forward_olmo (open_instruct/dpo_utils.py:959-1019) hands the labels to the model and,
+    for packed batches, position ids and document lengths; forward_for_logprobs with
+    pass_olmo_core_doc_lens (open_instruct/grpo_utils.py:551-557) replaces the attention mask by them.
+    Checked with a recording stand-in model up to the first kernel call (which needs a GPU)."""
+    calls = []
+
+    class Recorder(torch.nn.Module):
+        def forward(self, *args, **kwargs):
+            calls.append((args, kwargs))
+            raise RuntimeError("recorded")
+
+    chosen = {"input_ids": torch.ones(1, 5, dtype=torch.long), "labels": torch.ones(1, 5, dtype=torch.long),
+              "cu_seq_lens_q": torch.tensor([0, 2, 5]), "cu_seq_lens_k": torch.tensor([0, 2, 5]),
+              "max_length_q": 3, "max_length_k": 3, "position_ids": torch.tensor([[0, 1, 0, 1, 2]])}  # fmt: skip
+    rejected = {"input_ids": torch.ones(1, 4, dtype=torch.long), "labels": torch.ones(1, 4, dtype=torch.long),
+                "cu_seq_lens_q": torch.tensor([0, 1, 4]), "cu_seq_lens_k": torch.tensor([0, 1, 4]),
+                "max_length_q": 3, "max_length_k": 3, "position_ids": torch.tensor([[0, 0, 1, 2]])}  # fmt: skip
+    batch = {f"chosen_{k}": v for k, v in chosen.items()} | {f"rejected_{k}": v for k, v in rejected.items()}
+    with pytest.raises(RuntimeError, match="recorded"):
+        dpo_utils.concatenated_forward_olmo(Recorder(), batch, packing=True)
+    args, kwargs = calls.pop()
+    assert args[0].shape == (1, 9) and kwargs["labels"].shape == (1, 9)
+    assert kwargs["doc_lens"].tolist() == [[2, 3, 1, 3]] and kwargs["max_doc_lens"] == [3]
+    assert kwargs["position_ids"].tolist() == [[0, 1, 0, 1, 2, 0, 0, 1, 2]]
+    padded = {"chosen_input_ids": torch.ones(2, 5, dtype=torch.long), "chosen_labels": torch.ones(2, 5, dtype=torch.long),
+              "rejected_input_ids": torch.ones(2, 3, dtype=torch.long), "rejected_labels": torch.ones(2, 3, dtype=torch.long)}  # fmt: skip
+    with pytest.raises(RuntimeError, match="recorded"):
+        dpo_utils.concatenated_forward_olmo(Recorder(), padded, packing=False)
+    args, kwargs = calls.pop()
+    assert args[0].shape == (4, 5) and set(kwargs) == {"labels"} and (kwargs["labels"][2:, 3:] == -100).all()
+    mask = torch.tensor([[1, 1, 2, 2, 2, 0]])
+    with pytest.raises(RuntimeError, match="recorded"):
+        grpo_utils.forward_for_logprobs(Recorder(), torch.ones(1, 6, dtype=torch.long), mask, mask, 0, 1.0, pass_olmo_core_doc_lens=True)
+    _, kwargs = calls.pop()
+    assert kwargs["attention_mask"] is None and kwargs["doc_lens"].tolist() == [[2, 3, 1]] and kwargs["max_doc_lens"] == [3]
+    with pytest.raises(AssertionError):
+        grpo_utils.forward_for_logprobs(Recorder(), torch.ones(1, 6, dtype=torch.long), None, mask, 0, 1.0, pass_olmo_core_doc_lens=True)
