@@ -79,7 +79,7 @@ class EventTimer:
 # ------------------------------------------------------------------------------------------------
 # workloads
 # ------------------------------------------------------------------------------------------------
-def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False):
+def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=False):
     dev = "cuda:0"
     torch.manual_seed(0)
     hidden = torch.randn(n_tokens, hdim, device=dev).bfloat16().requires_grad_(True)
@@ -113,7 +113,12 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False):
     def step():
         hidden.grad = None
         weight.grad = None
-        if not dpo:
+        if one_call:
+            with fwd_timer:  # the whole step is one C call here: the timer brackets all of it
+                loss, _, _, _ = oi.grpo_utils.grpo_loss_on_hidden(
+                    hidden[None], weight, labels[None], old[None], ref[None], adv[None], mask[None], cfg
+                )
+        elif not dpo:
             with fwd_timer:
                 lp, ent = oi.fused_lm_head_logprobs(hidden, weight, labels, mask=mask, return_entropy=True)
             loss, _ = oi.grpo_utils.grpo_loss_fused(
@@ -139,6 +144,9 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False):
         "bound": "mfma",
         "timer": fwd_timer,
     }
+    if one_call:
+        info["kernel"] = "oi_lmhead_grpo_fwd_bwd (every launch of the step: forward, loss, dZ, dHidden, dW)"
+        info["alg_per_launch"] = 3.0 * flops_fwd
     return step, info
 
 
@@ -449,7 +457,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c2-two-pass", "c3", "c4", "c5", "pack"])
+    ap.add_argument("--workload", default="c3",
+                    choices=["c1", "c2", "c2-two-pass", "c3", "c3-one-call", "c4", "c5", "pack"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-library-gemm", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -471,6 +480,10 @@ def main():
     if args.workload == "c3":
         step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02)
         name = "c3: fused lm_head+logprob+entropy+GRPO loss fwd+bwd, hidden bf16 [32768,4096], W bf16 [128256,4096], 70% response tokens (rows compacted)"
+        dtype = "bf16"
+    elif args.workload == "c3-one-call":
+        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02, one_call=True)
+        name = "c3: the same step through the single entry point grpo_loss_on_hidden (oi_lmhead_grpo_fwd_bwd)"
         dtype = "bf16"
     elif args.workload == "c4":
         step, info = make_c4(torch, oi)

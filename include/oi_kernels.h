@@ -205,7 +205,7 @@ int oi_grpo_stats_from_terms(const float* pg_loss, const float* clipfrac, const 
                              int64_t rows, int64_t cols, int kl_estimator, float beta, float* out_stats,
                              int64_t out_stride, uint32_t write_mask, void* workspace, size_t workspace_bytes,
                              void* stream);
-/* d loss / d new_logprobs (fp32 [rows, cols]); grad_loss is a DEVICE scalar (upstream gradient). */
+/* d loss / d new_logprobs (fp32 [rows, cols]); grad_loss is a DEVICE scalar (upstream gradient; NULL = 1). */
 int oi_grpo_fused_bwd(const float* new_logprobs, const float* old_logprobs, const float* ref_logprobs,
                       const float* advantages, const uint8_t* mask, const float* rho_weights, int64_t rows,
                       int64_t cols, int loss_fn, float ratio_lo, float ratio_hi, int kl_estimator, float beta,
@@ -371,6 +371,32 @@ int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* la
                        const float* grad_logprob, const uint8_t* row_mask, int skip_zero_grad_rows, int64_t n_tokens,
                        int64_t hidden_dim, int64_t vocab, float inv_temperature, void* d_hidden, void* d_weight,
                        void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The whole GRPO step on hidden states in one call: fused lm_head forward (logprob, entropy),
+ * scalar loss with its statistics, and the backward to d_hidden / d_weight, for an upstream
+ * gradient of 1 on the loss.  It replaces, for a model that hands out its final hidden states, the
+ * sequence open_instruct/grpo_utils.py:558-572 (lm_head, log_softmax_and_gather, entropy) ->
+ * open_instruct/grpo_utils.py:504-538 (compute_grpo_loss) -> open_instruct/grpo_fast.py:702-724
+ * (masked_mean, loss.backward()); no single reference function computes it.
+ *
+ * hidden: bf16 [rows * cols, hidden_dim]; labels int64, mask (one byte per token) and the fp32 side
+ * tensors are [rows, cols]; `mask` is the response mask: it selects the rows that are multiplied
+ * and the tokens that enter the loss.  old_logprobs NULL: ratio 1 with gradient; ref_logprobs NULL:
+ * no KL term; rho_weights NULL: 1.  Loss arguments and out_stats as for oi_grpo_fused_fwd (the rho
+ * indicator statistics [10..12, 14] are 0 here).  logprob / entropy (may be NULL) are fp32
+ * [rows, cols], 0 off the mask.  d_weight NULL skips that product.  A token's upstream gradient
+ * depends only on its own logprob once the denominators are known, and those come from the mask, so
+ * the backward is enqueued straight behind the forward: nothing returns to the host in between.
+ */
+size_t oi_lmhead_grpo_workspace_bytes(int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab);
+int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, const int64_t* labels, const uint8_t* mask,
+                           const float* old_logprobs, const float* ref_logprobs, const float* advantages,
+                           const float* rho_weights, int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab,
+                           float inv_temperature, int loss_fn, float ratio_lo, float ratio_hi, int kl_estimator,
+                           float beta, int axis_mode, float denominator, float scale, float* logprob, float* entropy,
+                           float* out_stats, void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes,
+                           void* stream);
 
 /*
  * The bf16 MFMA main loop of the lm_head kernels as a plain product (no reference counterpart;

@@ -1034,6 +1034,102 @@ RowInputs launch_selection(const SelectionPlan& sp, char* ws, const void* hidden
     return RowInputs{hidden_c, labels_c, lse_c, grad_c, rows, count};
 }
 
+// lse and upstream gradient of the selected rows (the rows were selected and gathered earlier)
+__global__ void gather_f32_pair_kernel(const float* __restrict__ lse, const float* __restrict__ grad,
+                                       const int32_t* __restrict__ rows, const int32_t* __restrict__ count,
+                                       float* __restrict__ lse_c, float* __restrict__ grad_c) {
+    const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= *count) return;
+    const int64_t src = rows[j];
+    lse_c[j] = lse[src];
+    grad_c[j] = grad[src];
+}
+
+// forward launches: tile kernel + merge of the partial statistics.  `queue` must be zeroed.
+void enqueue_fwd(const FwdPlan& p, char* ws, const RowInputs& in, const uint8_t* row_mask, const void* weight,
+                 int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob,
+                 float* entropy, float* lse, hipStream_t s) {
+    float4* partial = reinterpret_cast<float4*>(ws + p.off_partial);
+    float* zy = reinterpret_cast<float*>(ws + p.off_zy);
+    uint32_t* queue = reinterpret_cast<uint32_t*>(ws + p.off_queue);
+    const float c = inv_temperature * OI_LOG2E;
+    hipLaunchKernelGGL(lmhead_fwd_kernel, dim3(resident_grid(p.n_splits, p.token_tiles)), dim3(NTHREADS), 0, s,
+                       static_cast<const uint16_t*>(weight), in.hidden, in.labels, n_tokens, in.n_dev, hidden_dim, vocab,
+                       c, p.n_splits, p.tiles_per_split, p.n_pad, partial, zy, queue);
+    hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
+                       zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, logprob,
+                       entropy, lse);
+}
+
+// backward launches.  Per vocabulary chunk: dZ [n_pad, cols] (token-major, bf16, zero in padded rows
+// and columns), then both products straight from W and the (selected) hidden rows, which enter as
+// k-major operands:
+//   d_hidden[n, h] (+)= sum_v dZ[n, v] * W[v_begin + v, h]      A k-contiguous, B k-major
+//   d_weight[v_begin + v, h] = sum_n dZ[n, v] * hidden[n, h]    A k-major,      B k-major
+// The sums stop at the last real vocabulary row / token (rounded up to a k-tile, whose missing
+// rows are read from the last real one and meet zeros of dZ).  The queue words must be zeroed.
+void enqueue_bwd(const BwdPlan& p, char* ws, const RowInputs& in, const void* weight, int64_t n_tokens,
+                 int64_t hidden_dim, int64_t vocab, float inv_temperature, void* d_hidden, void* d_weight,
+                 hipStream_t s) {
+    uint16_t* dz = reinterpret_cast<uint16_t*>(ws + p.off_dz);
+    float* dh32 = reinterpret_cast<float*>(ws + p.off_dh32);
+    uint32_t* queues = reinterpret_cast<uint32_t*>(ws + p.off_queues);
+    const uint16_t* Wp = static_cast<const uint16_t*>(weight);
+    const float c = inv_temperature * OI_LOG2E;
+    const int64_t h_tiles = (hidden_dim + BN - 1) / BN;
+    for (int64_t ci = 0; ci < p.n_chunks; ++ci) {
+        const int64_t v_begin = ci * p.chunk;
+        const int64_t cols = (p.v_pad - v_begin) < p.chunk ? (p.v_pad - v_begin) : p.chunk;  // multiple of 256
+        const int64_t valid = vocab - v_begin < cols ? vocab - v_begin : cols;               // real rows of W
+        uint32_t* q = queues + ci * 3 * QUEUE_WORDS;
+        hipLaunchKernelGGL(lmhead_dz_kernel, dim3(resident_grid(cols / BM, p.n_pad / BN)), dim3(NTHREADS), 0, s, Wp,
+                           in.hidden, in.labels, in.lse, in.grad, n_tokens, in.n_dev, hidden_dim, vocab, c,
+                           inv_temperature, v_begin, cols, p.n_pad, dz, q);
+        const bool first = ci == 0, last = ci == p.n_chunks - 1;
+        const int mode = last ? (first ? 2 : 3) : (first ? 0 : 1);
+        {
+            const Operand a = {dz, cols, 0, p.n_pad, cols};
+            const Operand b = {Wp + v_begin * hidden_dim, hidden_dim, 0, hidden_dim, valid};
+            const DynRows dyn = {in.n_dev, 1, in.rows};
+            hipLaunchKernelGGL((gemm_store_kernel<false, true>), dim3(resident_grid(p.n_pad / BM, h_tiles)),
+                               dim3(NTHREADS), 0, s, a, p.n_pad, b, hidden_dim, round_up(valid, BK), mode, dh32,
+                               static_cast<uint16_t*>(d_hidden), hidden_dim, n_tokens, dyn, q + QUEUE_WORDS);
+        }
+        if (d_weight) {
+            const Operand a = {dz, cols, 0, cols, p.n_pad};
+            const Operand b = {in.hidden, hidden_dim, 0, hidden_dim, n_tokens};
+            const DynRows dyn = {in.n_dev, 2, nullptr};
+            hipLaunchKernelGGL((gemm_store_kernel<true, true>), dim3(resident_grid(cols / BM, h_tiles)),
+                               dim3(NTHREADS), 0, s, a, cols, b, hidden_dim, round_up(n_tokens, BK), 2,
+                               static_cast<float*>(nullptr), static_cast<uint16_t*>(d_weight) + v_begin * hidden_dim,
+                               hidden_dim, valid, dyn, q + 2 * QUEUE_WORDS);
+        }
+    }
+}
+
+// workspace of the whole-step entry point: forward and backward regions side by side (they share
+// one row selection), the statistics partials, and the per-token vectors that connect the stages
+struct StepPlan {
+    FwdPlan fwd;
+    BwdPlan bwd;
+    size_t off_fwd, off_bwd, off_stats, off_lse, off_grad, off_denoms, total;
+};
+StepPlan plan_step(int64_t rows, int64_t cols, int64_t hdim, int64_t vocab) {
+    StepPlan p;
+    const int64_t n = rows * cols;
+    p.fwd = plan_fwd(n, hdim, vocab, false);
+    p.bwd = plan_bwd(n, hdim, vocab, true);
+    Carver cv;
+    p.off_fwd = cv.take(p.fwd.total);
+    p.off_bwd = cv.take(p.bwd.total);
+    p.off_stats = cv.take(oi_grpo_fused_workspace_bytes(rows, cols));
+    p.off_lse = cv.take((size_t)n * sizeof(float));
+    p.off_grad = cv.take((size_t)n * sizeof(float));
+    p.off_denoms = cv.take((size_t)rows * sizeof(float));
+    p.total = cv.off;
+    return p;
+}
+
 }  // namespace
 
 extern "C" size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
@@ -1054,23 +1150,15 @@ extern "C" int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const 
     const FwdPlan p = plan_fwd(n_tokens, hidden_dim, vocab, row_mask != nullptr);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     char* ws = static_cast<char*>(workspace);
-    float4* partial = reinterpret_cast<float4*>(ws + p.off_partial);
-    float* zy = reinterpret_cast<float*>(ws + p.off_zy);
     uint32_t* queue = reinterpret_cast<uint32_t*>(ws + p.off_queue);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const float c = inv_temperature * OI_LOG2E;
     RowInputs in = {static_cast<const uint16_t*>(hidden), labels, nullptr, nullptr, nullptr, nullptr};
     if (row_mask)
         in = launch_selection(p.sel, ws, hidden, labels, nullptr, nullptr, row_mask, false, n_tokens, hidden_dim, queue,
                               QUEUE_WORDS, s);
     else
         hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, queue, QUEUE_WORDS);
-    hipLaunchKernelGGL(lmhead_fwd_kernel, dim3(resident_grid(p.n_splits, p.token_tiles)), dim3(NTHREADS), 0, s,
-                       static_cast<const uint16_t*>(weight), in.hidden, in.labels, n_tokens, in.n_dev, hidden_dim, vocab,
-                       c, p.n_splits, p.tiles_per_split, p.n_pad, partial, zy, queue);
-    hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
-                       zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, logprob,
-                       entropy, lse);
+    enqueue_fwd(p, ws, in, row_mask, weight, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy, lse, s);
     return oi_launch_status();
 }
 
@@ -1092,70 +1180,89 @@ extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const 
     OI_RETURN_IF(!lse || !grad_logprob || !d_hidden || !workspace, OI_ENULL);
     // bf16 results are stored as pairs (4-byte words)
     OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 4) || !oi_aligned(d_weight, 4), OI_EALIGN);
-    const int want_dw = d_weight != nullptr;
     const bool selecting = row_mask != nullptr || skip_zero_grad_rows != 0;
     const BwdPlan p = plan_bwd(n_tokens, hidden_dim, vocab, selecting);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     hipStream_t s = static_cast<hipStream_t>(stream);
     char* ws = static_cast<char*>(workspace);
-    uint16_t* dz = reinterpret_cast<uint16_t*>(ws + p.off_dz);
-    float* dh32 = reinterpret_cast<float*>(ws + p.off_dh32);
-    const uint16_t* Wp = static_cast<const uint16_t*>(weight);
-    const float c = inv_temperature * OI_LOG2E;
-
     uint32_t* queues = reinterpret_cast<uint32_t*>(ws + p.off_queues);
     const int n_queue_words = (int)(3 * p.n_chunks * QUEUE_WORDS);
+    const float* zero_grad_probe = skip_zero_grad_rows ? grad_logprob : nullptr;
     RowInputs in = {static_cast<const uint16_t*>(hidden), labels, lse, grad_logprob, nullptr, nullptr};
-    if (selecting && n_queue_words <= SELECT_THREADS) {
-        in = launch_selection(p.sel, ws, hidden, labels, lse, grad_logprob, row_mask, skip_zero_grad_rows != 0, n_tokens,
-                              hidden_dim, queues, n_queue_words, s);
-    } else {
+    const bool select_clears_queues = selecting && n_queue_words <= SELECT_THREADS;
+    if (!select_clears_queues)
         hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_queue_words + 255) / 256)), dim3(256), 0, s, queues,
                            n_queue_words);
-        if (selecting)
-            in = launch_selection(p.sel, ws, hidden, labels, lse, grad_logprob, row_mask, skip_zero_grad_rows != 0,
-                                  n_tokens, hidden_dim, queues, 0, s);
-    }
-    if (selecting)
+    if (selecting) {
+        in = launch_selection(p.sel, ws, hidden, labels, lse, grad_logprob, row_mask, skip_zero_grad_rows != 0, n_tokens,
+                              hidden_dim, queues, select_clears_queues ? n_queue_words : 0, s);
         hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, row_mask,
-                           skip_zero_grad_rows ? grad_logprob : static_cast<const float*>(nullptr), hidden_dim,
-                           static_cast<uint16_t*>(d_hidden));
-
-    // Per vocabulary chunk: dZ [n_pad, cols] (token-major, bf16, zero in padded rows and columns),
-    // then both products straight from W and the (selected) hidden rows, which enter as k-major operands:
-    //   d_hidden[n, h] (+)= sum_v dZ[n, v] * W[v_begin + v, h]      A k-contiguous, B k-major
-    //   d_weight[v_begin + v, h] = sum_n dZ[n, v] * hidden[n, h]    A k-major,      B k-major
-    // The sums stop at the last real vocabulary row / token (rounded up to a k-tile, whose missing
-    // rows are read from the last real one and meet zeros of dZ).
-    const int64_t h_tiles = (hidden_dim + BN - 1) / BN;
-    for (int64_t ci = 0; ci < p.n_chunks; ++ci) {
-        const int64_t v_begin = ci * p.chunk;
-        const int64_t cols = (p.v_pad - v_begin) < p.chunk ? (p.v_pad - v_begin) : p.chunk;  // multiple of 256
-        const int64_t valid = vocab - v_begin < cols ? vocab - v_begin : cols;               // real rows of W
-        uint32_t* q = queues + ci * 3 * QUEUE_WORDS;
-        hipLaunchKernelGGL(lmhead_dz_kernel, dim3(resident_grid(cols / BM, p.n_pad / BN)), dim3(NTHREADS), 0, s, Wp,
-                           in.hidden, in.labels, in.lse, in.grad, n_tokens, in.n_dev, hidden_dim, vocab, c,
-                           inv_temperature, v_begin, cols, p.n_pad, dz, q);
-        const bool first = ci == 0, last = ci == p.n_chunks - 1;
-        const int mode = last ? (first ? 2 : 3) : (first ? 0 : 1);
-        {
-            const Operand a = {dz, cols, 0, p.n_pad, cols};
-            const Operand b = {Wp + v_begin * hidden_dim, hidden_dim, 0, hidden_dim, valid};
-            const DynRows dyn = {in.n_dev, 1, in.rows};
-            hipLaunchKernelGGL((gemm_store_kernel<false, true>), dim3(resident_grid(p.n_pad / BM, h_tiles)),
-                               dim3(NTHREADS), 0, s, a, p.n_pad, b, hidden_dim, round_up(valid, BK), mode, dh32,
-                               static_cast<uint16_t*>(d_hidden), hidden_dim, n_tokens, dyn, q + QUEUE_WORDS);
-        }
-        if (want_dw) {
-            const Operand a = {dz, cols, 0, cols, p.n_pad};
-            const Operand b = {in.hidden, hidden_dim, 0, hidden_dim, n_tokens};
-            const DynRows dyn = {in.n_dev, 2, nullptr};
-            hipLaunchKernelGGL((gemm_store_kernel<true, true>), dim3(resident_grid(cols / BM, h_tiles)),
-                               dim3(NTHREADS), 0, s, a, cols, b, hidden_dim, round_up(n_tokens, BK), 2,
-                               static_cast<float*>(nullptr), static_cast<uint16_t*>(d_weight) + v_begin * hidden_dim,
-                               hidden_dim, valid, dyn, q + 2 * QUEUE_WORDS);
-        }
+                           zero_grad_probe, hidden_dim, static_cast<uint16_t*>(d_hidden));
     }
+    enqueue_bwd(p, ws, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, d_weight, s);
+    return oi_launch_status();
+}
+
+extern "C" size_t oi_lmhead_grpo_workspace_bytes(int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab) {
+    if (rows <= 0 || cols <= 0 || hidden_dim <= 0 || vocab <= 0) return 0;
+    return plan_step(rows, cols, hidden_dim, vocab).total;
+}
+
+extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, const int64_t* labels,
+                                      const uint8_t* mask, const float* old_logprobs, const float* ref_logprobs,
+                                      const float* advantages, const float* rho_weights, int64_t rows, int64_t cols,
+                                      int64_t hidden_dim, int64_t vocab, float inv_temperature, int loss_fn,
+                                      float ratio_lo, float ratio_hi, int kl_estimator, float beta, int axis_mode,
+                                      float denominator, float scale, float* logprob, float* entropy, float* out_stats,
+                                      void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes,
+                                      void* stream) {
+    OI_RETURN_IF(rows <= 0 || cols <= 0 || rows > MAX_LD || cols > MAX_LD, OI_EINVAL);
+    const int64_t n_tokens = rows * cols;
+    int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
+    if (rc != OI_OK) return rc;
+    OI_RETURN_IF(!mask || !advantages || !logprob || !out_stats || !d_hidden || !workspace, OI_ENULL);
+    OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 4) || !oi_aligned(d_weight, 4), OI_EALIGN);
+    const StepPlan p = plan_step(rows, cols, hidden_dim, vocab);
+    OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    char* ws = static_cast<char*>(workspace);
+    char* ws_fwd = ws + p.off_fwd;
+    char* ws_bwd = ws + p.off_bwd;
+    float* lse = reinterpret_cast<float*>(ws + p.off_lse);
+    float* grad = reinterpret_cast<float*>(ws + p.off_grad);
+    float* row_denoms = reinterpret_cast<float*>(ws + p.off_denoms);
+
+    // one selection for both passes: it lives in the backward region; the select kernel also clears
+    // the backward queues, the forward queue gets the small fill kernel
+    uint32_t* fwd_queue = reinterpret_cast<uint32_t*>(ws_fwd + p.fwd.off_queue);
+    uint32_t* bwd_queues = reinterpret_cast<uint32_t*>(ws_bwd + p.bwd.off_queues);
+    const int n_queue_words = (int)(3 * p.bwd.n_chunks * QUEUE_WORDS);
+    const bool select_clears_queues = n_queue_words <= SELECT_THREADS;
+    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, fwd_queue, QUEUE_WORDS);
+    if (!select_clears_queues)
+        hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_queue_words + 255) / 256)), dim3(256), 0, s,
+                           bwd_queues, n_queue_words);
+    RowInputs in = launch_selection(p.bwd.sel, ws_bwd, hidden, labels, nullptr, nullptr, mask, false, n_tokens,
+                                    hidden_dim, bwd_queues, select_clears_queues ? n_queue_words : 0, s);
+    enqueue_fwd(p.fwd, ws_fwd, in, mask, weight, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy, lse, s);
+
+    // loss and statistics from the logprobs, then every token's d loss / d logprob (upstream gradient 1)
+    rc = oi_grpo_fused_fwd(logprob, old_logprobs, ref_logprobs, advantages, mask, rho_weights, entropy, nullptr, nullptr,
+                           nullptr, nullptr, rows, cols, loss_fn, ratio_lo, ratio_hi, kl_estimator, beta, axis_mode,
+                           denominator, scale, out_stats, row_denoms, ws + p.off_stats,
+                           oi_grpo_fused_workspace_bytes(rows, cols), stream);
+    if (rc != OI_OK) return rc;
+    rc = oi_grpo_fused_bwd(logprob, old_logprobs, ref_logprobs, advantages, mask, rho_weights, rows, cols, loss_fn,
+                           ratio_lo, ratio_hi, kl_estimator, beta, scale, row_denoms, nullptr, grad, stream);
+    if (rc != OI_OK) return rc;
+
+    in.lse = reinterpret_cast<float*>(ws_bwd + p.bwd.sel.off_lse);
+    in.grad = reinterpret_cast<float*>(ws_bwd + p.bwd.sel.off_grad);
+    hipLaunchKernelGGL(gather_f32_pair_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, lse, grad,
+                       in.rows, in.n_dev, const_cast<float*>(in.lse), const_cast<float*>(in.grad));
+    hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, mask,
+                       static_cast<const float*>(nullptr), hidden_dim, static_cast<uint16_t*>(d_hidden));
+    enqueue_bwd(p.bwd, ws_bwd, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, d_weight, s);
     return oi_launch_status();
 }
 

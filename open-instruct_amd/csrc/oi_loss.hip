@@ -199,7 +199,7 @@ __global__ void grpo_fused_bwd_kernel(const float* __restrict__ nlp, const float
     const float ratio = old ? expf(x - old[i]) : 1.f;
     const float w = rho ? rho[i] : 1.f;
     const float per_token = grpo_token_dnew(x, ratio, adv[i], ref != nullptr, ref ? ref[i] : 0.f, w, c, beta);
-    d_new[i] = grad_loss[0] * scale * row_denoms[r] * per_token;
+    d_new[i] = (grad_loss ? grad_loss[0] : 1.f) * scale * row_denoms[r] * per_token;
 }
 
 // ---- group-normalised advantages ----------------------------------------------------------------
@@ -719,7 +719,7 @@ extern "C" int oi_grpo_fused_bwd(const float* new_logprobs, const float* old_log
     OI_RETURN_IF(rows <= 0 || cols <= 0, OI_EINVAL);
     const int rc = check_cfg(loss_fn, kl_estimator);
     if (rc != OI_OK) return rc;
-    OI_RETURN_IF(!new_logprobs || !advantages || !mask || !row_denoms || !grad_loss || !d_new_logprobs, OI_ENULL);
+    OI_RETURN_IF(!new_logprobs || !advantages || !mask || !row_denoms || !d_new_logprobs, OI_ENULL);
     const GrpoCfg c = {loss_fn, ratio_lo, ratio_hi, kl_estimator};
     hipLaunchKernelGGL(grpo_fused_bwd_kernel, dim3(blocks_for(rows * cols, 256)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), new_logprobs, old_logprobs, ref_logprobs, advantages, mask,

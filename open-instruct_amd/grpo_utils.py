@@ -518,6 +518,117 @@ def grpo_loss_on_logits(
     return _AttachLogitsGrad.apply(loss, logits, dlogits), stats, logprob, entropy
 
 
+class _AttachHeadGrads(torch.autograd.Function):
+    """Identity on the loss value whose backward hands out the gradients computed in the forward."""
+
+    @staticmethod
+    def forward(ctx, loss, hidden, weight, d_hidden, d_weight):
+        ctx.save_for_backward(d_hidden, d_weight)
+        ctx.handed_out = False
+        return loss.clone()
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        d_hidden, d_weight = ctx.saved_tensors
+        if ctx.handed_out:  # a second backward over a retained graph must not scale the same memory twice
+            d_hidden = d_hidden.clone()
+            d_weight = None if d_weight is None else d_weight.clone()
+        ctx.handed_out = True
+        g = _lib.f32c(grad_loss.detach()).reshape(1)
+        for t in (d_hidden, d_weight):  # nothing is touched when the device scalar is exactly 1
+            if t is not None:
+                _lib.call(
+                    "oi_scale_by_device_scalar", t.data_ptr(), _lib.DTYPE_TAGS[t.dtype], t.numel(), g.data_ptr(),
+                    _lib.stream_of(t),
+                )  # fmt: skip
+        need_h, need_w = ctx.needs_input_grad[1], ctx.needs_input_grad[2]
+        return None, (d_hidden if need_h else None), (d_weight if need_w else None), None, None
+
+
+def grpo_loss_on_hidden(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    old_logprobs: torch.Tensor | None,
+    ref_logprobs: torch.Tensor | None,
+    advantages: torch.Tensor,
+    response_mask: torch.Tensor,
+    config,
+    temperature: float = 1.0,
+    rho_weights: torch.Tensor | None = None,
+    loss_denominator: float | None = None,
+    axis: int | None = None,
+    dp_scale: float = 1.0,
+) -> tuple[torch.Tensor, dict[str, torch.Tensor], torch.Tensor, torch.Tensor]:
+    """GRPO loss straight from final hidden states; returns ``(loss, stats, logprobs, entropy)``.
+
+    One call for ``fused_lm_head_logprobs`` → ``grpo_loss_fused`` → backward
+    (open_instruct/grpo_utils.py:558-572 → :504-538 → open_instruct/grpo_fast.py:702-724): the
+    ``[tokens, vocab]`` logits are never formed, rows off ``response_mask`` are not multiplied, and
+    the gradients with respect to ``hidden`` and ``weight`` are computed inside the same call and
+    handed out by ``loss.backward()`` (a token's upstream gradient depends only on its own logprob
+    once the denominators are known, and those come from the mask).  ``hidden`` is ``[B, T, H]``
+    bf16, ``weight`` ``[V, H]`` bf16, ``labels`` and the side tensors ``[B, T]`` (anything that
+    broadcasts).  ``logprobs`` and ``entropy`` are returned detached, 0 off the mask.  Without a
+    gradient to compute (``torch.no_grad()``, inputs without ``requires_grad``) only the forward runs.
+    """
+    if axis not in (None, 1, -1):
+        raise ValueError("axis must be None or the token axis (1)")
+    if loss_denominator is not None and float(loss_denominator) <= 0.0:
+        raise ValueError("loss_denominator must be positive when given")
+    if labels.ndim != 2 or tuple(response_mask.shape) != tuple(labels.shape):
+        raise ValueError("labels and response_mask must be [B, T]")
+    if tuple(hidden.shape[:-1]) != tuple(labels.shape):
+        raise ValueError(f"labels {tuple(labels.shape)} do not match hidden rows {tuple(hidden.shape[:-1])}")
+    inv_t = model_utils._inv_temperature(temperature)
+    wants_grad = torch.is_grad_enabled() and (hidden.requires_grad or weight.requires_grad)
+    if not wants_grad:
+        from . import lm_head
+
+        with torch.no_grad():
+            logprob, entropy = lm_head.fused_lm_head_logprobs(
+                hidden, weight, labels, temperature=temperature, mask=response_mask, return_entropy=True
+            )
+            loss, stats = grpo_loss_fused(
+                logprob, old_logprobs, ref_logprobs, advantages, response_mask, config, rho_weights=rho_weights,
+                entropy=entropy, loss_denominator=loss_denominator, axis=axis, dp_scale=dp_scale,
+            )  # fmt: skip
+        return loss, stats, logprob, entropy
+    dev = _lib.require_gpu(hidden, weight, labels, response_mask, advantages)
+    if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise ValueError("the fused lm_head expects bf16 hidden states and weight")
+    rows, cols = labels.shape
+    h, v = hidden.shape[-1], weight.shape[0]
+    if weight.ndim != 2 or weight.shape[1] != h or h % 64:
+        raise ValueError(f"weight {tuple(weight.shape)} does not fit hidden size {h} (a multiple of 64)")
+    shape = (rows, cols)
+    f32 = lambda t, name: None if t is None else _lib.f32c(_expand_to(t.detach(), shape, name))  # noqa: E731
+    old_c, ref_c = f32(old_logprobs, "old_logprobs"), f32(ref_logprobs, "ref_logprobs")
+    adv_c, rho_c = f32(advantages, "advantages"), f32(rho_weights, "rho_weights")
+    m = _lib.mask_u8(response_mask)
+    hid = hidden.detach().reshape(rows * cols, h).contiguous()
+    w = weight.detach().contiguous()
+    lab = labels.to(torch.int64).contiguous()
+    lo, hi = _clip_bounds(config)
+    logprob = torch.empty(shape, dtype=torch.float32, device=dev)
+    entropy = torch.empty(shape, dtype=torch.float32, device=dev)
+    stats = torch.empty(len(GRPO_STAT_NAMES), dtype=torch.float32, device=dev)
+    d_hidden = torch.empty_like(hid)
+    d_weight = torch.empty_like(w) if weight.requires_grad else None
+    ws_bytes = _lib.load().oi_lmhead_grpo_workspace_bytes(rows, cols, h, v)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    _lib.call(
+        "oi_lmhead_grpo_fwd_bwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), m.data_ptr(), _lib.ptr(old_c),
+        _lib.ptr(ref_c), adv_c.data_ptr(), _lib.ptr(rho_c), rows, cols, h, v, inv_t, _loss_fn_tag(config), lo, hi,
+        int(config.kl_estimator), float(config.beta), 0 if axis is None else 1,
+        0.0 if loss_denominator is None else float(loss_denominator), float(dp_scale), logprob.data_ptr(),
+        entropy.data_ptr(), stats.data_ptr(), d_hidden.data_ptr(), _lib.ptr(d_weight), ws.data_ptr(), ws_bytes,
+        _lib.stream_of(hid),
+    )  # fmt: skip
+    loss = _AttachHeadGrads.apply(stats[0], hidden, weight, d_hidden.reshape(hidden.shape), d_weight)
+    return loss, _StatsView(stats), logprob, entropy
+
+
 def group_advantages(scores: torch.Tensor, group_size: int, normalization: str = "standard") -> torch.Tensor:
     """Group-normalised advantages; open_instruct/data_loader.py:1472-1484 on the device.
 

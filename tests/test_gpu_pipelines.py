@@ -359,3 +359,91 @@ def test_concatenated_forward_olmo_through_dpo_lm_head(packing, average_log_prob
         got = got.float().cpu()
         assert (got - exp).abs().max().item() <= _bf16_tol(exp)
         assert ((got - exp).norm() / exp.norm()).item() <= 2e-2
+
+
+@pytest.mark.parametrize("loss_fn,axis,denominator,with_old,want_dw", [
+    ("dapo", None, None, True, True),
+    ("dapo", 1, None, True, False),
+    ("cispo", None, 300.0, False, True),
+])  # fmt: skip
+def test_grpo_loss_on_hidden_whole_step(loss_fn, axis, denominator, with_old, want_dw):
+    """One C call for lm_head -> logprob / entropy -> GRPO loss -> backward
+    (open_instruct/grpo_utils.py:558-572 -> :504-538 -> open_instruct/grpo_fast.py:702-724) against
+    the oracle chain and against the three-call chain of this package."""
+    torch.manual_seed(33)
+    b, t, h, v = 3, 130, 128, 40000  # two vocabulary chunks, two token tiles
+    hidden = torch.randn(b, t, h).bfloat16()
+    weight = (torch.randn(v, h) * 3.0 / math.sqrt(h)).bfloat16()
+    labels = torch.randint(0, v, (b, t))
+    mask = torch.rand(b, t) < 0.7
+    mask[1, :] = False  # a row without response tokens
+    adv = torch.randn(b, 1)  # broadcast along the tokens
+    rho = torch.rand(b, t) + 0.5
+    cfg = make_grpo_config(loss_fn=loss_fn, beta=0.05, kl_estimator=2, clip_higher=0.28)
+    temperature = 0.9
+
+    rh = hidden.float().requires_grad_(True)
+    rw = weight.float().requires_grad_(True)
+    lp_o, ent_o = o_lm.lm_head_logprobs(rh.reshape(b * t, h), rw, labels.reshape(-1), temperature, True)
+    lp_o, ent_o = lp_o.reshape(b, t), ent_o.reshape(b, t)
+    old = lp_o.detach() + 0.05 * torch.randn(b, t)
+    ref = lp_o.detach() + 0.1 * torch.randn(b, t)
+    loss_o, *_ = o_grpo.grpo_token_loss(
+        lp_o, old if with_old else lp_o.detach(), ref, adv.expand(b, t), mask.float(), cfg, rho_weights=rho,
+        loss_denominator=denominator, axis=axis, dp_scale=2.0,
+    )  # fmt: skip
+    torch.nan_to_num(loss_o, nan=0.0).backward()
+    exp_dh, exp_dw = torch.nan_to_num(rh.grad, nan=0.0), torch.nan_to_num(rw.grad, nan=0.0)
+
+    d = lambda x: x.to(DEV)  # noqa: E731
+    dh = d(hidden).requires_grad_(True)
+    dw = d(weight).requires_grad_(want_dw)
+    loss, stats, lp, ent = grpo_utils.grpo_loss_on_hidden(
+        dh, dw, d(labels), d(old) if with_old else None, d(ref), d(adv), d(mask), cfg, temperature=temperature,
+        rho_weights=d(rho), loss_denominator=denominator, axis=axis, dp_scale=2.0,
+    )  # fmt: skip
+    loss.backward()
+    assert ((lp.cpu() - lp_o.detach()) * mask).abs().max().item() <= TOL and (lp.cpu()[~mask] == 0).all()
+    assert ((ent.cpu() - ent_o) * mask).abs().max().item() <= TOL
+    if axis is None:
+        assert abs(loss.item() - loss_o.item()) <= TOL
+    assert (dh.grad.float().cpu() - exp_dh).abs().max().item() <= _bf16_tol(exp_dh)
+    assert ((dh.grad.float().cpu() - exp_dh).norm() / exp_dh.norm()).item() <= 2e-2
+    assert (dh.grad.cpu()[~mask] == 0).all()
+    if want_dw:
+        assert (dw.grad.float().cpu() - exp_dw).abs().max().item() <= _bf16_tol(exp_dw)
+        assert ((dw.grad.float().cpu() - exp_dw).norm() / exp_dw.norm()).item() <= 2e-2
+    else:
+        assert dw.grad is None
+
+    # the three-call chain of this package gives the same numbers
+    dh2 = d(hidden).requires_grad_(True)
+    dw2 = d(weight).requires_grad_(want_dw)
+    lp2, ent2 = lm_head.fused_lm_head_logprobs(dh2, dw2, d(labels), temperature, mask=d(mask), return_entropy=True)
+    loss2, stats2 = grpo_utils.grpo_loss_fused(
+        lp2, d(old) if with_old else None, d(ref), d(adv), d(mask), cfg, rho_weights=d(rho), entropy=ent2,
+        loss_denominator=denominator, axis=axis, dp_scale=2.0,
+    )  # fmt: skip
+    loss2.backward()
+    assert torch.equal(lp, lp2.detach()) and torch.equal(ent, ent2)
+    assert loss.item() == loss2.item()
+    for k in stats2:
+        assert stats[k].item() == stats2[k].item(), k
+    assert torch.equal(dh.grad, dh2.grad)
+    if want_dw:
+        assert torch.equal(dw.grad, dw2.grad)
+    # an upstream gradient other than 1 is applied on the device
+    dh3 = d(hidden).requires_grad_(True)
+    loss3, *_ = grpo_utils.grpo_loss_on_hidden(
+        dh3, d(weight), d(labels), d(old) if with_old else None, d(ref), d(adv), d(mask), cfg, temperature=temperature,
+        rho_weights=d(rho), loss_denominator=denominator, axis=axis, dp_scale=2.0,
+    )  # fmt: skip
+    (loss3 * 0.5).backward()
+    assert (dh3.grad.float() - 0.5 * dh.grad.float()).abs().max().item() <= 2.0**-8 * dh.grad.float().abs().max().item()
+    # no gradient wanted: forward only, same loss
+    with torch.no_grad():
+        loss4, _, lp4, _ = grpo_utils.grpo_loss_on_hidden(
+            dh, dw, d(labels), d(old) if with_old else None, d(ref), d(adv), d(mask), cfg, temperature=temperature,
+            rho_weights=d(rho), loss_denominator=denominator, axis=axis, dp_scale=2.0,
+        )  # fmt: skip
+    assert not loss4.requires_grad and loss4.item() == loss.item() and torch.equal(lp4, lp)
