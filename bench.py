@@ -200,7 +200,7 @@ def make_c2(torch, oi, rows_b=64, t=1024, vocab=128256, single_pass=True):
             "tokens": n,
             "rows_multiplied": n,
             "bytes_step": 2.0 * n * vocab * 2,
-            "kernel": "lsg_grpo_fused_kernel (row held in registers: logprob, entropy, GRPO derivative and dlogits in one read + one write)",
+            "kernel": "lsg_grpo_fused_kernel (one 1024-thread workgroup per row: statistics pass, GRPO derivative, gradient pass; 144 KB of the row wait in the LDS, the rest is read again from the caches)",
             "alg_per_launch": 2.0 * n * vocab * 2,
             "bound": "hbm",
             "timer": fwd_timer,
@@ -356,6 +356,8 @@ def cpu_baseline(torch, workload):
     threads = torch.get_num_threads()
     cfg = _cfg()
     torch.manual_seed(0)
+    if workload == "c3-one-call":
+        workload = "c3"
     if workload in ("c3", "c4", "c5"):
         hdim = 8192 if workload == "c5" else 4096
         vocab, n = (100352 if workload == "c4" else 128256), 2048
@@ -417,6 +419,7 @@ def cpu_baseline(torch, workload):
             o_red.masked_mean(lp, mask) + o_red.masked_mean(ent, mask)
 
         sample = "the full config-1 batch (2048 rows, V=32000, fp32)"
+    scaled = {"c3": 32768, "c4": 32768, "c5": 32768, "c2": 65536, "c2-two-pass": 65536}.get(workload)
     run()  # warm-up
     times = []
     t_end = time.time() + 20.0
@@ -432,7 +435,23 @@ def cpu_baseline(torch, workload):
         "cores": threads,
         "kind": "port",
         "sample": sample + f"; median of {len(times)} runs, {med:.3f} s each, torch CPU threads={threads}",
+        # a row slice of the workload was timed and tokens/s taken from it (cost is linear in the rows)
+        "scaled": scaled is not None,
+        "row_fraction": (n / scaled) if scaled else 1.0,
+        "os_cpu_count": os.cpu_count(),
+        "cpu_model": _cpu_model(),
     }
+
+
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def library_gemm_tflops(torch, n, hdim, vocab):
