@@ -625,9 +625,10 @@ __device__ __forceinline__ void lmhead_dz_tile(const uint16_t* __restrict__ W, c
     gemm_tile(acc, W, hdim, m0, vocab, hidden, hdim, n0, n_tokens, hdim, lds);
 
     // stage[n][v]: rows = tokens of the tile, 256 (+8 pad) vocabulary columns.  A lane stores 8 bytes
-    // (4 vocabulary entries of one token); with rows of 132 words the 32 lanes of a half wave would
-    // land on 16 bank pairs, two lanes each.  Rows 16..31 of every 32 swap the two 8-byte halves of
-    // each 16-byte piece, which spreads the half wave over all 64 banks; the copy-out swaps them back.
+    // (4 vocabulary entries of one token) and consecutive lanes store to consecutive rows, 132 words
+    // apart: the stores of rows 8 apart meet on the same banks (measured: 1000 conflict cycles per
+    // tile).  Rows 8..15 of every 16 therefore swap the two 8-byte halves of each 16-byte piece
+    // (0 conflict cycles); the copy-out swaps them back.
     uint16_t* stage = lds;
     const int rows_left = (int)(vocab - m0 < BM ? vocab - m0 : BM);  // real vocabulary rows of the tile
     const int wave_row0 = wm * 64;
@@ -660,14 +661,14 @@ __device__ __forceinline__ void lmhead_dz_tile(const uint16_t* __restrict__ W, c
                     if (rows_left < BM && acc_row(wm, i, r, lane) >= rows_left) val = 0.f;  // last tile only
                     d[e] = val;
                 }
-                const int vl = acc_row(wm, i, q * 4, lane) ^ (((nl >> 4) & 1) << 2);
+                const int vl = acc_row(wm, i, q * 4, lane) ^ (((nl >> 3) & 1) << 2);
                 uint2 pk = make_uint2(oi_pack_bf16x2(d[0], d[1]), oi_pack_bf16x2(d[2], d[3]));
                 *reinterpret_cast<uint2*>(stage + nl * STAGE_STRIDE + vl) = pk;
             }
         if (mine) {
             // same lane, same LDS word as the store above: program order keeps them apart
             const float val = fmaf(ng, __builtin_amdgcn_exp2f(fmaf(z_label, c, -l2)), g);
-            stage[nl * STAGE_STRIDE + ((wave_row0 + rel) ^ (((nl >> 4) & 1) << 2))] = (uint16_t)oi_f32_to_bf16_bits(val);
+            stage[nl * STAGE_STRIDE + ((wave_row0 + rel) ^ (((nl >> 3) & 1) << 2))] = (uint16_t)oi_f32_to_bf16_bits(val);
         }
     }
     __syncthreads();
@@ -678,7 +679,7 @@ __device__ __forceinline__ void lmhead_dz_tile(const uint16_t* __restrict__ W, c
         const int cidx = tid + it * NTHREADS;
         const int row = cidx >> 5, ch = cidx & 31;
         oi_u32x4 v = *reinterpret_cast<const oi_u32x4*>(stage + row * STAGE_STRIDE + ch * 8);
-        if (row & 16) v = oi_u32x4{v.z, v.w, v.x, v.y};
+        if (row & 8) v = oi_u32x4{v.z, v.w, v.x, v.y};
         *reinterpret_cast<oi_u32x4*>(dz + (n0 + row) * chunk_cols + vcol0 + ch * 8) = v;
     }
 }
