@@ -41,9 +41,13 @@ PEAK_BF16_TFLOPS = 2500.0
 # be read from inside the process, so the figures are carried here from the committed summaries in
 # profiles/; workloads without a counter run report null.
 MEASURED_TRAFFIC_BYTES = {
-    "c3": 42.90e9 + 0.19e9,  # lmhead_fwd_kernel: L2 misses of the tiled operand re-reads (1.24 GB unique)
-    "c2": 18.72e9 + 16.82e9,  # lsg_grpo_fused_kernel: reads beyond L2 (the second read of a row is served by the
-    # memory-side cache, which this counter cannot tell from HBM) + one write of dlogits
+    # lmhead_fwd_kernel: L2 misses of the tiled operand re-reads (1.24 GB of unique operands at c3) + the partials
+    "c3": 43.14e9 + 0.19e9,
+    "c4": 40.63e9 + 0.21e9,
+    "c5": 88.61e9 + 0.19e9,
+    # lsg_grpo_fused_kernel: reads beyond L2 (the second read of a row is served by the LDS and the caches; this
+    # counter cannot tell the memory-side cache from HBM) + one write of dlogits
+    "c2": 18.80e9 + 16.82e9,
     "c2-two-pass": 16.83e9 + 0.0e9,  # lsg_entropy_fwd_kernel: 1.00x the logits
 }
 
