@@ -402,9 +402,10 @@ int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, const int64_t
  * The bf16 MFMA main loop of the lm_head kernels as a plain product (no reference counterpart;
  * it exists so that the tile engine can be tested and timed on its own):
  *   out[m, n] (+)= sum_k A[m, k] * B[n, k]      A: bf16 [M, K] (row stride lda), B: bf16 [N, K] (ldb)
- * K must be a multiple of 64, pointers 16-byte aligned, lda/ldb multiples of 8 and at most 2^22 (or
- * 0 = every row aliases row 0).  Exactly one of out_f32 / out_bf16 is written (row stride ldo); accumulate != 0
- * adds to the existing fp32 output.
+ * K must be a multiple of 64, A and B 16-byte aligned, lda/ldb multiples of 8 and at most 2^22 (or
+ * 0 = every row aliases row 0).  Exactly one of out_f32 / out_bf16 is written (row stride ldo; out_bf16
+ * 4-byte aligned when ldo is even, its rows are then stored as pairs); accumulate != 0 adds to the
+ * existing fp32 output.
  */
 int oi_gemm_bf16_tn(const void* A, int64_t lda, int64_t M, const void* B, int64_t ldb, int64_t N, int64_t K,
                     float* out_f32, void* out_bf16, int64_t ldo, int accumulate, void* stream);

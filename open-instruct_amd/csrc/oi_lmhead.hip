@@ -1280,6 +1280,8 @@ extern "C" int oi_gemm_bf16_tn(const void* A, int64_t lda, int64_t M, const void
     OI_RETURN_IF(!A || !B || (!out_f32 && !out_bf16) || (out_f32 && out_bf16), OI_ENULL);
     OI_RETURN_IF(accumulate && !out_f32, OI_EINVAL);
     OI_RETURN_IF(!oi_aligned(A, 16) || !oi_aligned(B, 16), OI_EALIGN);
+    // bf16 rows of even pitch are written as pairs (4-byte words), fp32 results as single words
+    OI_RETURN_IF(!oi_aligned(out_f32, 4) || !oi_aligned(out_bf16, (ldo & 1) ? 2 : 4), OI_EALIGN);
     const int mode = out_f32 ? (accumulate ? 1 : 0) : 2;
     const Operand a = {static_cast<const uint16_t*>(A), lda, 0, M, K};
     const Operand b = {static_cast<const uint16_t*>(B), ldb, 0, N, K};
@@ -1300,6 +1302,8 @@ extern "C" int oi_gemm_bf16_layouts(const void* A, int64_t lda, int a_k_major, c
     OI_RETURN_IF(!A || !B || (!out_f32 && !out_bf16) || (out_f32 && out_bf16), OI_ENULL);
     OI_RETURN_IF(accumulate && !out_f32, OI_EINVAL);
     OI_RETURN_IF(!oi_aligned(A, 16) || !oi_aligned(B, 16), OI_EALIGN);
+    // bf16 rows of even pitch are written as pairs (4-byte words), fp32 results as single words
+    OI_RETURN_IF(!oi_aligned(out_f32, 4) || !oi_aligned(out_bf16, (ldo & 1) ? 2 : 4), OI_EALIGN);
     const int mode = out_f32 ? (accumulate ? 1 : 0) : 2;
     const Operand a = {static_cast<const uint16_t*>(A), lda, 0, M, K};
     const Operand b = {static_cast<const uint16_t*>(B), ldb, 0, N, K};
