@@ -83,7 +83,7 @@ class EventTimer:
 # ------------------------------------------------------------------------------------------------
 # workloads
 # ------------------------------------------------------------------------------------------------
-def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=False):
+def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=False, cache_chunks=0):
     dev = "cuda:0"
     torch.manual_seed(0)
     hidden = torch.randn(n_tokens, hdim, device=dev).bfloat16().requires_grad_(True)
@@ -120,17 +120,22 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=Fals
         if one_call:
             with fwd_timer:  # the whole step is one C call here: the timer brackets all of it
                 loss, _, _, _ = oi.grpo_utils.grpo_loss_on_hidden(
-                    hidden[None], weight, labels[None], old[None], ref[None], adv[None], mask[None], cfg
+                    hidden[None], weight, labels[None], old[None], ref[None], adv[None], mask[None], cfg,
+                    logit_cache_chunks=cache_chunks,
                 )
         elif not dpo:
             with fwd_timer:
-                lp, ent = oi.fused_lm_head_logprobs(hidden, weight, labels, mask=mask, return_entropy=True)
+                lp, ent = oi.fused_lm_head_logprobs(
+                    hidden, weight, labels, mask=mask, return_entropy=True, logit_cache_chunks=cache_chunks
+                )
             loss, _ = oi.grpo_utils.grpo_loss_fused(
                 lp[None], old[None], ref[None], adv[None], mask[None], cfg, entropy=ent[None]
             )
         else:
             with fwd_timer:
-                lp, _ = oi.fused_lm_head_logprobs(hidden, weight, shifted.view(-1), mask=mask)
+                lp, _ = oi.fused_lm_head_logprobs(
+                    hidden, weight, shifted.view(-1), mask=mask, logit_cache_chunks=cache_chunks
+                )
             logps = oi.padding_free_collator.get_batch_logps(lp.view(1, -1), labels, cu)
             bs = logps.shape[0] // 2
             losses, _, _ = oi.dpo_utils.dpo_loss(logps[:bs], logps[bs:], ref_c, ref_r, beta=0.1)
@@ -482,6 +487,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="c3",
                     choices=["c1", "c2", "c2-two-pass", "c3", "c3-one-call", "c4", "c5", "pack"])
+    ap.add_argument("--cache-chunks", type=int, default=0,
+                    help="c3 / c3-one-call / c5 only: keep 2^logit in bf16 for this many vocabulary chunks of 32768 "
+                         "columns instead of recomputing them in the backward pass (0 = the headline configuration: "
+                         "nothing of size [tokens, vocab] is stored)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-library-gemm", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -501,11 +510,11 @@ def main():
     oi._lib.load()
 
     if args.workload == "c3":
-        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02)
-        name = "c3: fused lm_head+logprob+entropy+GRPO loss fwd+bwd, hidden bf16 [32768,4096], W bf16 [128256,4096], 70% response tokens (rows compacted)"
+        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02, cache_chunks=args.cache_chunks)
+        name = "c3: fused lm_head+logprob+entropy+GRPO loss fwd+bwd, hidden bf16 [32768,4096], W bf16 [128256,4096], 70% response tokens (rows selected on the device)"
         dtype = "bf16"
     elif args.workload == "c3-one-call":
-        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02, one_call=True)
+        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02, one_call=True, cache_chunks=args.cache_chunks)
         name = "c3: the same step through the single entry point grpo_loss_on_hidden (oi_lmhead_grpo_fwd_bwd)"
         dtype = "bf16"
     elif args.workload == "c4":
@@ -513,7 +522,7 @@ def main():
         name = "c4: packed OLMo-2-7B shape, 16 sequences via cu_seqlens, hidden bf16 [N<=32768,4096], W bf16 [100352,4096]; per-sequence logprob sums + GRPO loss masked_mean(axis=1), fwd+bwd"
         dtype = "bf16"
     elif args.workload == "c5":
-        step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True)
+        step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True, cache_chunks=args.cache_chunks)
         name = "c5: fused lm_head+per-sequence logprob sums+sigmoid DPO loss, hidden bf16 [32768,8192], W bf16 [128256,8192], bwd to dHidden only"
         dtype = "bf16"
     elif args.workload == "c2":
@@ -533,6 +542,11 @@ def main():
         name = "c1: logprob+entropy+masked_mean on fp32 logits [4,512,32000], forward"
         dtype = "f32"
 
+    if args.cache_chunks:
+        if args.workload not in ("c3", "c3-one-call", "c5"):
+            print("--cache-chunks applies to c3, c3-one-call and c5")
+            sys.exit(2)
+        name += f" [NOT the headline configuration: 2^logit of {args.cache_chunks} vocabulary chunk(s) kept in bf16 for the backward pass]"
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_(0, 255)
         dst = torch.empty_like(src)

@@ -351,7 +351,25 @@ int oi_pack_sequences(const int64_t* q_tokens, const int64_t* q_offsets, const i
 size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int with_row_mask);
 int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* labels, const uint8_t* row_mask,
                        int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob,
-                       float* entropy, float* lse, void* workspace, size_t workspace_bytes, void* stream);
+                       float* entropy, float* lse, void* exp_cache, int64_t cache_chunks, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/*
+ * Optional cache of exponentials (cache_chunks > 0; 0 = off, the default of the Python mirror: the
+ * backward then recomputes every chunk and nothing of size [tokens, vocab] exists).  It trades memory
+ * for the recomputation: the forward also stores 2^(z * inv_T * log2 e) in bf16 (whose exponent
+ * range is that of fp32, so no per-token reference is needed) for the first cache_chunks chunks of
+ * 32768 vocabulary columns, token-major, oi_lmhead_cache_bytes() bytes at exp_cache (16-byte aligned,
+ * owned by the caller, handed unchanged to the backward call of the same rows).  For a cached chunk
+ * the backward multiplies the cache itself: dZ[n, v] = s_n (e'[n, v] - 1[v = label_n] 2^lse2_n) with
+ * the per-token factor s_n = -g_n inv_T 2^(-lse2_n) moved out of the products (a row factor of
+ * d_hidden, a factor of the hidden rows in d_weight), and the label's entry replaced by
+ * 2^lse2_n * expm1(logprob_n).  Costs 2 bytes per cached logit (8.4 GB for all four chunks at
+ * 32768 x 128256), saves a quarter of the step's matrix work when every chunk is cached.  Needs
+ * |z * inv_T| < 87 (2^126); the rounding of a cached entry is the bf16 rounding that a dZ entry
+ * undergoes anyway.
+ */
+size_t oi_lmhead_cache_bytes(int64_t n_tokens, int64_t vocab, int64_t cache_chunks);
 
 /*
  * Backward: recomputes the logits tile by tile,
@@ -363,14 +381,17 @@ int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* la
  * read weight, hidden and dZ where they lie (no transposed copies), so the workspace is the same
  * with and without d_weight.  row_mask as in the forward (rows left out get a zero d_hidden row
  * and add nothing to d_weight); skip_zero_grad_rows != 0 also leaves out rows whose grad_logprob is
- * exactly 0, which changes no result.  d_hidden and d_weight must be 4-byte aligned.
+ * exactly 0, which changes no result (not together with a cache, whose rows are the forward's).
+ * d_hidden and d_weight must be 4-byte aligned.  logprob (the forward's output) is read only with a
+ * cache.
  */
 size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int want_d_weight,
-                                     int with_row_selection);
+                                     int with_row_selection, int with_cache);
 int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
                        const float* grad_logprob, const uint8_t* row_mask, int skip_zero_grad_rows, int64_t n_tokens,
-                       int64_t hidden_dim, int64_t vocab, float inv_temperature, void* d_hidden, void* d_weight,
-                       void* workspace, size_t workspace_bytes, void* stream);
+                       int64_t hidden_dim, int64_t vocab, float inv_temperature, const float* logprob,
+                       void* exp_cache, int64_t cache_chunks, void* d_hidden, void* d_weight, void* workspace,
+                       size_t workspace_bytes, void* stream);
 
 /*
  * The whole GRPO step on hidden states in one call: fused lm_head forward (logprob, entropy),
@@ -388,15 +409,17 @@ int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* la
  * [rows, cols], 0 off the mask.  d_weight NULL skips that product.  A token's upstream gradient
  * depends only on its own logprob once the denominators are known, and those come from the mask, so
  * the backward is enqueued straight behind the forward: nothing returns to the host in between.
+ * exp_cache / cache_chunks: the optional cache of exponentials described at oi_lmhead_cache_bytes
+ * (scratch of this one call here; NULL / 0 = recompute every chunk).
  */
-size_t oi_lmhead_grpo_workspace_bytes(int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab);
+size_t oi_lmhead_grpo_workspace_bytes(int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab, int with_cache);
 int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, const int64_t* labels, const uint8_t* mask,
                            const float* old_logprobs, const float* ref_logprobs, const float* advantages,
                            const float* rho_weights, int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab,
                            float inv_temperature, int loss_fn, float ratio_lo, float ratio_hi, int kl_estimator,
                            float beta, int axis_mode, float denominator, float scale, float* logprob, float* entropy,
-                           float* out_stats, void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes,
-                           void* stream);
+                           float* out_stats, void* d_hidden, void* d_weight, void* exp_cache, int64_t cache_chunks,
+                           void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * The bf16 MFMA main loop of the lm_head kernels as a plain product (no reference counterpart;

@@ -441,7 +441,10 @@ __device__ __forceinline__ void merge_stats(float ma, float sa, float ta, float 
 // Fold the 32 logits that one lane holds for token column j of a finished tile into the running
 // statistics.  PARTIAL handles the last vocabulary tile: rows past the vocabulary are skipped by
 // predicate (weight exactly 0) instead of through a sentinel value.
-template <bool PARTIAL>
+// KEEP leaves 2^x in place of every logit (0 for rows past the vocabulary): the exponentials of the
+// statistics times 2^max, for the cache of exponentials that the backward pass can use in place of
+// a recomputation.
+template <bool PARTIAL, bool KEEP>
 __device__ __forceinline__ void stats_update(AccTile& acc, int j, int wm, int lane, int64_t m0, int64_t vocab, float c,
                                              float& st_m, float& st_s, float& st_t) {
     float vmax = OI_NEG_BIG;
@@ -458,6 +461,7 @@ __device__ __forceinline__ void stats_update(AccTile& acc, int j, int wm, int la
     const float alpha = __builtin_amdgcn_exp2f(shift);
     float s = st_s * alpha;
     float t = alpha * fmaf(shift, st_s, st_t);
+    const float pow2_max = KEEP ? __builtin_amdgcn_exp2f(fminf(mn, 126.f)) : 0.f;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -470,20 +474,58 @@ __device__ __forceinline__ void stats_update(AccTile& acc, int j, int wm, int la
             }
             s += e;
             t = fmaf(e, d, t);
+            if (KEEP) acc[i][j][r] = e * pow2_max;
         }
     st_m = mn;
     st_s = s;
     st_t = t;
 }
 
+// A finished tile as a bf16 image [256 tokens][256 vocabulary columns] in the LDS (rows of
+// STAGE_STRIDE entries; the two 8-byte halves of every 16-byte piece swapped in rows 8..15 of each
+// 16, which keeps the 8-byte stores of a wave off each other's banks), and from there to global
+// memory in 16-byte pieces of whole 512-byte rows.  Rows at or past rows_valid are written as zeros.
+__device__ __forceinline__ void stage_tile_bf16(const AccTile& acc, uint16_t* stage, int wm, int wn, int lane) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int nl = acc_col(wn, j, lane);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int vl = acc_row(wm, i, q * 4, lane) ^ (((nl >> 3) & 1) << 2);
+                const uint2 pk = make_uint2(oi_pack_bf16x2(acc[i][j][q * 4], acc[i][j][q * 4 + 1]),
+                                            oi_pack_bf16x2(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]));
+                *reinterpret_cast<uint2*>(stage + nl * STAGE_STRIDE + vl) = pk;
+            }
+    }
+}
+__device__ __forceinline__ void copy_staged_tile(const uint16_t* stage, uint16_t* __restrict__ dst, int64_t ld, int tid,
+                                                 int rows_valid) {
+#pragma unroll 4
+    for (int it = 0; it < 16; ++it) {
+        const int cidx = tid + it * NTHREADS;
+        const int row = cidx >> 5, ch = cidx & 31;
+        oi_u32x4 v = *reinterpret_cast<const oi_u32x4*>(stage + row * STAGE_STRIDE + ch * 8);
+        if (row & 8) v = oi_u32x4{v.z, v.w, v.x, v.y};
+        if (row >= rows_valid) v = oi_u32x4{0u, 0u, 0u, 0u};
+        *reinterpret_cast<oi_u32x4*>(dst + (int64_t)row * ld + ch * 8) = v;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // forward: per-token softmax statistics over the vocabulary tiles of one split
 // ---------------------------------------------------------------------------------------------
+// CACHE: the first cache_tiles vocabulary tiles also leave 2^(z c) behind as bf16, token-major
+// [n_pad, cache_ld] (bf16 has the exponent range of fp32, so no per-token reference is needed);
+// rows of tokens past the end are zero.
+template <bool CACHE>
 __device__ __forceinline__ void lmhead_fwd_item(const uint16_t* __restrict__ W, const uint16_t* __restrict__ hidden,
                                                 const int64_t* __restrict__ labels, int64_t n_tokens, int64_t hdim,
                                                 int64_t vocab, float c, int64_t tiles_per_split, int64_t n_pad,
                                                 float4* __restrict__ partial, float* __restrict__ zy, int64_t split,
-                                                int64_t tt, uint16_t* lds) {
+                                                int64_t tt, uint16_t* __restrict__ ecache, int64_t cache_ld,
+                                                int64_t cache_tiles, uint16_t* lds) {
     const int64_t vocab_tiles = (vocab + BM - 1) / BM;
     const int64_t vt_begin = split * tiles_per_split;
     int64_t vt_end = vt_begin + tiles_per_split;
@@ -529,9 +571,18 @@ __device__ __forceinline__ void lmhead_fwd_item(const uint16_t* __restrict__ W, 
                 }
             }
             if (partial_tile)
-                stats_update<true>(acc, j, wm, lane, m0, vocab, c, st_m[j], st_s[j], st_t[j]);
+                stats_update<true, CACHE>(acc, j, wm, lane, m0, vocab, c, st_m[j], st_s[j], st_t[j]);
             else
-                stats_update<false>(acc, j, wm, lane, m0, vocab, c, st_m[j], st_s[j], st_t[j]);
+                stats_update<false, CACHE>(acc, j, wm, lane, m0, vocab, c, st_m[j], st_s[j], st_t[j]);
+        }
+        if (CACHE && vt < cache_tiles) {
+            // the operand ring is free (the product ended with a barrier); the next tile's first loads
+            // must wait until the image has been read out again
+            stage_tile_bf16(acc, lds, wm, wn, lane);
+            __syncthreads();
+            const int64_t left = n_tokens - n0;
+            copy_staged_tile(lds, ecache + n0 * cache_ld + vt * BM, cache_ld, tid, (int)(left < BN ? left : BN));
+            __syncthreads();
         }
     }
 
@@ -563,17 +614,19 @@ __device__ __forceinline__ void lmhead_fwd_item(const uint16_t* __restrict__ W, 
     }
 }
 
+template <bool CACHE>
 __global__ void __launch_bounds__(NTHREADS)
     lmhead_fwd_kernel(const uint16_t* __restrict__ W, const uint16_t* __restrict__ hidden,
                       const int64_t* __restrict__ labels, int64_t n_tokens, const int32_t* __restrict__ n_dev,
                       int64_t hdim, int64_t vocab, float c, int64_t n_splits, int64_t tiles_per_split, int64_t n_pad,
-                      float4* __restrict__ partial, float* __restrict__ zy, uint32_t* __restrict__ queue) {
+                      float4* __restrict__ partial, float* __restrict__ zy, uint16_t* __restrict__ ecache,
+                      int64_t cache_ld, int64_t cache_tiles, uint32_t* __restrict__ queue) {
     __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
     if (n_dev) n_tokens = *n_dev;  // rows selected on the device: the host only knows an upper bound
     const int64_t token_tiles = (n_tokens + BN - 1) / BN;
     for_each_tile(queue, n_splits, token_tiles, lds, [&](int64_t split, int64_t tt) {
-        lmhead_fwd_item(W, hidden, labels, n_tokens, hdim, vocab, c, tiles_per_split, n_pad, partial, zy, split, tt,
-                        lds);
+        lmhead_fwd_item<CACHE>(W, hidden, labels, n_tokens, hdim, vocab, c, tiles_per_split, n_pad, partial, zy, split,
+                               tt, ecache, cache_ld, cache_tiles, lds);
     });
 }
 
@@ -712,8 +765,9 @@ __global__ void __launch_bounds__(NTHREADS)
 template <bool A_KM, bool B_KM>
 __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B, int64_t N, int64_t K, int mode,
                                                 float* out_f32, uint16_t* out_bf16, int64_t ldo, int64_t m_valid,
-                                                const int32_t* __restrict__ out_rows, int64_t tm, int64_t tn,
-                                                uint16_t* lds) {
+                                                const int32_t* __restrict__ out_rows,
+                                                const float* __restrict__ scale_a, const float* __restrict__ scale_b,
+                                                int64_t tm, int64_t tn, uint16_t* lds) {
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6, wm = wave & 3, wn = wave >> 2;
     const int64_t m0 = tm * BM, n0 = tn * BN;
     A.r0 = m0;
@@ -743,6 +797,7 @@ __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B,
                 // holds the row before it and needs this lane's half of that row
                 const bool row_ok = row < m_valid;
                 const int64_t dst_row = (row_ok && out_rows) ? (int64_t)out_rows[row] : row;
+                const float sa = (row_ok && scale_a) ? scale_a[row] : 1.f, sb = (row_ok && scale_a) ? scale_b[row] : 1.f;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int64_t col = n0 + (acc_col(wn, j, lane) & ~1);
@@ -752,6 +807,10 @@ __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B,
                         __builtin_amdgcn_mov_dpp(__float_as_int(send), 0xB1 /* quad_perm 1,0,3,2 */, 0xF, 0xF, true));
                     float lo = odd ? recv : own0, hi = odd ? own1 : recv;
                     if (!row_ok || col >= N) continue;
+                    if (scale_a) {
+                        lo = lo * sa * sb;
+                        hi = hi * sa * sb;
+                    }
                     const int64_t o = row * ldo + col, d = dst_row * ldo + col;
                     if (col + 1 < N) {
                         if (mode == 3) {
@@ -780,6 +839,7 @@ __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B,
                 if (row >= m_valid) continue;
                 const int64_t o = row * ldo + col;
                 float v = acc[i][j][r];
+                if (scale_a) v = v * scale_a[row] * scale_b[row];
                 if (mode == 1 || mode == 3) v += out_f32[o];
                 if (mode <= 1) out_f32[o] = v;
                 else out_bf16[(out_rows ? (int64_t)out_rows[row] : row) * ldo + col] = (uint16_t)oi_f32_to_bf16_bits(v);
@@ -794,6 +854,9 @@ struct DynRows {
     const int32_t* n_dev;
     int role;
     const int32_t* out_rows;
+    // optional factors of row r of the product, applied as (acc * scale_a[r]) * scale_b[r] before it
+    // is stored or accumulated (two factors so that neither has to leave the fp32 range)
+    const float *scale_a, *scale_b;
 };
 
 // `queue` null: one workgroup per tile id (blockIdx); otherwise a launch of resident workgroups
@@ -818,12 +881,14 @@ __global__ void __launch_bounds__(NTHREADS)
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (queue) {
         for_each_tile(queue, tiles_m, tiles_n, lds, [&](int64_t tm, int64_t tn) {
-            gemm_store_tile<A_KM, B_KM>(A, M, B, N, K, mode, out_f32, out_bf16, ldo, m_valid, dyn.out_rows, tm, tn, lds);
+            gemm_store_tile<A_KM, B_KM>(A, M, B, N, K, mode, out_f32, out_bf16, ldo, m_valid, dyn.out_rows, dyn.scale_a,
+                                        dyn.scale_b, tm, tn, lds);
         });
     } else {
         int64_t tm, tn;
         if (tile_of_block(tiles_m, tiles_n, &tm, &tn))
-            gemm_store_tile<A_KM, B_KM>(A, M, B, N, K, mode, out_f32, out_bf16, ldo, m_valid, dyn.out_rows, tm, tn, lds);
+            gemm_store_tile<A_KM, B_KM>(A, M, B, N, K, mode, out_f32, out_bf16, ldo, m_valid, dyn.out_rows, dyn.scale_a,
+                                        dyn.scale_b, tm, tn, lds);
     }
 }
 
@@ -882,9 +947,10 @@ __global__ void __launch_bounds__(SELECT_THREADS)
 __global__ void __launch_bounds__(256)
     gather_rows_kernel(const uint16_t* __restrict__ hidden, const int64_t* __restrict__ labels,
                        const float* __restrict__ lse, const float* __restrict__ grad,
-                       const int32_t* __restrict__ rows, const int32_t* __restrict__ count, int64_t hdim,
-                       uint16_t* __restrict__ hidden_c, int64_t* __restrict__ labels_c, float* __restrict__ lse_c,
-                       float* __restrict__ grad_c) {
+                       const float* __restrict__ logprob, const int32_t* __restrict__ rows,
+                       const int32_t* __restrict__ count, int64_t hdim, uint16_t* __restrict__ hidden_c,
+                       int64_t* __restrict__ labels_c, float* __restrict__ lse_c, float* __restrict__ grad_c,
+                       float* __restrict__ logprob_c) {
     const int64_t j = blockIdx.x;
     if (j >= *count) return;
     const int64_t src = rows[j];
@@ -895,6 +961,55 @@ __global__ void __launch_bounds__(256)
         labels_c[j] = labels[src];
         if (lse_c) lse_c[j] = lse[src];
         if (grad_c) grad_c[j] = grad[src];
+        if (logprob_c) logprob_c[j] = logprob[src];
+    }
+}
+
+// Backward from the cache of exponentials e'[n, v] = 2^(x_nv), x = z c:
+//   dZ[n, v] = g_n inv_T (1[v = y_n] - 2^(x_nv - lse2_n)) = s_n (e'[n, v] - 1[v = y_n] 2^lse2_n),
+//   s_n = -g_n inv_T 2^(-lse2_n).
+// The per-token factor leaves the products: d_hidden[n] = s_n (e'[n, :] W) (a row factor in the
+// store epilogue) and d_weight = e'^T (s h) (the hidden rows are scaled once).  This kernel writes
+// the two halves of s_n (so that neither leaves the fp32 range) and replaces the label's entry of
+// the cache by 2^x_y - 2^lse2 = 2^lse2 expm1(logprob), evaluated in fp32 from the forward's result.
+__global__ void cache_rows_prepare_kernel(const float* __restrict__ lse, const float* __restrict__ grad,
+                                          const float* __restrict__ logprob, const int64_t* __restrict__ labels,
+                                          const int32_t* __restrict__ n_dev, int64_t n_tokens, float inv_t,
+                                          int64_t vocab, uint16_t* __restrict__ ecache, int64_t cache_ld,
+                                          float* __restrict__ scale_a, float* __restrict__ scale_b) {
+    const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (n_dev) n_tokens = *n_dev;
+    if (n >= n_tokens) return;
+    const float l2 = lse[n] * OI_LOG2E;
+    const float half = __builtin_amdgcn_exp2f(-0.5f * l2);
+    scale_a[n] = half;
+    scale_b[n] = -grad[n] * inv_t * half;
+    int64_t y = labels[n];
+    y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
+    if (y < cache_ld)
+        ecache[n * cache_ld + y] =
+            (uint16_t)oi_f32_to_bf16_bits(__builtin_amdgcn_exp2f(fminf(l2, 126.f)) * expm1f(logprob[n]));
+}
+
+// scaled[n, :] = (hidden[n, :] * a_n) * b_n in bf16, one workgroup per row
+__global__ void __launch_bounds__(256)
+    scale_rows_kernel(const uint16_t* __restrict__ hidden, const float* __restrict__ scale_a,
+                      const float* __restrict__ scale_b, const int32_t* __restrict__ n_dev, int64_t n_tokens,
+                      int64_t hdim, uint16_t* __restrict__ scaled) {
+    const int64_t n = blockIdx.x;
+    if (n_dev) n_tokens = *n_dev;
+    if (n >= n_tokens) return;
+    const float a = scale_a[n], b = scale_b[n];
+    const oi_u32x4* from = reinterpret_cast<const oi_u32x4*>(hidden + n * hdim);
+    oi_u32x4* to = reinterpret_cast<oi_u32x4*>(scaled + n * hdim);
+    for (int64_t c = threadIdx.x; c < hdim / 8; c += blockDim.x) {
+        const oi_u32x4 v = from[c];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            o[k] = oi_pack_bf16x2(oi_bf16lo_to_f32(w[k]) * a * b, oi_bf16hi_to_f32(w[k]) * a * b);
+        to[c] = oi_u32x4{o[0], o[1], o[2], o[3]};
     }
 }
 
@@ -937,7 +1052,7 @@ struct Carver {
 
 // buffers of a row selection: the row index, the selected count and the compacted per-row inputs
 struct SelectionPlan {
-    size_t off_rows, off_count, off_hidden, off_labels, off_lse, off_grad;
+    size_t off_rows, off_count, off_hidden, off_labels, off_lse, off_grad, off_logprob;
 };
 SelectionPlan plan_selection(Carver& cv, int64_t n_pad, int64_t hdim, bool backward) {
     SelectionPlan p;
@@ -947,7 +1062,26 @@ SelectionPlan plan_selection(Carver& cv, int64_t n_pad, int64_t hdim, bool backw
     p.off_labels = cv.take((size_t)n_pad * sizeof(int64_t));
     p.off_lse = backward ? cv.take((size_t)n_pad * sizeof(float)) : 0;
     p.off_grad = backward ? cv.take((size_t)n_pad * sizeof(float)) : 0;
+    p.off_logprob = backward ? cv.take((size_t)n_pad * sizeof(float)) : 0;
     return p;
+}
+
+// The cache of exponentials: 2^(z c) in bf16 for the first `chunks` vocabulary chunks of the
+// backward pass, token-major [n_pad, ld].
+struct CachePlan {
+    int64_t chunks, ld, tiles;
+    size_t bytes;
+};
+CachePlan plan_cache(int64_t n_tokens, int64_t vocab, int64_t cache_chunks) {
+    const int64_t n_pad = (n_tokens + 255) / 256 * 256, v_pad = (vocab + 255) / 256 * 256;
+    const int64_t chunk = v_pad < BWD_VOCAB_CHUNK ? v_pad : BWD_VOCAB_CHUNK;
+    const int64_t n_chunks = (v_pad + chunk - 1) / chunk;
+    CachePlan c;
+    c.chunks = cache_chunks < 0 ? 0 : (cache_chunks > n_chunks ? n_chunks : cache_chunks);
+    c.ld = c.chunks * chunk < v_pad ? c.chunks * chunk : v_pad;
+    c.tiles = c.ld / BM;
+    c.bytes = (size_t)n_pad * c.ld * 2;
+    return c;
 }
 
 struct FwdPlan {
@@ -979,10 +1113,10 @@ FwdPlan plan_fwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_select
 
 struct BwdPlan {
     int64_t n_pad, v_pad, chunk, n_chunks;
-    size_t off_dz, off_dh32, off_queues, total;
+    size_t off_dz, off_dh32, off_queues, off_scale_a, off_scale_b, off_scaled_hidden, total;
     SelectionPlan sel;
 };
-BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_selection) {
+BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_selection, bool with_cache = false) {
     BwdPlan p;
     p.n_pad = round_up(n_tokens, 256);
     p.v_pad = round_up(vocab, 256);
@@ -994,6 +1128,12 @@ BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_select
     // one set of work-queue counters per tile-kernel launch (three per vocabulary chunk)
     p.off_queues = cv.take((size_t)(3 * p.n_chunks) * QUEUE_WORDS * sizeof(uint32_t));
     if (with_selection) p.sel = plan_selection(cv, p.n_pad, hdim, true);
+    p.off_scale_a = p.off_scale_b = p.off_scaled_hidden = 0;
+    if (with_cache) {
+        p.off_scale_a = cv.take((size_t)p.n_pad * sizeof(float));
+        p.off_scale_b = cv.take((size_t)p.n_pad * sizeof(float));
+        p.off_scaled_hidden = cv.take((size_t)p.n_pad * hdim * 2);
+    }
     p.total = cv.off;
     return p;
 }
@@ -1018,49 +1158,61 @@ struct RowInputs {
     const int64_t* labels;
     const float *lse, *grad;
     const int32_t *rows, *n_dev;  // null without a selection
+    const float* logprob;         // only with a cache of exponentials
 };
 
 // select + gather on `s`; clears `n_zero` queue words on the way
 RowInputs launch_selection(const SelectionPlan& sp, char* ws, const void* hidden, const int64_t* labels,
                            const float* lse, const float* grad, const uint8_t* row_mask, bool skip_zero_grad,
-                           int64_t n_tokens, int64_t hdim, uint32_t* zero_words, int n_zero, hipStream_t s) {
+                           int64_t n_tokens, int64_t hdim, uint32_t* zero_words, int n_zero, hipStream_t s,
+                           const float* logprob = nullptr) {
     int32_t* rows = reinterpret_cast<int32_t*>(ws + sp.off_rows);
     int32_t* count = reinterpret_cast<int32_t*>(ws + sp.off_count);
     uint16_t* hidden_c = reinterpret_cast<uint16_t*>(ws + sp.off_hidden);
     int64_t* labels_c = reinterpret_cast<int64_t*>(ws + sp.off_labels);
     float* lse_c = lse ? reinterpret_cast<float*>(ws + sp.off_lse) : nullptr;
     float* grad_c = grad ? reinterpret_cast<float*>(ws + sp.off_grad) : nullptr;
+    float* logprob_c = logprob ? reinterpret_cast<float*>(ws + sp.off_logprob) : nullptr;
     hipLaunchKernelGGL(select_rows_kernel, dim3(1), dim3(SELECT_THREADS), 0, s, row_mask,
                        skip_zero_grad ? grad : static_cast<const float*>(nullptr), n_tokens, rows, count, zero_words,
                        n_zero);
     hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s,
-                       static_cast<const uint16_t*>(hidden), labels, lse, grad, rows, count, hdim, hidden_c, labels_c,
-                       lse_c, grad_c);
-    return RowInputs{hidden_c, labels_c, lse_c, grad_c, rows, count};
+                       static_cast<const uint16_t*>(hidden), labels, lse, grad, logprob, rows, count, hdim, hidden_c,
+                       labels_c, lse_c, grad_c, logprob_c);
+    return RowInputs{hidden_c, labels_c, lse_c, grad_c, rows, count, logprob_c};
 }
 
-// lse and upstream gradient of the selected rows (the rows were selected and gathered earlier)
-__global__ void gather_f32_pair_kernel(const float* __restrict__ lse, const float* __restrict__ grad,
-                                       const int32_t* __restrict__ rows, const int32_t* __restrict__ count,
-                                       float* __restrict__ lse_c, float* __restrict__ grad_c) {
+// lse, upstream gradient and logprob of the selected rows (the rows were selected and gathered earlier)
+__global__ void gather_f32_kernel(const float* __restrict__ lse, const float* __restrict__ grad,
+                                  const float* __restrict__ logprob, const int32_t* __restrict__ rows,
+                                  const int32_t* __restrict__ count, float* __restrict__ lse_c,
+                                  float* __restrict__ grad_c, float* __restrict__ logprob_c) {
     const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (j >= *count) return;
     const int64_t src = rows[j];
     lse_c[j] = lse[src];
     grad_c[j] = grad[src];
+    logprob_c[j] = logprob[src];
 }
 
 // forward launches: tile kernel + merge of the partial statistics.  `queue` must be zeroed.
 void enqueue_fwd(const FwdPlan& p, char* ws, const RowInputs& in, const uint8_t* row_mask, const void* weight,
                  int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob,
-                 float* entropy, float* lse, hipStream_t s) {
+                 float* entropy, float* lse, uint16_t* ecache, const CachePlan& cache, hipStream_t s) {
     float4* partial = reinterpret_cast<float4*>(ws + p.off_partial);
     float* zy = reinterpret_cast<float*>(ws + p.off_zy);
     uint32_t* queue = reinterpret_cast<uint32_t*>(ws + p.off_queue);
     const float c = inv_temperature * OI_LOG2E;
-    hipLaunchKernelGGL(lmhead_fwd_kernel, dim3(resident_grid(p.n_splits, p.token_tiles)), dim3(NTHREADS), 0, s,
-                       static_cast<const uint16_t*>(weight), in.hidden, in.labels, n_tokens, in.n_dev, hidden_dim, vocab,
-                       c, p.n_splits, p.tiles_per_split, p.n_pad, partial, zy, queue);
+    const dim3 grid(resident_grid(p.n_splits, p.token_tiles));
+    const uint16_t* Wp = static_cast<const uint16_t*>(weight);
+    if (cache.chunks > 0)
+        hipLaunchKernelGGL(lmhead_fwd_kernel<true>, grid, dim3(NTHREADS), 0, s, Wp, in.hidden, in.labels, n_tokens,
+                           in.n_dev, hidden_dim, vocab, c, p.n_splits, p.tiles_per_split, p.n_pad, partial, zy, ecache,
+                           cache.ld, cache.tiles, queue);
+    else
+        hipLaunchKernelGGL(lmhead_fwd_kernel<false>, grid, dim3(NTHREADS), 0, s, Wp, in.hidden, in.labels, n_tokens,
+                           in.n_dev, hidden_dim, vocab, c, p.n_splits, p.tiles_per_split, p.n_pad, partial, zy,
+                           static_cast<uint16_t*>(nullptr), (int64_t)0, (int64_t)0, queue);
     hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
                        zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, logprob,
                        entropy, lse);
@@ -1072,38 +1224,56 @@ void enqueue_fwd(const FwdPlan& p, char* ws, const RowInputs& in, const uint8_t*
 //   d_hidden[n, h] (+)= sum_v dZ[n, v] * W[v_begin + v, h]      A k-contiguous, B k-major
 //   d_weight[v_begin + v, h] = sum_n dZ[n, v] * hidden[n, h]    A k-major,      B k-major
 // The sums stop at the last real vocabulary row / token (rounded up to a k-tile, whose missing
-// rows are read from the last real one and meet zeros of dZ).  The queue words must be zeroed.
+// rows are read from the last real one and meet zeros of dZ).  Chunks that the forward left in the
+// cache of exponentials skip the recomputation: the cache itself is the A operand of both products
+// (see cache_rows_prepare_kernel).  The queue words must be zeroed.
 void enqueue_bwd(const BwdPlan& p, char* ws, const RowInputs& in, const void* weight, int64_t n_tokens,
                  int64_t hidden_dim, int64_t vocab, float inv_temperature, void* d_hidden, void* d_weight,
-                 hipStream_t s) {
+                 uint16_t* ecache, const CachePlan& cache, hipStream_t s) {
     uint16_t* dz = reinterpret_cast<uint16_t*>(ws + p.off_dz);
     float* dh32 = reinterpret_cast<float*>(ws + p.off_dh32);
     uint32_t* queues = reinterpret_cast<uint32_t*>(ws + p.off_queues);
     const uint16_t* Wp = static_cast<const uint16_t*>(weight);
     const float c = inv_temperature * OI_LOG2E;
     const int64_t h_tiles = (hidden_dim + BN - 1) / BN;
+    float* scale_a = reinterpret_cast<float*>(ws + p.off_scale_a);
+    float* scale_b = reinterpret_cast<float*>(ws + p.off_scale_b);
+    uint16_t* scaled_hidden = reinterpret_cast<uint16_t*>(ws + p.off_scaled_hidden);
+    if (cache.chunks > 0) {
+        hipLaunchKernelGGL(cache_rows_prepare_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, in.lse,
+                           in.grad, in.logprob, in.labels, in.n_dev, n_tokens, inv_temperature, vocab, ecache, cache.ld,
+                           scale_a, scale_b);
+        if (d_weight)
+            hipLaunchKernelGGL(scale_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, in.hidden, scale_a, scale_b,
+                               in.n_dev, n_tokens, hidden_dim, scaled_hidden);
+    }
     for (int64_t ci = 0; ci < p.n_chunks; ++ci) {
         const int64_t v_begin = ci * p.chunk;
         const int64_t cols = (p.v_pad - v_begin) < p.chunk ? (p.v_pad - v_begin) : p.chunk;  // multiple of 256
         const int64_t valid = vocab - v_begin < cols ? vocab - v_begin : cols;               // real rows of W
+        const bool cached = ci < cache.chunks;
         uint32_t* q = queues + ci * 3 * QUEUE_WORDS;
-        hipLaunchKernelGGL(lmhead_dz_kernel, dim3(resident_grid(cols / BM, p.n_pad / BN)), dim3(NTHREADS), 0, s, Wp,
-                           in.hidden, in.labels, in.lse, in.grad, n_tokens, in.n_dev, hidden_dim, vocab, c,
-                           inv_temperature, v_begin, cols, p.n_pad, dz, q);
+        if (!cached)
+            hipLaunchKernelGGL(lmhead_dz_kernel, dim3(resident_grid(cols / BM, p.n_pad / BN)), dim3(NTHREADS), 0, s, Wp,
+                               in.hidden, in.labels, in.lse, in.grad, n_tokens, in.n_dev, hidden_dim, vocab, c,
+                               inv_temperature, v_begin, cols, p.n_pad, dz, q);
+        // the A operand of both products: this chunk's dZ, or this chunk's columns of the cache
+        const uint16_t* a_ptr = cached ? ecache + v_begin : dz;
+        const int64_t a_ld = cached ? cache.ld : cols;
         const bool first = ci == 0, last = ci == p.n_chunks - 1;
         const int mode = last ? (first ? 2 : 3) : (first ? 0 : 1);
         {
-            const Operand a = {dz, cols, 0, p.n_pad, cols};
+            const Operand a = {a_ptr, a_ld, 0, p.n_pad, cols};
             const Operand b = {Wp + v_begin * hidden_dim, hidden_dim, 0, hidden_dim, valid};
-            const DynRows dyn = {in.n_dev, 1, in.rows};
+            const DynRows dyn = {in.n_dev, 1, in.rows, cached ? scale_a : nullptr, cached ? scale_b : nullptr};
             hipLaunchKernelGGL((gemm_store_kernel<false, true>), dim3(resident_grid(p.n_pad / BM, h_tiles)),
                                dim3(NTHREADS), 0, s, a, p.n_pad, b, hidden_dim, round_up(valid, BK), mode, dh32,
                                static_cast<uint16_t*>(d_hidden), hidden_dim, n_tokens, dyn, q + QUEUE_WORDS);
         }
         if (d_weight) {
-            const Operand a = {dz, cols, 0, cols, p.n_pad};
-            const Operand b = {in.hidden, hidden_dim, 0, hidden_dim, n_tokens};
-            const DynRows dyn = {in.n_dev, 2, nullptr};
+            const Operand a = {a_ptr, a_ld, 0, cols, p.n_pad};
+            const Operand b = {cached ? scaled_hidden : in.hidden, hidden_dim, 0, hidden_dim, n_tokens};
+            const DynRows dyn = {in.n_dev, 2, nullptr, nullptr, nullptr};
             hipLaunchKernelGGL((gemm_store_kernel<true, true>), dim3(resident_grid(cols / BM, h_tiles)),
                                dim3(NTHREADS), 0, s, a, cols, b, hidden_dim, round_up(n_tokens, BK), 2,
                                static_cast<float*>(nullptr), static_cast<uint16_t*>(d_weight) + v_begin * hidden_dim,
@@ -1119,11 +1289,11 @@ struct StepPlan {
     BwdPlan bwd;
     size_t off_fwd, off_bwd, off_stats, off_lse, off_grad, off_denoms, total;
 };
-StepPlan plan_step(int64_t rows, int64_t cols, int64_t hdim, int64_t vocab) {
+StepPlan plan_step(int64_t rows, int64_t cols, int64_t hdim, int64_t vocab, bool with_cache) {
     StepPlan p;
     const int64_t n = rows * cols;
     p.fwd = plan_fwd(n, hdim, vocab, false);
-    p.bwd = plan_bwd(n, hdim, vocab, true);
+    p.bwd = plan_bwd(n, hdim, vocab, true, with_cache);
     Carver cv;
     p.off_fwd = cv.take(p.fwd.total);
     p.off_bwd = cv.take(p.bwd.total);
@@ -1135,7 +1305,19 @@ StepPlan plan_step(int64_t rows, int64_t cols, int64_t hdim, int64_t vocab) {
     return p;
 }
 
+int check_cache(const void* exp_cache, int64_t cache_chunks) {
+    OI_RETURN_IF(cache_chunks < 0, OI_EINVAL);
+    OI_RETURN_IF(cache_chunks > 0 && !exp_cache, OI_ENULL);
+    OI_RETURN_IF(!oi_aligned(exp_cache, 16), OI_EALIGN);
+    return OI_OK;
+}
+
 }  // namespace
+
+extern "C" size_t oi_lmhead_cache_bytes(int64_t n_tokens, int64_t vocab, int64_t cache_chunks) {
+    if (n_tokens <= 0 || vocab <= 0 || cache_chunks <= 0) return 0;
+    return plan_cache(n_tokens, vocab, cache_chunks).bytes;
+}
 
 extern "C" size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
                                                 int with_row_mask) {
@@ -1145,72 +1327,85 @@ extern "C" size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden
 
 extern "C" int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* labels,
                                   const uint8_t* row_mask, int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
-                                  float inv_temperature, float* logprob, float* entropy, float* lse, void* workspace,
-                                  size_t workspace_bytes, void* stream) {
-    const int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
+                                  float inv_temperature, float* logprob, float* entropy, float* lse, void* exp_cache,
+                                  int64_t cache_chunks, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
+    if (rc != OI_OK) return rc;
+    rc = check_cache(exp_cache, cache_chunks);
     if (rc != OI_OK) return rc;
     if (n_tokens == 0) return OI_OK;
     OI_RETURN_IF(!logprob || !workspace, OI_ENULL);
     OI_RETURN_IF(!oi_aligned(workspace, 256), OI_EALIGN);
     const FwdPlan p = plan_fwd(n_tokens, hidden_dim, vocab, row_mask != nullptr);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
+    const CachePlan cache = plan_cache(n_tokens, vocab, cache_chunks);
     char* ws = static_cast<char*>(workspace);
     uint32_t* queue = reinterpret_cast<uint32_t*>(ws + p.off_queue);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    RowInputs in = {static_cast<const uint16_t*>(hidden), labels, nullptr, nullptr, nullptr, nullptr};
+    RowInputs in = {static_cast<const uint16_t*>(hidden), labels, nullptr, nullptr, nullptr, nullptr, nullptr};
     if (row_mask)
         in = launch_selection(p.sel, ws, hidden, labels, nullptr, nullptr, row_mask, false, n_tokens, hidden_dim, queue,
                               QUEUE_WORDS, s);
     else
         hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, queue, QUEUE_WORDS);
-    enqueue_fwd(p, ws, in, row_mask, weight, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy, lse, s);
+    enqueue_fwd(p, ws, in, row_mask, weight, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy, lse,
+                static_cast<uint16_t*>(exp_cache), cache, s);
     return oi_launch_status();
 }
 
 extern "C" size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
-                                                int want_d_weight, int with_row_selection) {
+                                                int want_d_weight, int with_row_selection, int with_cache) {
     if (n_tokens <= 0 || hidden_dim <= 0 || vocab <= 0) return 0;
     (void)want_d_weight;
-    return plan_bwd(n_tokens, hidden_dim, vocab, with_row_selection != 0).total;
+    return plan_bwd(n_tokens, hidden_dim, vocab, with_row_selection != 0, with_cache != 0).total;
 }
 
 extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
                                   const float* grad_logprob, const uint8_t* row_mask, int skip_zero_grad_rows,
                                   int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature,
-                                  void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes,
-                                  void* stream) {
-    const int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
+                                  const float* logprob, void* exp_cache, int64_t cache_chunks, void* d_hidden,
+                                  void* d_weight, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
+    if (rc != OI_OK) return rc;
+    rc = check_cache(exp_cache, cache_chunks);
     if (rc != OI_OK) return rc;
     if (n_tokens == 0) return OI_OK;
     OI_RETURN_IF(!lse || !grad_logprob || !d_hidden || !workspace, OI_ENULL);
+    OI_RETURN_IF(cache_chunks > 0 && !logprob, OI_ENULL);
+    // a cache written for the rows of a mask can only be read back for the same rows
+    OI_RETURN_IF(cache_chunks > 0 && skip_zero_grad_rows, OI_EINVAL);
     // bf16 results are stored as pairs (4-byte words)
     OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 4) || !oi_aligned(d_weight, 4), OI_EALIGN);
     const bool selecting = row_mask != nullptr || skip_zero_grad_rows != 0;
-    const BwdPlan p = plan_bwd(n_tokens, hidden_dim, vocab, selecting);
+    const CachePlan cache = plan_cache(n_tokens, vocab, cache_chunks);
+    const BwdPlan p = plan_bwd(n_tokens, hidden_dim, vocab, selecting, cache.chunks > 0);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     hipStream_t s = static_cast<hipStream_t>(stream);
     char* ws = static_cast<char*>(workspace);
     uint32_t* queues = reinterpret_cast<uint32_t*>(ws + p.off_queues);
     const int n_queue_words = (int)(3 * p.n_chunks * QUEUE_WORDS);
     const float* zero_grad_probe = skip_zero_grad_rows ? grad_logprob : nullptr;
-    RowInputs in = {static_cast<const uint16_t*>(hidden), labels, lse, grad_logprob, nullptr, nullptr};
+    RowInputs in = {static_cast<const uint16_t*>(hidden), labels, lse, grad_logprob, nullptr, nullptr, logprob};
     const bool select_clears_queues = selecting && n_queue_words <= SELECT_THREADS;
     if (!select_clears_queues)
         hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_queue_words + 255) / 256)), dim3(256), 0, s, queues,
                            n_queue_words);
     if (selecting) {
         in = launch_selection(p.sel, ws, hidden, labels, lse, grad_logprob, row_mask, skip_zero_grad_rows != 0, n_tokens,
-                              hidden_dim, queues, select_clears_queues ? n_queue_words : 0, s);
+                              hidden_dim, queues, select_clears_queues ? n_queue_words : 0, s,
+                              cache.chunks > 0 ? logprob : nullptr);
         hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, row_mask,
                            zero_grad_probe, hidden_dim, static_cast<uint16_t*>(d_hidden));
     }
-    enqueue_bwd(p, ws, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, d_weight, s);
+    enqueue_bwd(p, ws, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, d_weight,
+                static_cast<uint16_t*>(exp_cache), cache, s);
     return oi_launch_status();
 }
 
-extern "C" size_t oi_lmhead_grpo_workspace_bytes(int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab) {
+extern "C" size_t oi_lmhead_grpo_workspace_bytes(int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab,
+                                                 int with_cache) {
     if (rows <= 0 || cols <= 0 || hidden_dim <= 0 || vocab <= 0) return 0;
-    return plan_step(rows, cols, hidden_dim, vocab).total;
+    return plan_step(rows, cols, hidden_dim, vocab, with_cache != 0).total;
 }
 
 extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, const int64_t* labels,
@@ -1219,15 +1414,18 @@ extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, co
                                       int64_t hidden_dim, int64_t vocab, float inv_temperature, int loss_fn,
                                       float ratio_lo, float ratio_hi, int kl_estimator, float beta, int axis_mode,
                                       float denominator, float scale, float* logprob, float* entropy, float* out_stats,
-                                      void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes,
-                                      void* stream) {
+                                      void* d_hidden, void* d_weight, void* exp_cache, int64_t cache_chunks,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
     OI_RETURN_IF(rows <= 0 || cols <= 0 || rows > MAX_LD || cols > MAX_LD, OI_EINVAL);
     const int64_t n_tokens = rows * cols;
     int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
     if (rc != OI_OK) return rc;
+    rc = check_cache(exp_cache, cache_chunks);
+    if (rc != OI_OK) return rc;
     OI_RETURN_IF(!mask || !advantages || !logprob || !out_stats || !d_hidden || !workspace, OI_ENULL);
     OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 4) || !oi_aligned(d_weight, 4), OI_EALIGN);
-    const StepPlan p = plan_step(rows, cols, hidden_dim, vocab);
+    const CachePlan cache = plan_cache(n_tokens, vocab, cache_chunks);
+    const StepPlan p = plan_step(rows, cols, hidden_dim, vocab, cache.chunks > 0);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     hipStream_t s = static_cast<hipStream_t>(stream);
     char* ws = static_cast<char*>(workspace);
@@ -1236,6 +1434,7 @@ extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, co
     float* lse = reinterpret_cast<float*>(ws + p.off_lse);
     float* grad = reinterpret_cast<float*>(ws + p.off_grad);
     float* row_denoms = reinterpret_cast<float*>(ws + p.off_denoms);
+    uint16_t* ecache = static_cast<uint16_t*>(exp_cache);
 
     // one selection for both passes: it lives in the backward region; the select kernel also clears
     // the backward queues, the forward queue gets the small fill kernel
@@ -1249,7 +1448,8 @@ extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, co
                            bwd_queues, n_queue_words);
     RowInputs in = launch_selection(p.bwd.sel, ws_bwd, hidden, labels, nullptr, nullptr, mask, false, n_tokens,
                                     hidden_dim, bwd_queues, select_clears_queues ? n_queue_words : 0, s);
-    enqueue_fwd(p.fwd, ws_fwd, in, mask, weight, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy, lse, s);
+    enqueue_fwd(p.fwd, ws_fwd, in, mask, weight, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy, lse,
+                ecache, cache, s);
 
     // loss and statistics from the logprobs, then every token's d loss / d logprob (upstream gradient 1)
     rc = oi_grpo_fused_fwd(logprob, old_logprobs, ref_logprobs, advantages, mask, rho_weights, entropy, nullptr, nullptr,
@@ -1261,13 +1461,18 @@ extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, co
                            ratio_lo, ratio_hi, kl_estimator, beta, scale, row_denoms, nullptr, grad, stream);
     if (rc != OI_OK) return rc;
 
-    in.lse = reinterpret_cast<float*>(ws_bwd + p.bwd.sel.off_lse);
-    in.grad = reinterpret_cast<float*>(ws_bwd + p.bwd.sel.off_grad);
-    hipLaunchKernelGGL(gather_f32_pair_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, lse, grad,
-                       in.rows, in.n_dev, const_cast<float*>(in.lse), const_cast<float*>(in.grad));
+    float* lse_c = reinterpret_cast<float*>(ws_bwd + p.bwd.sel.off_lse);
+    float* grad_c = reinterpret_cast<float*>(ws_bwd + p.bwd.sel.off_grad);
+    float* logprob_c = reinterpret_cast<float*>(ws_bwd + p.bwd.sel.off_logprob);
+    hipLaunchKernelGGL(gather_f32_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, lse, grad, logprob,
+                       in.rows, in.n_dev, lse_c, grad_c, logprob_c);
+    in.lse = lse_c;
+    in.grad = grad_c;
+    in.logprob = logprob_c;
     hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, mask,
                        static_cast<const float*>(nullptr), hidden_dim, static_cast<uint16_t*>(d_hidden));
-    enqueue_bwd(p.bwd, ws_bwd, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, d_weight, s);
+    enqueue_bwd(p.bwd, ws_bwd, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, d_weight, ecache,
+                cache, s);
     return oi_launch_status();
 }
 
@@ -1287,7 +1492,7 @@ extern "C" int oi_gemm_bf16_tn(const void* A, int64_t lda, int64_t M, const void
     const Operand b = {static_cast<const uint16_t*>(B), ldb, 0, N, K};
     hipLaunchKernelGGL((gemm_store_kernel<false, false>), dim3(grid_for_tiles((M + BM - 1) / BM, (N + BN - 1) / BN)),
                        dim3(NTHREADS), 0, static_cast<hipStream_t>(stream), a, M, b, N, K, mode, out_f32,
-                       static_cast<uint16_t*>(out_bf16), ldo, M, DynRows{nullptr, 0, nullptr}, static_cast<uint32_t*>(nullptr));
+                       static_cast<uint16_t*>(out_bf16), ldo, M, DynRows{nullptr, 0, nullptr, nullptr, nullptr}, static_cast<uint32_t*>(nullptr));
     return oi_launch_status();
 }
 
@@ -1311,7 +1516,7 @@ extern "C" int oi_gemm_bf16_layouts(const void* A, int64_t lda, int a_k_major, c
     hipStream_t s = static_cast<hipStream_t>(stream);
     uint16_t* o16 = static_cast<uint16_t*>(out_bf16);
     uint32_t* no_queue = nullptr;
-    const DynRows fixed = {nullptr, 0, nullptr};
+    const DynRows fixed = {nullptr, 0, nullptr, nullptr, nullptr};
     if (a_k_major && b_k_major)
         hipLaunchKernelGGL((gemm_store_kernel<true, true>), grid, dim3(NTHREADS), 0, s, a, M, b, N, K, mode, out_f32, o16,
                            ldo, M, fixed, no_queue);

@@ -559,6 +559,7 @@ def grpo_loss_on_hidden(
     loss_denominator: float | None = None,
     axis: int | None = None,
     dp_scale: float = 1.0,
+    logit_cache_chunks: int = 0,
 ) -> tuple[torch.Tensor, dict[str, torch.Tensor], torch.Tensor, torch.Tensor]:
     """GRPO loss straight from final hidden states; returns ``(loss, stats, logprobs, entropy)``.
 
@@ -615,15 +616,20 @@ def grpo_loss_on_hidden(
     stats = torch.empty(len(GRPO_STAT_NAMES), dtype=torch.float32, device=dev)
     d_hidden = torch.empty_like(hid)
     d_weight = torch.empty_like(w) if weight.requires_grad else None
-    ws_bytes = _lib.load().oi_lmhead_grpo_workspace_bytes(rows, cols, h, v)
+    lib = _lib.load()
+    cache_chunks = max(0, int(logit_cache_chunks))
+    cache = None
+    if cache_chunks:
+        cache = torch.empty(lib.oi_lmhead_cache_bytes(rows * cols, v, cache_chunks), dtype=torch.uint8, device=dev)
+    ws_bytes = lib.oi_lmhead_grpo_workspace_bytes(rows, cols, h, v, int(cache is not None))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     _lib.call(
         "oi_lmhead_grpo_fwd_bwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), m.data_ptr(), _lib.ptr(old_c),
         _lib.ptr(ref_c), adv_c.data_ptr(), _lib.ptr(rho_c), rows, cols, h, v, inv_t, _loss_fn_tag(config), lo, hi,
         int(config.kl_estimator), float(config.beta), 0 if axis is None else 1,
         0.0 if loss_denominator is None else float(loss_denominator), float(dp_scale), logprob.data_ptr(),
-        entropy.data_ptr(), stats.data_ptr(), d_hidden.data_ptr(), _lib.ptr(d_weight), ws.data_ptr(), ws_bytes,
-        _lib.stream_of(hid),
+        entropy.data_ptr(), stats.data_ptr(), d_hidden.data_ptr(), _lib.ptr(d_weight), _lib.ptr(cache), cache_chunks,
+        ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
     )  # fmt: skip
     loss = _AttachHeadGrads.apply(stats[0], hidden, weight, d_hidden.reshape(hidden.shape), d_weight)
     return loss, _StatsView(stats), logprob, entropy

@@ -19,7 +19,8 @@ from . import _lib
 
 class _FusedLMHead(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, labels, mask, inv_temperature, want_entropy, compact_backward=False):
+    def forward(ctx, hidden, weight, labels, mask, inv_temperature, want_entropy, compact_backward=False,
+                cache_chunks=0):
         dev = _lib.require_gpu(hidden, weight, labels, mask)
         if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
             raise ValueError("fused lm_head expects bf16 hidden states and weight")
@@ -41,44 +42,56 @@ class _FusedLMHead(torch.autograd.Function):
         logprob = torch.empty(n, dtype=torch.float32, device=dev)
         entropy = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
         lse = torch.empty(n, dtype=torch.float32, device=dev)
+        # the cache of exponentials only pays for itself when a backward pass follows
+        cache_chunks = int(cache_chunks) if (ctx.needs_input_grad[0] or ctx.needs_input_grad[1]) else 0
+        if cache_chunks and compact_backward:
+            raise ValueError("compact_backward re-selects rows in the backward pass; it cannot be combined with a cache")
+        cache = None
         if n > 0:
-            ws_bytes = _lib.load().oi_lmhead_fwd_workspace_bytes(n, h, v, int(m is not None))
+            lib = _lib.load()
+            if cache_chunks > 0:
+                cache = torch.empty(lib.oi_lmhead_cache_bytes(n, v, cache_chunks), dtype=torch.uint8, device=dev)
+            ws_bytes = lib.oi_lmhead_fwd_workspace_bytes(n, h, v, int(m is not None))
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
             _lib.call(
                 "oi_lmhead_logp_fwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), _lib.ptr(m), n, h, v,
-                inv_temperature, logprob.data_ptr(), _lib.ptr(entropy), lse.data_ptr(), ws.data_ptr(), ws_bytes,
-                _lib.stream_of(hid),
+                inv_temperature, logprob.data_ptr(), _lib.ptr(entropy), lse.data_ptr(), _lib.ptr(cache),
+                cache_chunks if cache is not None else 0, ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
             )  # fmt: skip
-        ctx.save_for_backward(hid, w, lab, lse, m)
+        ctx.save_for_backward(hid, w, lab, lse, m, cache, logprob if cache is not None else None)
         ctx.inv_temperature = inv_temperature
         ctx.compact_backward = bool(compact_backward)
+        ctx.cache_chunks = cache_chunks if cache is not None else 0
         if want_entropy:
             ctx.mark_non_differentiable(entropy)
         return logprob, entropy
 
     @staticmethod
     def backward(ctx, grad_logprob, _grad_entropy):
-        hid, w, lab, lse, m = ctx.saved_tensors
+        hid, w, lab, lse, m, cache, logprob = ctx.saved_tensors
         n, h = hid.shape
         v = w.shape[0]
         need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if grad_logprob is None or not (need_h or need_w):
-            return None, None, None, None, None, None, None
+            return None, None, None, None, None, None, None, None
         g = _lib.f32c(grad_logprob)
         d_hidden = torch.empty_like(hid)
         d_weight = torch.empty_like(w) if need_w else None
         if n > 0:
             selecting = m is not None or ctx.compact_backward
-            ws_bytes = _lib.load().oi_lmhead_bwd_workspace_bytes(n, h, v, int(need_w), int(selecting))
+            ws_bytes = _lib.load().oi_lmhead_bwd_workspace_bytes(
+                n, h, v, int(need_w), int(selecting), int(ctx.cache_chunks > 0)
+            )
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=hid.device)
             _lib.call(
                 "oi_lmhead_logp_bwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), lse.data_ptr(), g.data_ptr(),
-                _lib.ptr(m), int(ctx.compact_backward), n, h, v, ctx.inv_temperature, d_hidden.data_ptr(),
-                _lib.ptr(d_weight), ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
+                _lib.ptr(m), int(ctx.compact_backward), n, h, v, ctx.inv_temperature, _lib.ptr(logprob),
+                _lib.ptr(cache), ctx.cache_chunks, d_hidden.data_ptr(), _lib.ptr(d_weight), ws.data_ptr(), ws_bytes,
+                _lib.stream_of(hid),
             )  # fmt: skip
         elif d_weight is not None:
             d_weight.zero_()
-        return (d_hidden if need_h else None), d_weight, None, None, None, None, None
+        return (d_hidden if need_h else None), d_weight, None, None, None, None, None, None
 
 
 def fused_lm_head_logprobs(
@@ -89,6 +102,7 @@ def fused_lm_head_logprobs(
     mask: torch.Tensor | None = None,
     return_entropy: bool = False,
     compact_backward: bool = False,
+    logit_cache_chunks: int = 0,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """``log_softmax(hidden @ weight.T / temperature)[labels]`` (+ entropy) per token, fp32.
 
@@ -102,6 +116,12 @@ def fused_lm_head_logprobs(
     gradient, as in the reference.  ``compact_backward=True`` additionally leaves rows whose
     upstream gradient is exactly zero (zero-advantage completions, clipped ratios without a KL
     term) out of the backward products; it changes no result.
+
+    ``logit_cache_chunks`` (default 0: nothing of size ``[tokens, vocab]`` ever exists and the
+    backward recomputes every vocabulary chunk) trades memory for that recomputation: the forward
+    keeps ``2^(logit / temperature * log2 e)`` in bf16 for the first so many chunks of 32768 vocabulary
+    columns (2 bytes per cached logit, held until the backward pass) and the backward multiplies
+    the cache directly.  With every chunk cached a quarter of the step's matrix work goes away.
     """
     lead = hidden.shape[:-1]
     hid2 = hidden.reshape(-1, hidden.shape[-1])
@@ -111,7 +131,7 @@ def fused_lm_head_logprobs(
         raise ValueError(f"temperature must be positive, got {temperature}")
     if mask is not None and tuple(mask.shape) != tuple(lead):
         raise ValueError(f"mask {tuple(mask.shape)} does not match the rows of hidden {tuple(lead)}")
-    lp, ent = _FusedLMHead.apply(hid2, weight, lab1, mask, inv_t, return_entropy, compact_backward)
+    lp, ent = _FusedLMHead.apply(hid2, weight, lab1, mask, inv_t, return_entropy, compact_backward, logit_cache_chunks)
     return lp.reshape(lead), (ent.reshape(lead) if ent is not None else None)
 
 

@@ -132,10 +132,13 @@ def _check_fused_head(hidden, weight, labels_eff, mask, g_cpu, lp, ent, d_hidden
     assert (per_v <= 2 * REL).all(), per_v.max().item()
 
 
-def test_c3_llama8b_head_grpo_full_shape():
+@pytest.mark.parametrize("cache_chunks", [0, 4, 1])
+def test_c3_llama8b_head_grpo_full_shape(cache_chunks):
     """hidden bf16 [32768, 4096], W bf16 [128256, 4096], 70 % response rows: fused lm_head + logprob +
-    entropy + GRPO loss, forward and backward to dHidden and dW, as the benchmark's default step."""
-    print("case c3 N=32768 H=4096 V=128256", flush=True)
+    entropy + GRPO loss, forward and backward to dHidden and dW, as the benchmark's default step
+    (cache_chunks = 0: every chunk recomputed) and with the optional cache of exponentials for all
+    four vocabulary chunks or for the first one only."""
+    print(f"case c3 N=32768 H=4096 V=128256 cached chunks={cache_chunks}", flush=True)
     torch.manual_seed(0)
     n, h, v = 32768, 4096, 128256
     hidden = torch.randn(n, h, device=DEV).bfloat16().requires_grad_(True)
@@ -149,10 +152,13 @@ def test_c3_llama8b_head_grpo_full_shape():
     old = lp0 + 0.05 * torch.randn(n, device=DEV)
     ref = lp0 + 0.1 * torch.randn(n, device=DEV)
 
-    lp, ent = lm_head.fused_lm_head_logprobs(hidden, weight, labels, mask=mask, return_entropy=True)
+    lp, ent = lm_head.fused_lm_head_logprobs(
+        hidden, weight, labels, mask=mask, return_entropy=True, logit_cache_chunks=cache_chunks
+    )
     loss, stats = grpo_utils.grpo_loss_fused(lp[None], old[None], ref[None], adv[None], mask[None], cfg, entropy=ent[None])
     loss.backward()
     torch.cuda.synchronize()
+    assert torch.equal(lp.detach(), lp0)  # the cache changes nothing in the forward results
 
     # loss and upstream gradient of every token from the oracle's loss chain on the kernel's logprobs
     lp_leaf = lp.detach().cpu().requires_grad_(True)
@@ -215,11 +221,12 @@ def test_c4_packed_olmo2_head_grpo_full_shape():
     _check_fused_head(hidden, weight, shifted.view(-1), mask, lp_leaf.grad, lp, ent, hidden.grad, weight.grad, seed=4)
 
 
-def test_c5_llama70b_head_dpo_full_shape():
+@pytest.mark.parametrize("cache_chunks", [0, 4])
+def test_c5_llama70b_head_dpo_full_shape(cache_chunks):
     """8 chosen / rejected pairs of 2048 tokens with the prompt (128..1024 tokens) masked out, hidden
     bf16 [32768, 8192] (128 k-tiles), W bf16 [128256, 8192] frozen: per-sequence sums, sigmoid DPO loss
-    (beta 0.1), backward to dHidden only."""
-    print("case c5 N=32768 H=8192 V=128256", flush=True)
+    (beta 0.1), backward to dHidden only; with and without the cache of exponentials."""
+    print(f"case c5 N=32768 H=8192 V=128256 cached chunks={cache_chunks}", flush=True)
     torch.manual_seed(0)
     n, h, v, per = 32768, 8192, 128256, 2048
     seqs = n // per
@@ -236,7 +243,7 @@ def test_c5_llama70b_head_dpo_full_shape():
     ref_c = torch.randn(seqs // 2, device=DEV) * 50 - 400
     ref_r = torch.randn(seqs // 2, device=DEV) * 50 - 400
 
-    lp, _ = lm_head.fused_lm_head_logprobs(hidden, weight, shifted.view(-1), mask=mask)
+    lp, _ = lm_head.fused_lm_head_logprobs(hidden, weight, shifted.view(-1), mask=mask, logit_cache_chunks=cache_chunks)
     logps = padding_free_collator.get_batch_logps(lp.view(1, -1), labels, cu)
     bs = logps.shape[0] // 2
     losses, cr, rr = dpo_utils.dpo_loss(logps[:bs], logps[bs:], ref_c, ref_r, beta=0.1)

@@ -290,3 +290,90 @@ def test_row_selection_with_compact_backward_and_mask():
     assert ((dh.grad.float().cpu() - rh.grad).norm() / rh.grad.norm()).item() <= 2e-2
     assert ((dw.grad.float().cpu() - rw.grad).norm() / rw.grad.norm()).item() <= 2e-2
     assert (dw.grad.float().cpu() - rw.grad).abs().max().item() <= TOL + rw.grad.abs().max().item() * 2**-7
+
+
+@pytest.mark.parametrize(
+    "n,h,v,chunks",
+    [
+        (300, 128, 1000, 1),  # one chunk, all of it cached; ragged tokens and vocabulary
+        (700, 256, 5000, 1),
+        (260, 64, 70000, 1),  # three chunks: the first from the cache, the others recomputed
+        (260, 64, 70000, 2),
+        (260, 64, 70000, 3),  # everything from the cache: no recomputation at all
+        (130, 128, 100000, 9),  # more chunks asked for than there are
+        (2, 64, 7, 1),
+    ],
+)
+@pytest.mark.parametrize("want_dw", [True, False])
+@pytest.mark.parametrize("masked", [False, True])
+def test_backward_from_cache_of_exponentials(n, h, v, chunks, want_dw, masked):
+    """The optional cache of 2^(logit) written by the forward replaces the recomputation of the cached
+    vocabulary chunks in the backward: same gradients as the oracle (and as the recomputing path, up to
+    bf16 rounding), forward results bit-identical with and without the cache."""
+    print(f"case N={n} H={h} V={v} cached chunks={chunks} dW={want_dw} masked={masked}", flush=True)
+    hidden, weight, labels = _case(n, h, v, seed=31, w_scale=3.0 / math.sqrt(h))
+    g = torch.Generator().manual_seed(32)
+    upstream = torch.randn(n, generator=g)
+    upstream[::5] = 0.0
+    mask = (torch.rand(n, generator=g) < 0.7) if masked else torch.ones(n, dtype=torch.bool)
+    labels[0], labels[n - 1] = v - 1, 0
+    rh = hidden.float().requires_grad_(True)
+    rw = weight.float().requires_grad_(True)
+    lp_o, _ = o_lm.lm_head_logprobs(rh, rw, labels, 0.9)
+    (lp_o * mask).backward(upstream)
+
+    def run(cache_chunks):
+        dh = hidden.to(DEV).requires_grad_(True)
+        dw = weight.to(DEV).requires_grad_(want_dw)
+        lp, ent = lm_head.fused_lm_head_logprobs(
+            dh, dw, labels.to(DEV), 0.9, mask=mask.to(DEV) if masked else None, return_entropy=True,
+            logit_cache_chunks=cache_chunks,
+        )  # fmt: skip
+        lp.backward(upstream.to(DEV))
+        return lp.detach(), ent, dh.grad, (dw.grad if want_dw else None)
+
+    lp_c, ent_c, dh_c, dw_c = run(chunks)
+    lp_r, ent_r, dh_r, dw_r = run(0)
+    assert torch.equal(lp_c, lp_r) and torch.equal(ent_c, ent_r)
+    assert ((lp_c.cpu() - lp_o.detach()) * mask).abs().max().item() <= TOL
+    tol_h = TOL + rh.grad.abs().max().item() * 2**-7
+    assert (dh_c.float().cpu() - rh.grad).abs().max().item() <= tol_h
+    assert ((dh_c.float().cpu() - rh.grad).norm() / rh.grad.norm()).item() <= 2e-2
+    assert (dh_c.cpu()[~mask] == 0).all() and (dh_c.cpu()[::5] == 0).all()
+    assert (dh_c.float() - dh_r.float()).abs().max().item() <= 2**-6 * dh_r.float().abs().max().item()
+    if n >= 130:  # another order of roundings: the two routes are not the same code
+        assert not torch.equal(dh_c, dh_r)
+    if want_dw:
+        tol_w = TOL + rw.grad.abs().max().item() * 2**-7
+        assert (dw_c.float().cpu() - rw.grad).abs().max().item() <= tol_w
+        assert ((dw_c.float().cpu() - rw.grad).norm() / rw.grad.norm()).item() <= 2e-2
+
+
+def test_cache_of_exponentials_confident_tokens_and_no_grad():
+    """Tokens whose label carries almost all of the probability (1 - p around 1e-2): the label's entry
+    of the cache is rebuilt from the fp32 logprob, so the gradient stays accurate where the bf16 entry
+    (relative error 2^-9 of p, i.e. tens of percent of 1 - p) would have cancelled.  Under no_grad no
+    cache is made at all."""
+    torch.manual_seed(41)
+    n, h, v = 256, 64, 2000
+    hidden = torch.randn(n, h).bfloat16()
+    weight = (torch.randn(v, h) * 0.05).bfloat16()
+    labels = torch.randint(0, v, (n,))
+    labels[:64] = torch.arange(64)  # distinct rows of W for the confident tokens
+    weight[:64] = (hidden[:64].float() * 0.19).bfloat16()  # logit of the label ~ 0.19 |h|^2 ~ 12
+    rh = hidden.float().requires_grad_(True)
+    lp_o, _ = o_lm.lm_head_logprobs(rh, weight.float(), labels, 1.0)
+    assert lp_o[:64].median().item() > -0.05  # p(label) > 0.95 on most of these rows
+    up = torch.randn(n)
+    lp_o.backward(up)
+    dh = hidden.to(DEV).requires_grad_(True)
+    lp, _ = lm_head.fused_lm_head_logprobs(dh, weight.to(DEV), labels.to(DEV), logit_cache_chunks=1)
+    lp.backward(up.to(DEV))
+    assert (lp.detach().cpu() - lp_o.detach()).abs().max().item() <= TOL
+    rel_rows = (dh.grad.float().cpu() - rh.grad).norm(dim=1) / rh.grad.norm(dim=1).clamp(min=1e-12)
+    assert rel_rows.max().item() <= 3e-2, rel_rows.max().item()
+    with torch.no_grad():
+        lp2, _ = lm_head.fused_lm_head_logprobs(dh, weight.to(DEV), labels.to(DEV), logit_cache_chunks=1)
+    assert torch.equal(lp2, lp.detach())
+    with pytest.raises(ValueError, match="compact_backward"):
+        lm_head.fused_lm_head_logprobs(dh, weight.to(DEV), labels.to(DEV), compact_backward=True, logit_cache_chunks=1)

@@ -447,3 +447,17 @@ def test_grpo_loss_on_hidden_whole_step(loss_fn, axis, denominator, with_old, wa
             rho_weights=d(rho), loss_denominator=denominator, axis=axis, dp_scale=2.0,
         )  # fmt: skip
     assert not loss4.requires_grad and loss4.item() == loss.item() and torch.equal(lp4, lp)
+    # the cache of exponentials (one chunk of two, then both): same forward bits, gradients within bf16 rounding
+    for chunks in (1, 2):
+        dh5 = d(hidden).requires_grad_(True)
+        dw5 = d(weight).requires_grad_(want_dw)
+        loss5, _, lp5, _ = grpo_utils.grpo_loss_on_hidden(
+            dh5, dw5, d(labels), d(old) if with_old else None, d(ref), d(adv), d(mask), cfg, temperature=temperature,
+            rho_weights=d(rho), loss_denominator=denominator, axis=axis, dp_scale=2.0, logit_cache_chunks=chunks,
+        )  # fmt: skip
+        loss5.backward()
+        assert loss5.item() == loss.item() and torch.equal(lp5, lp)
+        assert ((dh5.grad.float().cpu() - exp_dh).norm() / exp_dh.norm()).item() <= 2e-2
+        assert (dh5.grad.cpu()[~mask] == 0).all()
+        if want_dw:
+            assert ((dw5.grad.float().cpu() - exp_dw).norm() / exp_dw.norm()).item() <= 2e-2
