@@ -379,14 +379,15 @@ size_t oi_lmhead_cache_bytes(int64_t n_tokens, int64_t vocab, int64_t cache_chun
  * Vocabulary is processed in chunks of 32768 columns; only one chunk of dZ (bf16, token-major)
  * lives in the workspace at a time, next to the fp32 accumulator of d_hidden.  Both products
  * read weight, hidden and dZ where they lie (no transposed copies), so the workspace is the same
- * with and without d_weight.  row_mask as in the forward (rows left out get a zero d_hidden row
+ * with and without d_weight (cached chunks are multiplied as one chunk; with every chunk cached
+ * neither the dZ chunk nor the fp32 accumulator is part of the workspace).  row_mask as in the forward (rows left out get a zero d_hidden row
  * and add nothing to d_weight); skip_zero_grad_rows != 0 also leaves out rows whose grad_logprob is
  * exactly 0, which changes no result (not together with a cache, whose rows are the forward's).
  * d_hidden and d_weight must be 4-byte aligned.  logprob (the forward's output) is read only with a
  * cache.
  */
 size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int want_d_weight,
-                                     int with_row_selection, int with_cache);
+                                     int with_row_selection, int64_t cache_chunks);
 int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
                        const float* grad_logprob, const uint8_t* row_mask, int skip_zero_grad_rows, int64_t n_tokens,
                        int64_t hidden_dim, int64_t vocab, float inv_temperature, const float* logprob,
@@ -412,7 +413,8 @@ int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* la
  * exp_cache / cache_chunks: the optional cache of exponentials described at oi_lmhead_cache_bytes
  * (scratch of this one call here; NULL / 0 = recompute every chunk).
  */
-size_t oi_lmhead_grpo_workspace_bytes(int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab, int with_cache);
+size_t oi_lmhead_grpo_workspace_bytes(int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab,
+                                      int64_t cache_chunks);
 int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, const int64_t* labels, const uint8_t* mask,
                            const float* old_logprobs, const float* ref_logprobs, const float* advantages,
                            const float* rho_weights, int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab,

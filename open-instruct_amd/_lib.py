@@ -62,12 +62,12 @@ SIGNATURES: dict[str, tuple] = {
     "oi_lmhead_fwd_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I]),
     "oi_lmhead_logp_fwd": (_I, [_P, _P, _P, _P, _I64, _I64, _I64, _F, _P, _P, _P, _P, _I64, _P, _SZ, _P]),
     "oi_lmhead_cache_bytes": (_SZ, [_I64, _I64, _I64]),
-    "oi_lmhead_bwd_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I, _I, _I]),
+    "oi_lmhead_bwd_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I, _I, _I64]),
     "oi_lmhead_logp_bwd": (
         _I,
         [_P, _P, _P, _P, _P, _P, _I, _I64, _I64, _I64, _F, _P, _P, _I64, _P, _P, _P, _SZ, _P],
     ),
-    "oi_lmhead_grpo_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I64, _I]),
+    "oi_lmhead_grpo_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I64, _I64]),
     "oi_lmhead_grpo_fwd_bwd": (
         _I,
         [_P] * 8 + [_I64, _I64, _I64, _I64, _F, _I, _F, _F, _I, _F, _I, _F, _F] + [_P] * 6 + [_I64, _P, _SZ, _P],

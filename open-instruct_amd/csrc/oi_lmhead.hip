@@ -1116,15 +1116,19 @@ struct BwdPlan {
     size_t off_dz, off_dh32, off_queues, off_scale_a, off_scale_b, off_scaled_hidden, total;
     SelectionPlan sel;
 };
-BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_selection, bool with_cache = false) {
+BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_selection, int64_t cache_chunks = 0) {
     BwdPlan p;
     p.n_pad = round_up(n_tokens, 256);
     p.v_pad = round_up(vocab, 256);
     p.chunk = p.v_pad < BWD_VOCAB_CHUNK ? p.v_pad : BWD_VOCAB_CHUNK;
     p.n_chunks = (p.v_pad + p.chunk - 1) / p.chunk;
+    const bool with_cache = cache_chunks > 0;
+    // with every chunk in the cache nothing is recomputed and d_hidden is stored once: neither the
+    // dZ chunk nor the fp32 accumulator is needed
+    const bool all_cached = cache_chunks >= p.n_chunks;
     Carver cv;
-    p.off_dz = cv.take((size_t)p.n_pad * p.chunk * 2);
-    p.off_dh32 = cv.take((size_t)n_tokens * hdim * 4);
+    p.off_dz = cv.take(all_cached ? 0 : (size_t)p.n_pad * p.chunk * 2);
+    p.off_dh32 = cv.take(all_cached ? 0 : (size_t)n_tokens * hdim * 4);
     // one set of work-queue counters per tile-kernel launch (three per vocabulary chunk)
     p.off_queues = cv.take((size_t)(3 * p.n_chunks) * QUEUE_WORDS * sizeof(uint32_t));
     if (with_selection) p.sel = plan_selection(cv, p.n_pad, hdim, true);
@@ -1247,9 +1251,13 @@ void enqueue_bwd(const BwdPlan& p, char* ws, const RowInputs& in, const void* we
             hipLaunchKernelGGL(scale_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, in.hidden, scale_a, scale_b,
                                in.n_dev, n_tokens, hidden_dim, scaled_hidden);
     }
-    for (int64_t ci = 0; ci < p.n_chunks; ++ci) {
-        const int64_t v_begin = ci * p.chunk;
-        const int64_t cols = (p.v_pad - v_begin) < p.chunk ? (p.v_pad - v_begin) : p.chunk;  // multiple of 256
+    // The cached chunks need no dZ buffer between the recomputation and the products, so they are
+    // multiplied as ONE chunk (fewer, longer tiles; d_hidden is stored once instead of accumulated).
+    for (int64_t ci = cache.chunks > 0 ? cache.chunks - 1 : 0; ci < p.n_chunks; ++ci) {
+        const bool merged = cache.chunks > 0 && ci == cache.chunks - 1;
+        const int64_t v_begin = merged ? 0 : ci * p.chunk;
+        const int64_t v_end = (ci + 1) * p.chunk < p.v_pad ? (ci + 1) * p.chunk : p.v_pad;
+        const int64_t cols = v_end - v_begin;                                                // multiple of 256
         const int64_t valid = vocab - v_begin < cols ? vocab - v_begin : cols;               // real rows of W
         const bool cached = ci < cache.chunks;
         uint32_t* q = queues + ci * 3 * QUEUE_WORDS;
@@ -1260,7 +1268,7 @@ void enqueue_bwd(const BwdPlan& p, char* ws, const RowInputs& in, const void* we
         // the A operand of both products: this chunk's dZ, or this chunk's columns of the cache
         const uint16_t* a_ptr = cached ? ecache + v_begin : dz;
         const int64_t a_ld = cached ? cache.ld : cols;
-        const bool first = ci == 0, last = ci == p.n_chunks - 1;
+        const bool first = v_begin == 0, last = ci == p.n_chunks - 1;
         const int mode = last ? (first ? 2 : 3) : (first ? 0 : 1);
         {
             const Operand a = {a_ptr, a_ld, 0, p.n_pad, cols};
@@ -1289,11 +1297,11 @@ struct StepPlan {
     BwdPlan bwd;
     size_t off_fwd, off_bwd, off_stats, off_lse, off_grad, off_denoms, total;
 };
-StepPlan plan_step(int64_t rows, int64_t cols, int64_t hdim, int64_t vocab, bool with_cache) {
+StepPlan plan_step(int64_t rows, int64_t cols, int64_t hdim, int64_t vocab, int64_t cache_chunks) {
     StepPlan p;
     const int64_t n = rows * cols;
     p.fwd = plan_fwd(n, hdim, vocab, false);
-    p.bwd = plan_bwd(n, hdim, vocab, true, with_cache);
+    p.bwd = plan_bwd(n, hdim, vocab, true, cache_chunks);
     Carver cv;
     p.off_fwd = cv.take(p.fwd.total);
     p.off_bwd = cv.take(p.bwd.total);
@@ -1354,10 +1362,10 @@ extern "C" int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const 
 }
 
 extern "C" size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
-                                                int want_d_weight, int with_row_selection, int with_cache) {
+                                                int want_d_weight, int with_row_selection, int64_t cache_chunks) {
     if (n_tokens <= 0 || hidden_dim <= 0 || vocab <= 0) return 0;
     (void)want_d_weight;
-    return plan_bwd(n_tokens, hidden_dim, vocab, with_row_selection != 0, with_cache != 0).total;
+    return plan_bwd(n_tokens, hidden_dim, vocab, with_row_selection != 0, cache_chunks).total;
 }
 
 extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
@@ -1378,7 +1386,7 @@ extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const 
     OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 4) || !oi_aligned(d_weight, 4), OI_EALIGN);
     const bool selecting = row_mask != nullptr || skip_zero_grad_rows != 0;
     const CachePlan cache = plan_cache(n_tokens, vocab, cache_chunks);
-    const BwdPlan p = plan_bwd(n_tokens, hidden_dim, vocab, selecting, cache.chunks > 0);
+    const BwdPlan p = plan_bwd(n_tokens, hidden_dim, vocab, selecting, cache.chunks);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     hipStream_t s = static_cast<hipStream_t>(stream);
     char* ws = static_cast<char*>(workspace);
@@ -1403,9 +1411,9 @@ extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const 
 }
 
 extern "C" size_t oi_lmhead_grpo_workspace_bytes(int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab,
-                                                 int with_cache) {
+                                                 int64_t cache_chunks) {
     if (rows <= 0 || cols <= 0 || hidden_dim <= 0 || vocab <= 0) return 0;
-    return plan_step(rows, cols, hidden_dim, vocab, with_cache != 0).total;
+    return plan_step(rows, cols, hidden_dim, vocab, cache_chunks).total;
 }
 
 extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, const int64_t* labels,
@@ -1425,7 +1433,7 @@ extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, co
     OI_RETURN_IF(!mask || !advantages || !logprob || !out_stats || !d_hidden || !workspace, OI_ENULL);
     OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 4) || !oi_aligned(d_weight, 4), OI_EALIGN);
     const CachePlan cache = plan_cache(n_tokens, vocab, cache_chunks);
-    const StepPlan p = plan_step(rows, cols, hidden_dim, vocab, cache.chunks > 0);
+    const StepPlan p = plan_step(rows, cols, hidden_dim, vocab, cache.chunks);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     hipStream_t s = static_cast<hipStream_t>(stream);
     char* ws = static_cast<char*>(workspace);

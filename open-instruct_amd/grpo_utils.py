@@ -621,7 +621,7 @@ def grpo_loss_on_hidden(
     cache = None
     if cache_chunks:
         cache = torch.empty(lib.oi_lmhead_cache_bytes(rows * cols, v, cache_chunks), dtype=torch.uint8, device=dev)
-    ws_bytes = lib.oi_lmhead_grpo_workspace_bytes(rows, cols, h, v, int(cache is not None))
+    ws_bytes = lib.oi_lmhead_grpo_workspace_bytes(rows, cols, h, v, cache_chunks if cache is not None else 0)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     _lib.call(
         "oi_lmhead_grpo_fwd_bwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), m.data_ptr(), _lib.ptr(old_c),

@@ -80,7 +80,7 @@ class _FusedLMHead(torch.autograd.Function):
         if n > 0:
             selecting = m is not None or ctx.compact_backward
             ws_bytes = _lib.load().oi_lmhead_bwd_workspace_bytes(
-                n, h, v, int(need_w), int(selecting), int(ctx.cache_chunks > 0)
+                n, h, v, int(need_w), int(selecting), ctx.cache_chunks
             )
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=hid.device)
             _lib.call(

@@ -99,7 +99,9 @@ def test_rejected_arguments_return_codes_without_launching():
     # a row selection adds the row index, the count, the gathered hidden rows / labels / lse / gradient
     assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1, 1, 0) == plain + 256 * 4 + 256 + 256 * 64 * 2 + 256 * 8 + 3 * 256 * 4
     # a cache of exponentials adds the two per-token factors and the scaled hidden rows
-    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1, 0, 1) == plain + 2 * 256 * 4 + 256 * 64 * 2
+    # (every chunk cached: no dZ chunk, no fp32 accumulator)
+    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1, 0, 1) == 256 + 2 * 256 * 4 + 256 * 64 * 2
+    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 70000, 1, 0, 1) == 256 * 32768 * 2 + 256 * 64 * 4 + 512 + 2 * 256 * 4 + 256 * 64 * 2
     # 2 bytes per cached logit, whole chunks of 32768 columns (or the padded vocabulary)
     assert lib.oi_lmhead_cache_bytes(300, 1000, 1) == 512 * 1024 * 2
     assert lib.oi_lmhead_cache_bytes(256, 70000, 1) == 256 * 32768 * 2 and lib.oi_lmhead_cache_bytes(256, 70000, 9) == 256 * 70144 * 2
