@@ -143,6 +143,7 @@ def fused_linear_cross_entropy(
     shift_labels: torch.Tensor | None = None,
     num_items_in_batch: torch.Tensor | int | float | None = None,
     ignore_index: int = -100,
+    logit_cache_chunks: int = 0,
 ) -> torch.Tensor:
     """Causal-LM cross-entropy of ``hidden @ weight.T`` against next-token labels, scalar fp32.
 
@@ -152,6 +153,7 @@ def fused_linear_cross_entropy(
     label equals ``ignore_index`` are never multiplied.  The result is the mean over kept tokens,
     or ``sum / num_items_in_batch`` when that count is given (gradient accumulation over several
     micro-batches).  Differentiable with respect to ``hidden`` and ``weight``.
+    ``logit_cache_chunks`` as for :func:`fused_lm_head_logprobs`.
     """
     if (labels is None) == (shift_labels is None):
         raise ValueError("pass exactly one of labels / shift_labels")
@@ -161,7 +163,7 @@ def fused_linear_cross_entropy(
     if shift_labels.shape != hidden.shape[:-1]:
         raise ValueError(f"labels {tuple(shift_labels.shape)} do not match hidden {tuple(hidden.shape)}")
     keep = shift_labels != ignore_index
-    logps, _ = fused_lm_head_logprobs(hidden, weight, shift_labels, mask=keep)
+    logps, _ = fused_lm_head_logprobs(hidden, weight, shift_labels, mask=keep, logit_cache_chunks=logit_cache_chunks)
     total = -logps.sum()
     if num_items_in_batch is None:
         return total / keep.sum().clamp(min=1)
