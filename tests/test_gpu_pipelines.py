@@ -461,3 +461,58 @@ def test_grpo_loss_on_hidden_whole_step(loss_fn, axis, denominator, with_old, wa
         assert (dh5.grad.cpu()[~mask] == 0).all()
         if want_dw:
             assert ((dw5.grad.float().cpu() - exp_dw).norm() / exp_dw.norm()).item() <= 2e-2
+
+
+def test_entry_points_replay_from_a_hip_graph():
+    """The C entry points enqueue kernels only (no allocation, no synchronisation, no memset nodes), so a
+    caller may capture them in a HIP graph.  Two launch-bound cases: logprob + entropy + masked means on
+    small logits, and the whole GRPO step on hidden states in one call.  Every replay is compared with the
+    eager result on inputs that eager work changed between the replays."""
+    torch.manual_seed(51)
+    logits = (torch.randn(4, 128, 8000, device=DEV) * 2.0)
+    ids = torch.randint(0, 8000, (4, 128), device=DEV)
+    mask = torch.rand(4, 128, device=DEV) > 0.3
+    b, t, h, v = 2, 140, 128, 3000
+    hidden = torch.randn(b, t, h, device=DEV).bfloat16().requires_grad_(True)
+    weight = (torch.randn(v, h, device=DEV) * 0.2).bfloat16().requires_grad_(True)
+    labels = torch.randint(0, v, (b, t), device=DEV)
+    rmask = torch.rand(b, t, device=DEV) < 0.7
+    adv = torch.randn(b, t, device=DEV)
+    cfg = make_grpo_config(loss_fn="dapo", beta=0.05, kl_estimator=2, clip_higher=0.28)
+
+    def small_step():
+        lp, ent = model_utils.logprob_and_entropy(logits, ids)
+        from open_instruct_amd import rl_utils
+
+        return rl_utils.masked_mean(lp, mask) + rl_utils.masked_mean(ent, mask)
+
+    def grpo_step():
+        hidden.grad = None
+        weight.grad = None
+        loss, _, lp, _ = grpo_utils.grpo_loss_on_hidden(hidden, weight, labels, None, None, adv, rmask, cfg)
+        loss.backward()
+        return loss.detach(), hidden.grad, weight.grad
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            small_step()
+            grpo_step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_small = small_step()
+        g_loss, g_dh, g_dw = grpo_step()
+    for i in range(4):
+        with torch.no_grad():  # eager work between the replays changes the inputs in place
+            logits.mul_(1.02)
+            hidden.mul_(0.97)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (g_small.clone(), g_loss.clone(), g_dh.clone(), g_dw.clone())
+        e_small = small_step()
+        e_loss, e_dh, e_dw = grpo_step()
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], e_small), i
+        assert torch.equal(got[1], e_loss) and torch.equal(got[2], e_dh) and torch.equal(got[3], e_dw), i
