@@ -45,9 +45,9 @@ MEASURED_TRAFFIC_BYTES = {
     "c3": 43.14e9 + 0.19e9,
     "c4": 40.63e9 + 0.21e9,
     "c5": 88.61e9 + 0.19e9,
-    # lsg_grpo_fused_kernel: reads beyond L2 (the second read of a row is served by the LDS and the caches; this
-    # counter cannot tell the memory-side cache from HBM) + one write of dlogits
-    "c2": 18.80e9 + 16.82e9,
+    # lsg_grpo_fused_kernel: one read of the logits (the row waits on the CU for the gradient pass) + one write of
+    # dlogits
+    "c2": 16.88e9 + 16.95e9,
     "c2-two-pass": 16.83e9 + 0.0e9,  # lsg_entropy_fwd_kernel: 1.00x the logits
 }
 
@@ -209,7 +209,7 @@ def make_c2(torch, oi, rows_b=64, t=1024, vocab=128256, single_pass=True):
             "tokens": n,
             "rows_multiplied": n,
             "bytes_step": 2.0 * n * vocab * 2,
-            "kernel": "lsg_grpo_fused_kernel (one 1024-thread workgroup per row: statistics pass, GRPO derivative, gradient pass; 144 KB of the row wait in the LDS, the rest is read again from the caches)",
+            "kernel": "lsg_grpo_fused_kernel (one resident 1024-thread workgroup per CU: statistics pass, GRPO derivative, gradient pass; the row waits in the LDS and in registers between the passes)",
             "alg_per_launch": 2.0 * n * vocab * 2,
             "bound": "hbm",
             "timer": fwd_timer,

@@ -100,8 +100,8 @@ int oi_lsg_bwd(const void* logits, int dtype, int64_t n_outer, int64_t n_inner, 
  *   dlogits[row, j] = g * inv_T * (1[j == index] - softmax_j).
  * token_coef (fp32 per row) carries the loss denominators, which depend on the mask alone:
  * scale / denominator on response tokens, 0 elsewhere (such rows get a zero gradient row).
- * Requirement: 16-byte aligned rows (pointers and strides of logits and dlogits); OI_EALIGN
- * otherwise (use the two-pass entry points).  dlogits must not alias logits (OI_EINVAL).  The scalar loss and
+ * Requirement: 16-byte aligned rows (pointers and strides of logits and dlogits) of at least 16
+ * bytes; OI_EALIGN otherwise (use the two-pass entry points).  dlogits must not alias logits (OI_EINVAL).  The scalar loss and
  * its statistics come from oi_grpo_fused_fwd on `logprob`.
  */
 int oi_lsg_grpo_fwd_bwd(const void* logits, int dtype, int64_t n_outer, int64_t n_inner, int64_t stride_outer,

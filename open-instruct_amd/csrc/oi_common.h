@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "oi_kernels.h"
 
 #define OI_WAVE 64
@@ -25,6 +27,20 @@ static inline int oi_launch_status() {
 }
 
 static inline bool oi_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// Number of CUs of the current device.  Looked up once per device and source file; the value never
+// changes afterwards, so a relaxed atomic is all the concurrency control the cache needs.
+static inline int oi_cu_count() {
+    static std::atomic<int> cus_of_device[64];  // 0 = not looked up yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    int cus = cus_of_device[dev].load(std::memory_order_relaxed);
+    if (cus == 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        cus_of_device[dev].store(cus, std::memory_order_relaxed);
+    }
+    return cus;
+}
 
 typedef uint32_t oi_u32x4 __attribute__((ext_vector_type(4)));
 typedef float oi_f32x4 __attribute__((ext_vector_type(4)));

@@ -22,7 +22,6 @@
 // CU that draws tile ids from per-XCD counters.
 #include "oi_common.h"
 
-#include <atomic>
 #include <type_traits>
 
 namespace {
@@ -1026,14 +1025,7 @@ __global__ void __launch_bounds__(256)
 // Workgroups of a queue-driven launch: one per CU of the current device (each takes a whole CU's
 // LDS), a multiple of 8 so that every XCD gets the same number, and no more than there are tiles.
 unsigned resident_grid(int64_t tiles_m, int64_t tiles_n) {
-    static std::atomic<int> cus_of_device[64];  // 0 = not looked up yet; the value never changes afterwards
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-    int cus = cus_of_device[dev].load(std::memory_order_relaxed);
-    if (cus == 0) {
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-        cus_of_device[dev].store(cus, std::memory_order_relaxed);
-    }
+    const int cus = oi_cu_count();
     const int64_t grid = (cus + 7) / 8 * 8;
     const int64_t pids = pids_for_tiles(tiles_m, tiles_n);
     return (unsigned)(pids < grid ? pids : grid);

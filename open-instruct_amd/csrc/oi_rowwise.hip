@@ -8,6 +8,8 @@
 #include "oi_common.h"
 #include "oi_grpo_math.h"
 
+#include <type_traits>
+
 namespace {
 
 struct F32Row {
@@ -106,6 +108,32 @@ __device__ __forceinline__ void stat_update(RowStat& st, const float (&z)[VEC], 
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
         const float d = x[j] - mn;
+        const float e = __builtin_amdgcn_exp2f(d);
+        s += e;
+        if (ENT) t = fmaf(e, d, t);
+    }
+    st.m = mn;
+    st.s = s;
+    st.t = t;
+}
+
+// The same update with one multiply less per logit: the maximum is taken over the unscaled logits
+// (c > 0) and every exponent is a single fma.  The running maximum is then the rounded product
+// max(z) * c while the exponents are rounded once, so the largest term is 2^(a few ulp) instead of
+// exactly 1: far below the accuracy of the sum.
+template <int VEC, bool ENT>
+__device__ __forceinline__ void stat_update_fma(RowStat& st, const float (&z)[VEC], float c) {
+    float zmax = z[0];
+#pragma unroll
+    for (int j = 1; j < VEC; ++j) zmax = fmaxf(zmax, z[j]);
+    const float mn = fmaxf(st.m, zmax * c);
+    const float shift = st.m - mn;  // <= 0
+    const float alpha = __builtin_amdgcn_exp2f(shift);
+    float s = st.s * alpha;
+    float t = ENT ? alpha * fmaf(shift, st.s, st.t) : 0.f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        const float d = fmaf(z[j], c, -mn);
         const float e = __builtin_amdgcn_exp2f(d);
         s += e;
         if (ENT) t = fmaf(e, d, t);
@@ -420,181 +448,221 @@ int launch_bwd(const void* logits, int64_t rows, int64_t n_inner, int64_t so, in
 
 // ---------------------------------------------------------------------------------------------
 // GRPO on materialised logits in one launch: forward statistics and the gradient with respect to
-// the logits, with the second read of a row served by the caches instead of HBM.
+// the logits, with HBM seeing every row read once and its gradient written once.
 //
 // A token's upstream gradient depends on nothing but that token's own logprob and side inputs
 // (old / reference logprobs, advantage, weight) once the loss denominators are known, and those
-// depend on the mask alone.  So one 1024-thread workgroup per row reduces the softmax statistics
-// (ordinary loads, so that the row stays in the memory-side cache), evaluates the GRPO derivative
-// of the token and immediately streams the same row again (non-temporal loads, it is not needed
-// any more) to write d logits.  Only a few hundred rows (one or two per CU, 256 KB each at a 128 k
-// vocabulary) are between their two reads at any time, far less than the 256 MB of that cache.
-// A version that kept the row in registers between the passes (512 threads x 32 vectors) was
-// slower than two separate kernels: one workgroup per CU with nothing to overlap its load, compute
-// and store phases.  `token_coef` carries scale / denominator per token (0 on masked-out tokens).
+// depend on the mask alone.  So a 1024-thread workgroup reduces the softmax statistics of a row
+// while parking the row on the CU (144 KB of it in the LDS, the rest in registers: 16 sweeps of
+// 1024 16-byte pieces hold a row of 131072 bf16 logits), evaluates the GRPO derivative of the
+// token and writes d logits from the parked copy.  What a longer row has beyond that is read a
+// second time, from the caches.
+//
+// One workgroup per CU stays for the whole launch and takes every gridDim.x-th row: the loads of
+// the next row are issued while the stores of the previous one are still draining (a fresh
+// workgroup per row cannot start before the last store of its predecessor has left the CU, 4 us of
+// a 25 us row), and the row's side inputs are requested at the top of the row, long before the
+// lane that needs them gets there.  `token_coef` carries scale / denominator per token (0 on
+// masked-out tokens).
 // ---------------------------------------------------------------------------------------------
 constexpr int FUSED_ROW_THREADS = 1024;
-constexpr int FUSED_ROW_U = 4;
-// 16-byte pieces of a row that wait in the LDS for the second pass: 144 KB of the CU's 160 KB (the
-// kernel runs one 1024-thread workgroup per CU anyway), a whole number of sweeps of the workgroup
-constexpr int FUSED_STASH_VECS = 9 * FUSED_ROW_THREADS;
+// sweeps of the workgroup over the row that are parked in the LDS (9 x 16 KB = 144 KB of the CU's
+// 160 KB) and in registers (7 x 4 VGPRs per thread)
+constexpr int FUSED_STASH_SWEEPS = 9;
+constexpr int FUSED_KEEP_SWEEPS = 7;
+constexpr int FUSED_SWEEPS = FUSED_STASH_SWEEPS + FUSED_KEEP_SWEEPS;
+constexpr int FUSED_STASH_VECS = FUSED_STASH_SWEEPS * FUSED_ROW_THREADS;
+constexpr int FUSED_RESIDENT_VECS = FUSED_SWEEPS * FUSED_ROW_THREADS;
+// 16-byte loads per thread in flight during the first pass
+constexpr int FUSED_LOOKAHEAD = 7;
 
 template <typename R>
 __global__ void __launch_bounds__(FUSED_ROW_THREADS)
-    lsg_grpo_fused_kernel(const typename R::elem_t* __restrict__ logits, int64_t n_inner, int64_t stride_outer,
-                          int64_t stride_inner, int64_t vocab, const int64_t* __restrict__ index, float inv_t,
-                          const float* __restrict__ old_lp, const float* __restrict__ ref_lp,
-                          const float* __restrict__ adv, const float* __restrict__ rho,
-                          const float* __restrict__ token_coef, GrpoCfg cfg, float beta,
-                          float* __restrict__ logprob, float* __restrict__ entropy, float* __restrict__ lse_out,
-                          typename R::elem_t* __restrict__ dlogits, int64_t out_stride_outer,
-                          int64_t out_stride_inner) {
+    lsg_grpo_fused_kernel(const typename R::elem_t* __restrict__ logits, int64_t n_rows, int64_t n_inner,
+                          int64_t stride_outer, int64_t stride_inner, int64_t vocab,
+                          const int64_t* __restrict__ index, float inv_t, const float* __restrict__ old_lp,
+                          const float* __restrict__ ref_lp, const float* __restrict__ adv,
+                          const float* __restrict__ rho, const float* __restrict__ token_coef, GrpoCfg cfg,
+                          float beta, float* __restrict__ logprob, float* __restrict__ entropy,
+                          float* __restrict__ lse_out, typename R::elem_t* __restrict__ dlogits,
+                          int64_t out_stride_outer, int64_t out_stride_inner) {
     constexpr int VEC = R::VEC;
     constexpr int NW = FUSED_ROW_THREADS / OI_WAVE;
-    constexpr int U = FUSED_ROW_U;
     constexpr int64_t nthr = FUSED_ROW_THREADS;
     __shared__ float sm[3][NW];
     __shared__ float bcast[2];
     __shared__ __align__(16) typename R::raw_t stash[FUSED_STASH_VECS];
     static_assert(sizeof(typename R::raw_t) == 16, "row pieces are 16 bytes");
-    const int64_t row = blockIdx.x;
-    const typename R::elem_t* p = logits + row_offset(row, n_inner, stride_outer, stride_inner);
-    typename R::elem_t* q = dlogits + row_offset(row, n_inner, out_stride_outer, out_stride_inner);
     const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
     const int64_t nvec = vocab / VEC;
     const float c = inv_t * OI_LOG2E;
+    // the offset of this thread's first piece of a row, as a value the optimiser cannot trace: the
+    // addresses of the 16 sweeps are then formed where they are used instead of once for both passes,
+    // where they would occupy 64 registers from the first load to the last store
+    auto untraced = [](int off) {
+        asm volatile("" : "+v"(off));
+        return off;
+    };
+    const int first_piece = tid * VEC;
+    // loads past the end of a short row are redirected to its last piece instead of being skipped:
+    // unconditional loads are waited for one by one, guarded ones all at once
+    const int last_piece = (int)((nvec - 1) * VEC);  // the launcher refuses rows without a whole piece
 
-    // The first FUSED_STASH_VECS 16-byte pieces of the row stay in the LDS between the two passes
-    // (every thread keeps exactly the pieces it will need again, so no barrier guards them); only
-    // the rest of the row is read a second time, from the caches.  Pieces that go into the LDS
-    // are fetched with non-temporal loads, the others with ordinary ones so that they stay cached.
-    RowStat st = {OI_NEG_BIG, 0.f, 0.f};
-    {
-        int64_t i = tid;
-        for (; i + (U - 1) * nthr < nvec; i += U * nthr) {
-            typename R::raw_t raw[U];
+    typename R::raw_t raw[FUSED_SWEEPS];  // sweeps past the LDS part stay here for the second pass
+    auto issue = [&](const typename R::elem_t* src, int k) {
+        const int piece = untraced(first_piece) + k * (int)nthr * VEC;
+        raw[k] = R::load_raw(src + (piece < last_piece ? piece : last_piece));
+    };
+    static_assert(FUSED_LOOKAHEAD <= FUSED_STASH_SWEEPS, "the registers of the first sweeps must be free in the second pass");
+    if ((int64_t)blockIdx.x < n_rows) {
+        const typename R::elem_t* first = logits + row_offset(blockIdx.x, n_inner, stride_outer, stride_inner);
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int64_t v = i + u * nthr;
-                raw[u] = (v - tid < FUSED_STASH_VECS) ? R::load_raw(p + v * VEC) : R::load_raw_cached(p + v * VEC);
-            }
+        for (int k = 0; k < FUSED_LOOKAHEAD; ++k) issue(first, k);
+    }
+    for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+        const typename R::elem_t* p = logits + row_offset(row, n_inner, stride_outer, stride_inner);
+        typename R::elem_t* q = dlogits + row_offset(row, n_inner, out_stride_outer, out_stride_inner);
+        // side inputs of the row, requested now and consumed after the first pass
+        int64_t y = index[row];
+        y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
+        const float coef = token_coef[row];
+        const float old_row = old_lp ? old_lp[row] : 0.f;
+        const float ref_row = ref_lp ? ref_lp[row] : 0.f;
+        const float adv_row = adv[row];
+        const float rho_row = rho ? rho[row] : 1.f;
+
+        // first pass: statistics, and the row is parked.  A rolling window: the load of sweep
+        // k + FUSED_LOOKAHEAD is issued before sweep k is consumed, so that many 16-byte loads per
+        // thread are in flight throughout; the first FUSED_LOOKAHEAD sweeps were requested before
+        // the previous row's second pass and arrived while it ran.  Parked pieces are fetched with
+        // non-temporal loads, what lies beyond with ordinary ones so that it stays cached for the
+        // second pass.
+        RowStat st = {OI_NEG_BIG, 0.f, 0.f};
+        const float zy = R::load_one(p + y);
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int64_t v = i + u * nthr;
-                if (v - tid < FUSED_STASH_VECS) stash[v] = raw[u];
+        for (int k = 0; k < FUSED_SWEEPS; ++k) {
+            if (k + FUSED_LOOKAHEAD < FUSED_SWEEPS) issue(p, k + FUSED_LOOKAHEAD);
+            const int64_t v = tid + (int64_t)k * nthr;
+            if (k < FUSED_STASH_SWEEPS) stash[v] = raw[k];
+            if (v < nvec) {
                 float z[VEC];
-                R::unpack(raw[u], z);
-                stat_update<VEC, true>(st, z, c);
+                R::unpack(raw[k], z);
+                stat_update_fma<VEC, true>(st, z, c);
             }
+            // one piece's temporaries at a time: the parked pieces need the registers
+            __builtin_amdgcn_sched_barrier(0);
         }
-        for (; i < nvec; i += nthr) {
-            if (i - tid < FUSED_STASH_VECS) {
-                const typename R::raw_t r = R::load_raw(p + i * VEC);
-                stash[i] = r;
-                float z[VEC];
-                R::unpack(r, z);
-                stat_update<VEC, true>(st, z, c);
-                continue;
-            }
+        for (int64_t i = FUSED_RESIDENT_VECS + tid; i < nvec; i += nthr) {
             float z[VEC];
             R::unpack(R::load_raw_cached(p + i * VEC), z);
             stat_update<VEC, true>(st, z, c);
         }
         for (int64_t j = nvec * VEC + tid; j < vocab; j += nthr) stat_update1<true>(st, R::load_one(p + j), c);
-    }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        RowStat o;
-        o.m = __shfl_xor(st.m, off, OI_WAVE);
-        o.s = __shfl_xor(st.s, off, OI_WAVE);
-        o.t = __shfl_xor(st.t, off, OI_WAVE);
-        st = stat_merge(st, o);
-    }
-    const int wave = tid >> 6, lane = tid & 63;
-    if (lane == 0) {
-        sm[0][wave] = st.m;
-        sm[1][wave] = st.s;
-        sm[2][wave] = st.t;
-    }
-    __syncthreads();
-    int64_t y = index[row];
-    y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
-    if (tid == 0) {
-        RowStat tot = {sm[0][0], sm[1][0], sm[2][0]};
-        for (int w = 1; w < NW; ++w) {
-            RowStat o = {sm[0][w], sm[1][w], sm[2][w]};
-            tot = stat_merge(tot, o);
+        for (int off = 32; off > 0; off >>= 1) {
+            RowStat o;
+            o.m = __shfl_xor(st.m, off, OI_WAVE);
+            o.s = __shfl_xor(st.s, off, OI_WAVE);
+            o.t = __shfl_xor(st.t, off, OI_WAVE);
+            st = stat_merge(st, o);
         }
-        const double ln2 = 0.69314718055994530942;
-        const double log2s = log2((double)tot.s);
-        const double lse = ((double)tot.m + log2s) * ln2;
-        const float zy = R::load_one(p + y);
-        const float lp = (float)((double)zy * (double)inv_t - lse);
-        logprob[row] = lp;
-        if (entropy) entropy[row] = (float)((log2s - (double)tot.t / (double)tot.s) * ln2);
-        if (lse_out) lse_out[row] = (float)lse;
-        const float coef = token_coef[row];
-        float g = 0.f;
-        if (coef != 0.f) {
-            const float ratio = old_lp ? expf(lp - old_lp[row]) : 1.f;
-            const float w = rho ? rho[row] : 1.f;
-            g = coef * grpo_token_dnew(lp, ratio, adv[row], ref_lp != nullptr, ref_lp ? ref_lp[row] : 0.f, w, cfg, beta);
+        if (lane == 0) {
+            sm[0][wave] = st.m;
+            sm[1][wave] = st.s;
+            sm[2][wave] = st.t;
         }
-        bcast[0] = g * inv_t;
-        bcast[1] = (float)lse * OI_LOG2E;
-    }
-    __syncthreads();
-    const float g = bcast[0], l2 = bcast[1];
-    const float ng = -g;
-    if (g == 0.f) {
-        float zero[VEC];
+        __syncthreads();
+        {
+            // The registers of the first sweeps are free now (those sweeps wait in the LDS): the next
+            // row's first loads travel while this row's gradient is computed and stored, so the CU
+            // keeps reading during its write phase.  After the last row the same row is read again,
+            // which keeps the loads unconditional.
+            const int64_t next = row + gridDim.x < n_rows ? row + gridDim.x : row;
+            const typename R::elem_t* pn = logits + row_offset(next, n_inner, stride_outer, stride_inner);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) zero[j] = 0.f;
-        for (int64_t i = tid; i < nvec; i += nthr) R::store_vec(q + i * VEC, zero);
-        for (int64_t j = nvec * VEC + tid; j < vocab; j += nthr) R::store_one(q + j, 0.f);
-        return;
-    }
-    // second pass.  The tail of the row (read moments ago by this workgroup) comes from the
-    // caches: its first loads are requested now and consumed after the part that waits in the LDS.
-    const int64_t head = nvec < FUSED_STASH_VECS ? nvec : (int64_t)FUSED_STASH_VECS;
-    int64_t i = FUSED_STASH_VECS + tid;
-    typename R::raw_t rz[U], rn[U];
-    if (i + (U - 1) * nthr < nvec) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) rz[u] = R::load_raw(p + (i + u * nthr) * VEC);
-    }
-    auto emit = [&](typename R::raw_t raw, int64_t base) {
-        float w[VEC];
-        R::unpack(raw, w);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) w[j] = ng * __builtin_amdgcn_exp2f(fmaf(w[j], c, -l2));
-        if (y >= base && y < base + VEC) {
-#pragma unroll
-            for (int j = 0; j < VEC; ++j)
-                if (base + j == y) w[j] += g;
+            for (int k = 0; k < FUSED_LOOKAHEAD; ++k) issue(pn, k);
         }
-        R::store_vec(q + base, w);
-    };
-    for (int64_t k = tid; k < head; k += nthr) emit(stash[k], k * VEC);
-    for (; i + (U - 1) * nthr < nvec; i += U * nthr) {
-        const int64_t nx = i + U * nthr;
-        const bool more = nx + (U - 1) * nthr < nvec;
-        if (more) {
-#pragma unroll
-            for (int u = 0; u < U; ++u) rn[u] = R::load_raw(p + (nx + u * nthr) * VEC);
+        if (tid == 0) {
+            RowStat tot = {sm[0][0], sm[1][0], sm[2][0]};
+            for (int w = 1; w < NW; ++w) {
+                RowStat o = {sm[0][w], sm[1][w], sm[2][w]};
+                tot = stat_merge(tot, o);
+            }
+            const double ln2 = 0.69314718055994530942;
+            const double log2s = log2((double)tot.s);
+            const double lse = ((double)tot.m + log2s) * ln2;
+            const float lp = (float)((double)zy * (double)inv_t - lse);
+            logprob[row] = lp;
+            if (entropy) entropy[row] = (float)((log2s - (double)tot.t / (double)tot.s) * ln2);
+            if (lse_out) lse_out[row] = (float)lse;
+            float g = 0.f;
+            if (coef != 0.f) {
+                const float ratio = old_lp ? expf(lp - old_row) : 1.f;
+                g = coef * grpo_token_dnew(lp, ratio, adv_row, ref_lp != nullptr, ref_row, rho_row, cfg, beta);
+            }
+            bcast[0] = g * inv_t;
+            bcast[1] = (float)lse * OI_LOG2E;
         }
+        __syncthreads();
+        // (the next row's writes of sm / bcast come after that row's first barrier, which no thread
+        // passes before it has read these two values)
+        const float g = bcast[0], l2 = bcast[1];
+        const float ng = -g;
+        // - g 2^(x - l2) = -+ 2^(x - l2 + log2 |g|): one multiply less per logit in the parked part
+        const float l2g = l2 - __builtin_amdgcn_logf(fabsf(g));
+        const bool g_positive = g > 0.f;
+        if (g == 0.f) {
+            float zero[VEC];
 #pragma unroll
-        for (int u = 0; u < U; ++u) emit(rz[u], (i + u * nthr) * VEC);
-        if (more) {
-#pragma unroll
-            for (int u = 0; u < U; ++u) rz[u] = rn[u];
+            for (int j = 0; j < VEC; ++j) zero[j] = 0.f;
+            for (int64_t i = tid; i < nvec; i += nthr) R::store_vec(q + i * VEC, zero);
+            for (int64_t j = nvec * VEC + tid; j < vocab; j += nthr) R::store_one(q + j, 0.f);
+            continue;
         }
-    }
-    for (; i < nvec; i += nthr) emit(R::load_raw(p + i * VEC), i * VEC);
-    for (int64_t j = nvec * VEC + tid; j < vocab; j += nthr) {
-        float d = ng * __builtin_amdgcn_exp2f(fmaf(R::load_one(p + j), c, -l2));
-        if (j == y) d += g;
-        R::store_one(q + j, d);
+        // second pass: the parked part (every thread reads back exactly the LDS entries it wrote, so
+        // no barrier guards them), then what lies beyond it
+        auto emit = [&](typename R::raw_t piece, typename R::elem_t* dst) {
+            float w[VEC];
+            R::unpack(piece, w);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) w[j] = ng * __builtin_amdgcn_exp2f(fmaf(w[j], c, -l2));
+            R::store_vec(dst, w);
+        };
+        auto emit_signed = [&](typename R::raw_t piece, typename R::elem_t* dst, auto negative_tag) {
+            float w[VEC];
+            R::unpack(piece, w);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float e = __builtin_amdgcn_exp2f(fmaf(w[j], c, -l2g));
+                w[j] = decltype(negative_tag)::value ? -e : e;
+            }
+            R::store_vec(dst, w);
+        };
+        auto parked_sweeps = [&](auto negative_tag) {
+#pragma unroll
+            for (int k = 0; k < FUSED_SWEEPS; ++k) {
+                const int64_t v = tid + (int64_t)k * nthr;
+                if (v < nvec) {
+                    typename R::elem_t* dst = q + untraced(first_piece) + (int64_t)k * nthr * VEC;
+                    if (k < FUSED_STASH_SWEEPS) emit_signed(stash[v], dst, negative_tag);
+                    else emit_signed(raw[k], dst, negative_tag);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        if (g_positive) parked_sweeps(std::true_type{});  // d logits = - g softmax
+        else parked_sweeps(std::false_type{});
+        for (int64_t i = FUSED_RESIDENT_VECS + tid; i < nvec; i += nthr) emit(R::load_raw(p + i * VEC), q + i * VEC);
+        // the label's entry gets + g.  The thread that stored the piece holding it stores the entry
+        // again (stores of one thread to one address keep their order): no sweep has to look for it.
+        if (y < nvec * VEC && (int)((y / VEC) % nthr) == tid)
+            R::store_one(q + y, ng * __builtin_amdgcn_exp2f(fmaf(zy, c, -l2)) + g);
+        for (int64_t j = nvec * VEC + tid; j < vocab; j += nthr) {
+            float d = ng * __builtin_amdgcn_exp2f(fmaf(R::load_one(p + j), c, -l2));
+            if (j == y) d += g;
+            R::store_one(q + j, d);
+        }
     }
 }
 
@@ -606,10 +674,12 @@ int launch_grpo_fused(const void* logits, int64_t rows, int64_t n_inner, int64_t
     typedef typename R::elem_t E;
     const bool vec = oi_aligned(logits, 16) && oi_aligned(dlogits, 16) && (so % R::VEC == 0) && (si % R::VEC == 0) &&
                      (oso % R::VEC == 0) && (osi % R::VEC == 0);
-    OI_RETURN_IF(!vec, OI_EALIGN);
-    hipLaunchKernelGGL((lsg_grpo_fused_kernel<R>), dim3((unsigned)rows), dim3(FUSED_ROW_THREADS), 0, stream,
-                       static_cast<const E*>(logits), n_inner, so, si, vocab, index, inv_t, old_lp, ref_lp, adv, rho, coef,
-                       cfg, beta, logprob, entropy, lse, static_cast<E*>(dlogits), oso, osi);
+    OI_RETURN_IF(!vec || vocab < R::VEC, OI_EALIGN);
+    // one resident workgroup per CU (its LDS share leaves room for no second one)
+    const int64_t cus = oi_cu_count();
+    hipLaunchKernelGGL((lsg_grpo_fused_kernel<R>), dim3((unsigned)(rows < cus ? rows : cus)), dim3(FUSED_ROW_THREADS), 0,
+                       stream, static_cast<const E*>(logits), rows, n_inner, so, si, vocab, index, inv_t, old_lp, ref_lp,
+                       adv, rho, coef, cfg, beta, logprob, entropy, lse, static_cast<E*>(dlogits), oso, osi);
     return oi_launch_status();
 }
 

@@ -468,7 +468,7 @@ def grpo_loss_on_logits(
     Same result as ``forward_for_logprobs`` → ``grpo_loss_fused`` (open_instruct/grpo_utils.py:541-574,
     open_instruct/grpo_fast.py:702-724) and the same gradient with respect to ``logits`` after
     ``loss.backward()``, but HBM sees the ``[B, T, V]`` tensor read once and its gradient written
-    once (the second read of a row comes from the caches): a token's upstream gradient depends only on its own logprob and side inputs once the
+    once (a row waits on its CU between the two passes): a token's upstream gradient depends only on its own logprob and side inputs once the
     denominators are known, and those come from the mask.  The gradient is computed in the
     forward call and stored (one tensor of the logits' shape and dtype, which the backward pass
     would allocate anyway).  ``logits`` is ``[B, T, V]`` (``[B, T + 1, V]`` with ``drop_last``),

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from conftest import make_grpo_config
-from open_instruct_amd import dpo_utils, grpo_utils, model_utils, padding_free_collator, rl_utils
+from open_instruct_amd import _lib, dpo_utils, grpo_utils, model_utils, padding_free_collator, rl_utils
 from oracle import dpo as o_dpo
 from oracle import grpo as o_grpo
 from oracle import logprob as o_logprob
@@ -605,7 +605,11 @@ def test_reference_cache_build_through_concatenated_forward():
     assert picked["chosen_logps"].shape == (2,)
 
 
-@pytest.mark.parametrize("dtype,vocab", [(torch.float32, 64), (torch.bfloat16, 4096), (torch.bfloat16, 4099), (torch.float16, 1000)])
+@pytest.mark.parametrize("dtype,vocab", [
+    (torch.float32, 64), (torch.bfloat16, 4096), (torch.bfloat16, 4099), (torch.float16, 1000),
+    # rows longer than what a workgroup parks on its CU (16384 16-byte pieces): the rest is read twice
+    (torch.bfloat16, 151936), (torch.float32, 70000),
+])  # fmt: skip
 @pytest.mark.parametrize("loss_fn,axis,denominator,with_old,with_ref,drop_last", [
     ("dapo", None, None, True, True, False),
     ("dapo", 1, None, True, True, True),
@@ -682,6 +686,55 @@ def test_grpo_loss_on_logits_single_pass(dtype, vocab, loss_fn, axis, denominato
     )  # fmt: skip
     (loss3 * 2.0).backward()
     assert (lg3.grad.float() - 2.0 * lg.grad.float()).abs().max().item() <= 2.0 * step * max(1e-3, lg.grad.float().abs().max().item())
+
+
+def test_grpo_on_logits_raw_c_abi_rows_with_scalar_tail():
+    """oi_lsg_grpo_fwd_bwd through ctypes on rows whose length is not a multiple of the 16-byte piece
+    (a [rows, 4099] view of a [rows, 4104] buffer, gradient into a buffer of the same pitch), more rows
+    than workgroups' first round, labels in the last whole piece, in the scalar tail and at 0; against
+    the oracle's autograd (open_instruct/grpo_utils.py:504-538 on open_instruct/model_utils.py:587-603)."""
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(17)
+    rows, vocab, pitch = 700, 4099, 4104
+    buf = (torch.randn(rows, pitch, generator=g) * 2.0).bfloat16()
+    labels = torch.randint(0, vocab, (rows,), generator=g)
+    labels[:4] = torch.tensor([0, vocab - 1, vocab - 3, 4095])
+    adv = torch.randn(rows, generator=g)
+    mask = torch.rand(rows, generator=g) > 0.3
+    cfg = make_grpo_config(loss_fn="dapo", beta=0.05, kl_estimator=2, clip_higher=0.28)
+    ref_in = buf[:, :vocab].float().clone().requires_grad_(True)
+    lp_o = o_logprob.log_softmax_and_gather(ref_in, labels, None, 1.0)
+    ent_o = o_logprob.entropy_from_logits(ref_in.detach(), None, 1.0)
+    old = lp_o.detach() + 0.05 * torch.randn(rows, generator=g)
+    ref = lp_o.detach() + 0.1 * torch.randn(rows, generator=g)
+    loss_o, *_ = o_grpo.grpo_token_loss(
+        lp_o[None], old[None], ref[None], adv[None], mask.float()[None], cfg, rho_weights=torch.ones(1, rows),
+        loss_denominator=None, axis=None, dp_scale=1.0,
+    )  # fmt: skip
+    loss_o.backward()
+    d = lambda x: x.to(DEV).contiguous()  # noqa: E731
+    lg, out = d(buf), torch.full((rows, pitch), 7.0, device=DEV).bfloat16()
+    coef = d(mask.float() / mask.sum())
+    lp, ent = torch.empty(rows, device=DEV), torch.empty(rows, device=DEV)
+    lab, old_d, ref_d, adv_d = d(labels), d(old), d(ref), d(adv)
+    rc = lib.oi_lsg_grpo_fwd_bwd(
+        lg.data_ptr(), 1, rows, 1, pitch, pitch, vocab, lab.data_ptr(), 1.0, old_d.data_ptr(), ref_d.data_ptr(),
+        adv_d.data_ptr(), None, coef.data_ptr(), 0, 1.0 - cfg.clip_lower, 1.0 + cfg.clip_higher, 2, cfg.beta,
+        lp.data_ptr(), ent.data_ptr(), None, out.data_ptr(), pitch, pitch, torch.cuda.current_stream().cuda_stream,
+    )  # fmt: skip
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert (lp.cpu() - lp_o.detach()).abs().max().item() <= 2e-3
+    assert (ent.cpu() - ent_o).abs().max().item() <= 2e-3
+    assert (out[:, :vocab].float().cpu() - ref_in.grad).abs().max().item() <= 2e-3
+    assert (out[:, :vocab].float().cpu() - ref_in.grad).abs().max().item() <= 2.0**-7 * ref_in.grad.abs().max().item()
+    assert (out[:, vocab:] == 7.0).all()  # the padding of the gradient buffer is not touched
+    # rows shorter than one piece are refused, as are unaligned pitches
+    args = lambda v, so: (lg.data_ptr(), 1, rows, 1, so, so, v, lab.data_ptr(), 1.0, None, None, adv_d.data_ptr(), None,  # noqa: E731
+                          coef.data_ptr(), 0, 0.8, 1.28, 2, 0.0, lp.data_ptr(), ent.data_ptr(), None, out.data_ptr(), so, so,
+                          torch.cuda.current_stream().cuda_stream)  # fmt: skip
+    assert lib.oi_lsg_grpo_fwd_bwd(*args(5, pitch)) < 0
+    assert lib.oi_lsg_grpo_fwd_bwd(*args(vocab, vocab)) < 0
 
 
 def test_grpo_loss_on_logits_full_vocabulary_rows():
