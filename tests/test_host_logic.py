@@ -287,3 +287,21 @@ def test_olmo_forward_plumbing_passes_labels_and_doc_lens():
     assert kwargs["attention_mask"] is None and kwargs["doc_lens"].tolist() == [[2, 3, 1]] and kwargs["max_doc_lens"] == [3]
     with pytest.raises(AssertionError):
         grpo_utils.forward_for_logprobs(Recorder(), torch.ones(1, 6, dtype=torch.long), None, mask, 0, 1.0, pass_olmo_core_doc_lens=True)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures the one-GPU hot path only: any other GPU count ends with a message, before
+    torch or the library are touched."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                         timeout=120)  # fmt: skip
+    assert res.returncode == 2
+    assert "one-GPU" in res.stdout
+    env = dict(os.environ, WORLD_SIZE="4")
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py")], capture_output=True, text=True, env=env,
+                         timeout=120)  # fmt: skip
+    assert res.returncode == 2 and "one-GPU" in res.stdout
