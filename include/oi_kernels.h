@@ -88,10 +88,10 @@ int oi_lsg_bwd(const void* logits, int dtype, int64_t n_outer, int64_t n_inner, 
 
 /*
  * GRPO on materialised logits in one launch: forward (logprob / entropy / lse as
- * oi_lsg_entropy_fwd) and the gradient of the GRPO loss with respect to the logits.  Every row is
- * read twice by the same workgroup in close succession, so the second read is served by the
- * caches: HBM sees one read and one write of the [rows, vocab] tensor instead of two reads and a
- * write.  Fuses the sequence open_instruct/grpo_utils.py:541-574 (forward_for_logprobs) ->
+ * oi_lsg_entropy_fwd) and the gradient of the GRPO loss with respect to the logits.  A row stays
+ * on its CU (LDS and registers) between the statistics pass and the gradient pass; only what a row
+ * has beyond 16384 16-byte pieces is read a second time, from the caches.  HBM sees one read and
+ * one write of the [rows, vocab] tensor instead of two reads and a write.  Fuses the sequence open_instruct/grpo_utils.py:541-574 (forward_for_logprobs) ->
  * open_instruct/grpo_utils.py:504-538 (compute_grpo_loss) -> open_instruct/grpo_fast.py:702-724
  * (masked mean, backward) for callers that hold the logits.
  *
