@@ -383,8 +383,9 @@ size_t oi_lmhead_cache_bytes(int64_t n_tokens, int64_t vocab, int64_t cache_chun
  * neither the dZ chunk nor the fp32 accumulator is part of the workspace).  row_mask as in the forward (rows left out get a zero d_hidden row
  * and add nothing to d_weight); skip_zero_grad_rows != 0 also leaves out rows whose grad_logprob is
  * exactly 0, which changes no result (not together with a cache, whose rows are the forward's).
- * d_hidden and d_weight must be 4-byte aligned.  logprob (the forward's output) is read only with a
- * cache.
+ * d_hidden and d_weight must be 4-byte aligned.  logprob is the forward's output for the same rows:
+ * the label's entry of dZ is taken from it as -grad * inv_T * expm1(logprob), which stays exact
+ * where the label's probability is close to 1.
  */
 size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int want_d_weight,
                                      int with_row_selection, int64_t cache_chunks);

@@ -446,16 +446,16 @@ __device__ __forceinline__ void merge_stats(float ma, float sa, float ta, float 
 template <bool PARTIAL, bool KEEP>
 __device__ __forceinline__ void stats_update(AccTile& acc, int j, int wm, int lane, int64_t m0, int64_t vocab, float c,
                                              float& st_m, float& st_s, float& st_t) {
-    float vmax = OI_NEG_BIG;
+    // the maximum is taken over the unscaled logits (c > 0) and every exponent is one fma: the new
+    // maximum is the rounded product max(z) * c while the exponents are rounded once, so the largest
+    // term is 2^(a few ulp) rather than exactly 1, far below the accuracy of the sums
+    float zmax = OI_NEG_BIG;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            // keep the rounded product: the maximum and the exponents must see the same x
-            acc[i][j][r] *= c;
-            if (!PARTIAL || m0 + acc_row(wm, i, r, lane) < vocab) vmax = fmaxf(vmax, acc[i][j][r]);
-        }
-    const float mn = fmaxf(st_m, vmax);
+        for (int r = 0; r < 16; ++r)
+            if (!PARTIAL || m0 + acc_row(wm, i, r, lane) < vocab) zmax = fmaxf(zmax, acc[i][j][r]);
+    const float mn = fmaxf(st_m, fmaxf(zmax * c, OI_NEG_BIG));
     const float shift = st_m - mn;
     const float alpha = __builtin_amdgcn_exp2f(shift);
     float s = st_s * alpha;
@@ -465,7 +465,7 @@ __device__ __forceinline__ void stats_update(AccTile& acc, int j, int wm, int la
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            float d = acc[i][j][r] - mn;
+            float d = fmaf(acc[i][j][r], c, -mn);
             float e = __builtin_amdgcn_exp2f(d);
             if (PARTIAL && m0 + acc_row(wm, i, r, lane) >= vocab) {
                 d = 0.f;
@@ -666,10 +666,10 @@ __global__ void lmhead_fwd_combine_kernel(const float4* __restrict__ partial, co
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ void lmhead_dz_tile(const uint16_t* __restrict__ W, const uint16_t* __restrict__ hidden,
                                                const int64_t* __restrict__ labels, const float* __restrict__ lse,
-                                               const float* __restrict__ grad, int64_t n_tokens, int64_t hdim,
-                                               int64_t vocab, float c, float inv_t, int64_t v_begin, int64_t chunk_cols,
-                                               int64_t n_pad, uint16_t* __restrict__ dz, int64_t vt, int64_t tt,
-                                               uint16_t* lds) {
+                                               const float* __restrict__ grad, const float* __restrict__ logprob,
+                                               int64_t n_tokens, int64_t hdim, int64_t vocab, float c, float inv_t,
+                                               int64_t v_begin, int64_t chunk_cols, int64_t n_pad,
+                                               uint16_t* __restrict__ dz, int64_t vt, int64_t tt, uint16_t* lds) {
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6, wm = wave & 3, wn = wave >> 2;
     const int64_t n0 = tt * BN, m0 = v_begin + vt * BM;
 
@@ -694,32 +694,35 @@ __device__ __forceinline__ void lmhead_dz_tile(const uint16_t* __restrict__ W, c
         const float l2 = g != 0.f ? lse[n] * OI_LOG2E : 3.0e38f;
         int64_t y = live ? labels[n] : -1;
         if (live) y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
-        // the label's entry gets + g; find out whether this lane holds it and in which register
+        // The label's entry is g (1 - p_label) = - g expm1(logprob), taken from the forward's result
+        // (exact also where p_label is close to 1) and written over the entry that the sweep below
+        // leaves there: the sweep itself then treats all entries alike.
         const int rel = (live && y >= m0 && y < m0 + BM) ? (int)(y - m0) - wave_row0 : -1;
         const bool mine = rel >= 0 && rel < 64 && (((rel & 31) >> 2) & 1) == (lane >> 5);
-        const int target = mine ? (rel >> 5) * 16 + ((rel & 31) >> 3) * 4 + (rel & 3) : -1;
         const float ng = -g;
-        float z_label = 0.f;
+        auto sweep = [&](auto last_tile_tag) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                float d[4];
+                for (int q = 0; q < 4; ++q) {
+                    float d[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int r = q * 4 + e;
-                    if (i * 16 + r == target) z_label = acc[i][j][r];
-                    float val = ng * __builtin_amdgcn_exp2f(fmaf(acc[i][j][r], c, -l2));
-                    if (rows_left < BM && acc_row(wm, i, r, lane) >= rows_left) val = 0.f;  // last tile only
-                    d[e] = val;
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = q * 4 + e;
+                        float val = ng * __builtin_amdgcn_exp2f(fmaf(acc[i][j][r], c, -l2));
+                        if (decltype(last_tile_tag)::value && acc_row(wm, i, r, lane) >= rows_left) val = 0.f;
+                        d[e] = val;
+                    }
+                    const int vl = acc_row(wm, i, q * 4, lane) ^ (((nl >> 3) & 1) << 2);
+                    uint2 pk = make_uint2(oi_pack_bf16x2(d[0], d[1]), oi_pack_bf16x2(d[2], d[3]));
+                    *reinterpret_cast<uint2*>(stage + nl * STAGE_STRIDE + vl) = pk;
                 }
-                const int vl = acc_row(wm, i, q * 4, lane) ^ (((nl >> 3) & 1) << 2);
-                uint2 pk = make_uint2(oi_pack_bf16x2(d[0], d[1]), oi_pack_bf16x2(d[2], d[3]));
-                *reinterpret_cast<uint2*>(stage + nl * STAGE_STRIDE + vl) = pk;
-            }
+        };
+        if (rows_left < BM) sweep(std::true_type{});  // the last vocabulary tile: rows past the vocabulary hold 0
+        else sweep(std::false_type{});
         if (mine) {
             // same lane, same LDS word as the store above: program order keeps them apart
-            const float val = fmaf(ng, __builtin_amdgcn_exp2f(fmaf(z_label, c, -l2)), g);
+            const float val = ng * expm1f(logprob[n]);
             stage[nl * STAGE_STRIDE + ((wave_row0 + rel) ^ (((nl >> 3) & 1) << 2))] = (uint16_t)oi_f32_to_bf16_bits(val);
         }
     }
@@ -739,16 +742,17 @@ __device__ __forceinline__ void lmhead_dz_tile(const uint16_t* __restrict__ W, c
 __global__ void __launch_bounds__(NTHREADS)
     lmhead_dz_kernel(const uint16_t* __restrict__ W, const uint16_t* __restrict__ hidden,
                      const int64_t* __restrict__ labels, const float* __restrict__ lse,
-                     const float* __restrict__ grad, int64_t n_tokens, const int32_t* __restrict__ n_dev,
-                     int64_t hdim, int64_t vocab, float c, float inv_t, int64_t v_begin, int64_t chunk_cols,
-                     int64_t n_pad, uint16_t* __restrict__ dz, uint32_t* __restrict__ queue) {
+                     const float* __restrict__ grad, const float* __restrict__ logprob, int64_t n_tokens,
+                     const int32_t* __restrict__ n_dev, int64_t hdim, int64_t vocab, float c, float inv_t,
+                     int64_t v_begin, int64_t chunk_cols, int64_t n_pad, uint16_t* __restrict__ dz,
+                     uint32_t* __restrict__ queue) {
     __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
     if (n_dev) {
         n_tokens = *n_dev;
         n_pad = (n_tokens + BN - 1) / BN * BN;
     }
     for_each_tile(queue, chunk_cols / BM, n_pad / BN, lds, [&](int64_t vt, int64_t tt) {
-        lmhead_dz_tile(W, hidden, labels, lse, grad, n_tokens, hdim, vocab, c, inv_t, v_begin, chunk_cols, n_pad, dz,
+        lmhead_dz_tile(W, hidden, labels, lse, grad, logprob, n_tokens, hdim, vocab, c, inv_t, v_begin, chunk_cols, n_pad, dz,
                        vt, tt, lds);
     });
 }
@@ -1154,7 +1158,7 @@ struct RowInputs {
     const int64_t* labels;
     const float *lse, *grad;
     const int32_t *rows, *n_dev;  // null without a selection
-    const float* logprob;         // only with a cache of exponentials
+    const float* logprob;         // the forward's result: the label's entry of dZ is rebuilt from it
 };
 
 // select + gather on `s`; clears `n_zero` queue words on the way
@@ -1255,7 +1259,7 @@ void enqueue_bwd(const BwdPlan& p, char* ws, const RowInputs& in, const void* we
         uint32_t* q = queues + ci * 3 * QUEUE_WORDS;
         if (!cached)
             hipLaunchKernelGGL(lmhead_dz_kernel, dim3(resident_grid(cols / BM, p.n_pad / BN)), dim3(NTHREADS), 0, s, Wp,
-                               in.hidden, in.labels, in.lse, in.grad, n_tokens, in.n_dev, hidden_dim, vocab, c,
+                               in.hidden, in.labels, in.lse, in.grad, in.logprob, n_tokens, in.n_dev, hidden_dim, vocab, c,
                                inv_temperature, v_begin, cols, p.n_pad, dz, q);
         // the A operand of both products: this chunk's dZ, or this chunk's columns of the cache
         const uint16_t* a_ptr = cached ? ecache + v_begin : dz;
@@ -1370,8 +1374,7 @@ extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const 
     rc = check_cache(exp_cache, cache_chunks);
     if (rc != OI_OK) return rc;
     if (n_tokens == 0) return OI_OK;
-    OI_RETURN_IF(!lse || !grad_logprob || !d_hidden || !workspace, OI_ENULL);
-    OI_RETURN_IF(cache_chunks > 0 && !logprob, OI_ENULL);
+    OI_RETURN_IF(!lse || !grad_logprob || !logprob || !d_hidden || !workspace, OI_ENULL);
     // a cache written for the rows of a mask can only be read back for the same rows
     OI_RETURN_IF(cache_chunks > 0 && skip_zero_grad_rows, OI_EINVAL);
     // bf16 results are stored as pairs (4-byte words)
@@ -1393,7 +1396,7 @@ extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const 
     if (selecting) {
         in = launch_selection(p.sel, ws, hidden, labels, lse, grad_logprob, row_mask, skip_zero_grad_rows != 0, n_tokens,
                               hidden_dim, queues, select_clears_queues ? n_queue_words : 0, s,
-                              cache.chunks > 0 ? logprob : nullptr);
+                              logprob);
         hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, row_mask,
                            zero_grad_probe, hidden_dim, static_cast<uint16_t*>(d_hidden));
     }

@@ -58,7 +58,7 @@ class _FusedLMHead(torch.autograd.Function):
                 inv_temperature, logprob.data_ptr(), _lib.ptr(entropy), lse.data_ptr(), _lib.ptr(cache),
                 cache_chunks if cache is not None else 0, ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
             )  # fmt: skip
-        ctx.save_for_backward(hid, w, lab, lse, m, cache, logprob if cache is not None else None)
+        ctx.save_for_backward(hid, w, lab, lse, m, cache, logprob)
         ctx.inv_temperature = inv_temperature
         ctx.compact_backward = bool(compact_backward)
         ctx.cache_chunks = cache_chunks if cache is not None else 0
