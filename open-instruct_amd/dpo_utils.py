@@ -14,7 +14,7 @@ from collections.abc import Callable, Iterable
 
 import torch
 
-from . import _lib, model_utils, olmo_core_utils, padding_free_collator
+from . import _lib, lm_head, model_utils, olmo_core_utils, padding_free_collator
 from .padding_free_collator import get_batch_logps_padded
 
 
@@ -200,13 +200,16 @@ def _sequence_logps(per_token, labels, concat: dict, packing: bool, average_log_
 
 
 def concatenated_forward(
-    model, batch: dict, average_log_prob: bool = False, output_router_logits: bool = False, packing: bool = False
-):
+    model, batch: dict, average_log_prob: bool = False, output_router_logits: bool = False, packing: bool = False,
+    fused_head: bool = False,
+):  # fmt: skip
     """One model forward over chosen+rejected, then per-sequence logps; open_instruct/dpo_utils.py:826-878.
 
     HuggingFace interface: ``model(**inputs).logits``; with ``output_router_logits`` the model is
     asked for its router logits and the ``aux_loss`` of its output is passed through.  Returns
-    ``(chosen_logps, rejected_logps, aux_loss)``.
+    ``(chosen_logps, rejected_logps, aux_loss)``.  ``fused_head=True`` (not in the reference) runs
+    the model's trunk only and sends its hidden states through the fused lm_head, so the ``[B, T, V]``
+    logits are never formed and prompt / padding positions are not multiplied; same results.
     """
     if packing:
         concat, bs = padding_free_collator.concatenated_inputs(batch)
@@ -219,14 +222,19 @@ def concatenated_forward(
         if k.startswith("concatenated_") and not k.endswith("labels")
     }
     aux_loss = None
-    if output_router_logits:
-        output = model(**inputs, output_router_logits=True)
-        aux_loss = output.aux_loss
-    else:
-        output = model(**inputs)
-    logits = getattr(output, "logits", output)
     labels = concat["concatenated_labels"]
-    per_token = padding_free_collator.calculate_per_token_logps(logits, labels)
+    if fused_head:
+        if output_router_logits:
+            raise ValueError("fused_head runs the trunk only: the router's aux_loss is not available")
+        per_token = lm_head.per_token_logps_from_trunk(model, labels, **inputs)
+    else:
+        if output_router_logits:
+            output = model(**inputs, output_router_logits=True)
+            aux_loss = output.aux_loss
+        else:
+            output = model(**inputs)
+        logits = getattr(output, "logits", output)
+        per_token = padding_free_collator.calculate_per_token_logps(logits, labels)
     chosen, rejected = _split_pairs(_sequence_logps(per_token, labels, concat, packing, average_log_prob), bs)
     return chosen, rejected, aux_loss
 
@@ -239,16 +247,27 @@ def process_batch(batch: dict, prefix: str, pad_value: int = 0) -> dict[str, tor
     return {k[len(lead) :]: v for k, v in batch.items() if k.startswith(prefix) and isinstance(v, torch.Tensor)}
 
 
-def separate_forward(model, batch: dict, average_log_prob: bool = False, output_router_logits: bool = False):
+def separate_forward(
+    model, batch: dict, average_log_prob: bool = False, output_router_logits: bool = False, fused_head: bool = False
+):
     """Chosen and rejected sequences in two model forwards (selectable through ``forward_fn``);
     open_instruct/dpo_utils.py:881-956.  The logits are read in their own dtype with fp32
-    accumulation, so the reference's fp32 copy of them is not made."""
+    accumulation, so the reference's fp32 copy of them is not made.  ``fused_head`` as in
+    :func:`concatenated_forward`."""
+    if fused_head and output_router_logits:
+        raise ValueError("fused_head runs the trunk only: the router's aux_loss is not available")
     logps, aux = [], []
     for side in ("chosen", "rejected"):
         part = process_batch(batch, side)
-        kwargs = {"output_router_logits": True} if output_router_logits else {}
-        output = model(input_ids=part["input_ids"], attention_mask=part["attention_mask"], **kwargs)
-        per_token = padding_free_collator.calculate_per_token_logps(output.logits, part["labels"])
+        if fused_head:
+            per_token = lm_head.per_token_logps_from_trunk(
+                model, part["labels"], input_ids=part["input_ids"], attention_mask=part["attention_mask"]
+            )
+            output = None
+        else:
+            kwargs = {"output_router_logits": True} if output_router_logits else {}
+            output = model(input_ids=part["input_ids"], attention_mask=part["attention_mask"], **kwargs)
+            per_token = padding_free_collator.calculate_per_token_logps(output.logits, part["labels"])
         logps.append(_get_batch_logps(per_token, part["labels"], average_log_prob))
         aux.append(output.aux_loss if output_router_logits else None)
         del output, per_token

@@ -703,6 +703,8 @@ def forward_for_logprobs(
     temperature: float,
     return_entropy: bool = False,
     pass_olmo_core_doc_lens: bool = False,
+    fused_head: bool = False,
+    response_mask: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """Model forward, then logprob (and entropy) of each next token; open_instruct/grpo_utils.py:541-574.
 
@@ -712,6 +714,12 @@ def forward_for_logprobs(
     logits as the logprob.  With ``pass_olmo_core_doc_lens`` the integer-coded attention mask is
     turned into ``doc_lens`` / ``max_doc_lens`` for models with the olmo-core interface and no
     attention mask is passed, as in the reference.
+
+    ``fused_head=True`` (not in the reference; HuggingFace-style models) runs the model's trunk only
+    and sends its final hidden states through the fused lm_head: the ``[B, T, V]`` logits are never
+    formed.  With ``response_mask`` (``[B, T]``, the caller's mask before the shift) positions off
+    the mask are not multiplied and hold 0; the callers mask them anyway
+    (open_instruct/grpo_utils.py:340-344, open_instruct/grpo_fast.py:702-724).
     """
     extra_kwargs = {}
     if pass_olmo_core_doc_lens:
@@ -720,6 +728,18 @@ def forward_for_logprobs(
         doc_lens, max_doc_lens = olmo_core_utils.doc_lens_from_attention_mask(attention_mask)
         extra_kwargs = {"doc_lens": doc_lens, "max_doc_lens": max_doc_lens}
         attention_mask = None
+    if fused_head:
+        from . import lm_head
+
+        trunk, weight = lm_head.split_causal_lm(model)
+        out = trunk(input_ids=query_responses, attention_mask=attention_mask, position_ids=position_ids, **extra_kwargs)
+        hidden = getattr(out, "last_hidden_state", out[0] if isinstance(out, (tuple, list)) else out)
+        labels = query_responses[:, 1:].clone().to(hidden.device)
+        labels[labels == pad_token_id] = 0
+        keep = None if response_mask is None else response_mask[:, 1:].to(hidden.device) != 0
+        return lm_head.fused_lm_head_logprobs(
+            hidden[:, :-1], weight, labels, temperature=temperature, mask=keep, return_entropy=return_entropy
+        )
     output = model(input_ids=query_responses, attention_mask=attention_mask, position_ids=position_ids, **extra_kwargs)
     logits = getattr(output, "logits", output)
     labels = query_responses[:, 1:].clone().to(logits.device)

@@ -170,3 +170,34 @@ def fused_linear_cross_entropy(
     if torch.is_tensor(num_items_in_batch):
         num_items_in_batch = num_items_in_batch.to(total.device)
     return total / num_items_in_batch
+
+
+def split_causal_lm(model) -> tuple[torch.nn.Module, torch.Tensor]:
+    """``(trunk, lm_head weight)`` of a HuggingFace-style causal LM: the module that returns
+    ``last_hidden_state`` and the ``[V, H]`` matrix its logits are projected with (the pieces the
+    reference reaches through ``model(...)`` at open_instruct/grpo_utils.py:558-559 and
+    open_instruct/dpo_utils.py:859-863).  Raises ``TypeError`` when the model does not expose them
+    or projects with a bias."""
+    head = model.get_output_embeddings() if hasattr(model, "get_output_embeddings") else getattr(model, "lm_head", None)
+    trunk = getattr(model, "base_model", None)
+    if trunk is None or trunk is model:
+        trunk = getattr(model, "model", None)
+    if head is None or trunk is None or not hasattr(head, "weight"):
+        raise TypeError("fused_head needs a causal LM with a trunk (base_model / model) and an output embedding")
+    if getattr(head, "bias", None) is not None:
+        raise TypeError("fused_head needs a bias-free lm_head")
+    return trunk, head.weight
+
+
+def per_token_logps_from_trunk(model, labels: torch.Tensor, ignore_index: int = -100, **inputs) -> torch.Tensor:
+    """``calculate_per_token_logps(model(**inputs).logits, labels)``
+    (open_instruct/padding_free_collator.py:10-16) without the logits: the trunk's final hidden
+    states go through the fused head.  Positions whose next label is ``ignore_index`` are not
+    multiplied and hold 0 (the per-sequence sums mask them anyway)."""
+    trunk, weight = split_causal_lm(model)
+    out = trunk(**inputs)
+    hidden = getattr(out, "last_hidden_state", out[0] if isinstance(out, (tuple, list)) else out)
+    shifted = torch.full_like(labels, ignore_index)
+    shifted[..., :-1] = labels[..., 1:]
+    logps, _ = fused_lm_head_logprobs(hidden, weight, shifted, mask=shifted != ignore_index)
+    return logps

@@ -516,3 +516,116 @@ def test_entry_points_replay_from_a_hip_graph():
         torch.cuda.synchronize()
         assert torch.equal(got[0], e_small), i
         assert torch.equal(got[1], e_loss) and torch.equal(got[2], e_dh) and torch.equal(got[3], e_dw), i
+
+
+class _TinyCausalLM(torch.nn.Module):
+    """HuggingFace-shaped stand-in: ``base_model`` returns ``last_hidden_state``, ``get_output_embeddings``
+    the bias-free lm_head, the model itself ``.logits`` (and ``.aux_loss``)."""
+
+    class _Out:
+        def __init__(self, **kw):
+            self.__dict__.update(kw)
+
+    class _Trunk(torch.nn.Module):
+        def __init__(self, vocab, hidden):
+            super().__init__()
+            self.embed = torch.nn.Embedding(vocab, hidden, dtype=torch.bfloat16)
+            self.mix = torch.nn.Linear(hidden, hidden, bias=False, dtype=torch.bfloat16)
+
+        def forward(self, input_ids, attention_mask=None, position_ids=None):
+            h = self.embed(input_ids)
+            h = h + torch.tanh(self.mix(h)) + (0.01 * position_ids.unsqueeze(-1).to(h.dtype) if position_ids is not None else 0)
+            return _TinyCausalLM._Out(last_hidden_state=h)
+
+    def __init__(self, vocab=300, hidden=64):
+        super().__init__()
+        self.model = self._Trunk(vocab, hidden)
+        self.lm_head = torch.nn.Linear(hidden, vocab, bias=False, dtype=torch.bfloat16)
+
+    @property
+    def base_model(self):
+        return self.model
+
+    def get_output_embeddings(self):
+        return self.lm_head
+
+    def forward(self, input_ids, attention_mask=None, position_ids=None, output_router_logits=False):
+        h = self.model(input_ids, attention_mask, position_ids).last_hidden_state
+        return self._Out(logits=self.lm_head(h), aux_loss=None)
+
+
+def test_fused_head_option_of_the_huggingface_call_paths():
+    """``fused_head=True`` in forward_for_logprobs (open_instruct/grpo_utils.py:541-574), concatenated_forward
+    and separate_forward (open_instruct/dpo_utils.py:826-956): trunk + fused lm_head instead of the model's
+    logits, against the default routes and against the oracle on the model's own (bf16) logits, values and
+    gradients of the trunk and of the lm_head weight."""
+    torch.manual_seed(31)
+    vocab, b, t = 300, 3, 17
+    model = _TinyCausalLM(vocab).to(DEV)
+    qr = torch.randint(1, vocab, (b, t), device=DEV)
+    qr[0, -4:] = 0  # padding
+    pos = torch.arange(t, device=DEV).unsqueeze(0).expand(b, -1)
+    att = (qr != 0).long()
+    resp = torch.zeros(b, t, dtype=torch.bool, device=DEV)
+    resp[:, 6:] = True
+    resp &= qr != 0
+
+    def grads():
+        out = [p.grad.float().clone() for p in model.parameters()]
+        model.zero_grad()
+        return out
+
+    # GRPO: logprob / entropy of the next token
+    lp_a, ent_a = grpo_utils.forward_for_logprobs(model, qr, att, pos, 0, 0.8, return_entropy=True)
+    w = torch.randn(b, t - 1, device=DEV) * resp[:, 1:]
+    (lp_a * w).sum().backward()
+    g_a = grads()
+    lp_b, ent_b = grpo_utils.forward_for_logprobs(
+        model, qr, att, pos, 0, 0.8, return_entropy=True, fused_head=True, response_mask=resp
+    )
+    (lp_b * w).sum().backward()
+    g_b = grads()
+    keep = resp[:, 1:]
+    with torch.no_grad():
+        logits = model(qr, att, pos).logits
+    e_lp, e_ent = o_grpo.forward_for_logprobs(logits.float().cpu(), qr.cpu(), 0, 0.8, True)
+    # the default route rounds the logits to bf16 (the model's output dtype), the fused head does not
+    assert (lp_a.detach().cpu() - e_lp).abs().max().item() <= 2e-3
+    assert ((lp_b.detach() - lp_a.detach()) * keep).abs().max().item() <= 3e-2
+    assert ((ent_b - ent_a) * keep).abs().max().item() <= 3e-2
+    assert (lp_b[~keep] == 0).all() and (ent_b[~keep] == 0).all()
+    for x, y in zip(g_a, g_b):
+        assert (x - y).abs().max().item() <= 2e-2 * max(1e-3, x.abs().max().item())
+    # fp32 check of the fused route against the same trunk output multiplied in fp32
+    with torch.no_grad():
+        h = model.base_model(qr, att, pos).last_hidden_state[:, :-1].float()
+        z = (h @ model.lm_head.weight.float().T) / 0.8
+        labels = qr[:, 1:].clone()
+        ref = torch.log_softmax(z, -1).gather(-1, labels[..., None])[..., 0]
+    assert ((lp_b.detach() - ref) * keep).abs().max().item() <= 2e-3
+
+    # DPO: per-sequence logps, two forwards or one
+    batch = {
+        "chosen_input_ids": torch.randint(1, vocab, (2, 12), device=DEV), "rejected_input_ids": torch.randint(1, vocab, (2, 9), device=DEV),
+        "chosen_attention_mask": torch.ones(2, 12, dtype=torch.long, device=DEV),
+        "rejected_attention_mask": torch.ones(2, 9, dtype=torch.long, device=DEV),
+    }  # fmt: skip
+    batch["chosen_labels"] = batch["chosen_input_ids"].clone()
+    batch["rejected_labels"] = batch["rejected_input_ids"].clone()
+    batch["chosen_labels"][:, :4] = -100
+    batch["rejected_labels"][:, :3] = -100
+    for fn in (dpo_utils.concatenated_forward, dpo_utils.separate_forward):
+        c0, r0, _ = fn(model, batch)
+        (c0.sum() - r0.sum()).backward()
+        g0 = grads()
+        c1, r1, aux = fn(model, batch, fused_head=True)
+        (c1.sum() - r1.sum()).backward()
+        g1 = grads()
+        assert aux is None and c1.requires_grad
+        assert (c0 - c1).abs().max().item() <= 0.1 and (r0 - r1).abs().max().item() <= 0.1  # bf16 logits on one side
+        for x, y in zip(g0, g1):
+            assert (x - y).abs().max().item() <= 2e-2 * max(1e-3, x.abs().max().item())
+        with pytest.raises(ValueError):
+            fn(model, batch, output_router_logits=True, fused_head=True)
+    with pytest.raises(TypeError):
+        grpo_utils.forward_for_logprobs(torch.nn.Linear(4, 4), qr, att, pos, 0, 1.0, fused_head=True)
