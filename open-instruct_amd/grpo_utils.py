@@ -559,7 +559,7 @@ def grpo_loss_on_hidden(
     loss_denominator: float | None = None,
     axis: int | None = None,
     dp_scale: float = 1.0,
-    logit_cache_chunks: int = 0,
+    logit_cache_chunks: int | str = 0,
 ) -> tuple[torch.Tensor, dict[str, torch.Tensor], torch.Tensor, torch.Tensor]:
     """GRPO loss straight from final hidden states; returns ``(loss, stats, logprobs, entropy)``.
 
@@ -617,7 +617,9 @@ def grpo_loss_on_hidden(
     d_hidden = torch.empty_like(hid)
     d_weight = torch.empty_like(w) if weight.requires_grad else None
     lib = _lib.load()
-    cache_chunks = max(0, int(logit_cache_chunks))
+    from . import lm_head
+
+    cache_chunks = lm_head.resolve_cache_chunks(logit_cache_chunks, rows * cols, v, dev) if rows * cols > 0 else 0
     cache = None
     if cache_chunks:
         cache = torch.empty(lib.oi_lmhead_cache_bytes(rows * cols, v, cache_chunks), dtype=torch.uint8, device=dev)

@@ -17,6 +17,26 @@ import torch
 from . import _lib
 
 
+# share of the free device memory that ``logit_cache_chunks="auto"`` may take for the cache of exponentials
+AUTO_CACHE_MEMORY_SHARE = 0.25
+
+
+def resolve_cache_chunks(logit_cache_chunks, n_tokens: int, vocab: int, device) -> int:
+    """Number of vocabulary chunks to cache.  An integer is taken as it is; ``"auto"`` takes as many
+    chunks as fit into a quarter of the device memory that is free right now (2 bytes per cached
+    logit), which on a 288 GB part is all of them for any batch the path is used with."""
+    if logit_cache_chunks != "auto":
+        return max(0, int(logit_cache_chunks))
+    lib = _lib.load()
+    n_chunks = -(-int(vocab) // 32768)
+    free, _total = torch.cuda.mem_get_info(device)
+    budget = int(free * AUTO_CACHE_MEMORY_SHARE)
+    chunks = n_chunks
+    while chunks > 0 and lib.oi_lmhead_cache_bytes(n_tokens, vocab, chunks) > budget:
+        chunks -= 1
+    return chunks
+
+
 class _FusedLMHead(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, weight, labels, mask, inv_temperature, want_entropy, compact_backward=False,
@@ -43,7 +63,8 @@ class _FusedLMHead(torch.autograd.Function):
         entropy = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
         lse = torch.empty(n, dtype=torch.float32, device=dev)
         # the cache of exponentials only pays for itself when a backward pass follows
-        cache_chunks = int(cache_chunks) if (ctx.needs_input_grad[0] or ctx.needs_input_grad[1]) else 0
+        wants_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        cache_chunks = resolve_cache_chunks(cache_chunks, n, v, dev) if wants_grad and n > 0 else 0
         if cache_chunks and compact_backward:
             raise ValueError("compact_backward re-selects rows in the backward pass; it cannot be combined with a cache")
         cache = None
@@ -102,7 +123,7 @@ def fused_lm_head_logprobs(
     mask: torch.Tensor | None = None,
     return_entropy: bool = False,
     compact_backward: bool = False,
-    logit_cache_chunks: int = 0,
+    logit_cache_chunks: int | str = 0,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """``log_softmax(hidden @ weight.T / temperature)[labels]`` (+ entropy) per token, fp32.
 
@@ -122,6 +143,7 @@ def fused_lm_head_logprobs(
     keeps ``2^(logit / temperature * log2 e)`` in bf16 for the first so many chunks of 32768 vocabulary
     columns (2 bytes per cached logit, held until the backward pass) and the backward multiplies
     the cache directly.  With every chunk cached a quarter of the step's matrix work goes away.
+    ``"auto"`` caches as many chunks as fit into a quarter of the free device memory.
     """
     lead = hidden.shape[:-1]
     hid2 = hidden.reshape(-1, hidden.shape[-1])

@@ -9,7 +9,7 @@ import math
 import pytest
 import torch
 
-from open_instruct_amd import lm_head
+from open_instruct_amd import _lib, lm_head
 from open_instruct_amd.olmo_core_train_modules import DPOLMHead
 from oracle import lm_head as o_lm
 from oracle import logprob as o_logprob
@@ -377,3 +377,34 @@ def test_cache_of_exponentials_confident_tokens_and_no_grad():
     assert torch.equal(lp2, lp.detach())
     with pytest.raises(ValueError, match="compact_backward"):
         lm_head.fused_lm_head_logprobs(dh, weight.to(DEV), labels.to(DEV), compact_backward=True, logit_cache_chunks=1)
+
+
+def test_cache_chunks_auto_takes_what_fits(monkeypatch):
+    """``logit_cache_chunks="auto"``: as many chunks as fit into the allowed share of the free device
+    memory - all of them on an empty GPU (bitwise the same gradients as an explicit count), none when the
+    share is made tiny (bitwise the recomputing path)."""
+    n, h, v = 130, 64, 70000  # three vocabulary chunks
+    hidden, weight, labels = _case(n, h, v, seed=41, w_scale=3.0 / math.sqrt(h))
+    upstream = torch.randn(n, generator=torch.Generator().manual_seed(42))
+
+    def run(cache_chunks):
+        dh = hidden.to(DEV).requires_grad_(True)
+        dw = weight.to(DEV).requires_grad_(True)
+        lp, _ = lm_head.fused_lm_head_logprobs(dh, dw, labels.to(DEV), logit_cache_chunks=cache_chunks)
+        lp.backward(upstream.to(DEV))
+        return dh.grad, dw.grad
+
+    assert lm_head.resolve_cache_chunks("auto", n, v, torch.device(DEV)) == 3
+    assert lm_head.resolve_cache_chunks(2, n, v, torch.device(DEV)) == 2
+    auto, full, none = run("auto"), run(3), run(0)
+    assert torch.equal(auto[0], full[0]) and torch.equal(auto[1], full[1])
+    assert not torch.equal(auto[0], none[0])
+    monkeypatch.setattr(lm_head, "AUTO_CACHE_MEMORY_SHARE", 1e-9)
+    assert lm_head.resolve_cache_chunks("auto", n, v, torch.device(DEV)) == 0
+    tiny = run("auto")
+    assert torch.equal(tiny[0], none[0]) and torch.equal(tiny[1], none[1])
+    # a share that holds one chunk of this shape but not two
+    one_chunk = _lib.load().oi_lmhead_cache_bytes(n, v, 1)
+    free, _ = torch.cuda.mem_get_info(torch.device(DEV))
+    monkeypatch.setattr(lm_head, "AUTO_CACHE_MEMORY_SHARE", 1.5 * one_chunk / free)
+    assert lm_head.resolve_cache_chunks("auto", n, v, torch.device(DEV)) == 1
