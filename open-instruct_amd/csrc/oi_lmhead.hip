@@ -64,9 +64,13 @@ __host__ __device__ inline int64_t pids_for_tiles(int64_t tiles_m, int64_t tiles
 // no second one) that stays for the whole launch and draws tile ids from a counter, rather than
 // one short-lived workgroup per tile.  There is one counter per XCD (workgroup b is taken to run
 // on XCD b mod 8, as the tile order assumes), so the ids an XCD draws are the ones tile_of_pid
-// maps onto shared operand slabs; a wrong guess costs cache hits, never correctness.  The next id
-// is requested before the current tile is computed and handed to the other waves through one LDS
-// word afterwards.  `counters` are 8 zeroed words.
+// maps onto shared operand slabs; a wrong guess costs cache hits, never correctness.  The XCDs do
+// not finish their shares together (measured on the forward: 1.7 ms apart in an 18 ms launch), so
+// a workgroup whose own queue has run dry goes on with the queues of the other XCDs, one after the
+// other: the launch then ends within one work item for all of them.  The next id is requested
+// before the current tile is computed and handed to the other waves through one LDS word
+// afterwards.  `counters` are 8 zeroed words; every workgroup leaves each of them raised past the
+// number of ids at most once.
 constexpr int QUEUE_WORDS = 8;
 // threadIdx.x as a value the optimiser cannot trace: everything derived from it (fragment and
 // epilogue addresses) is then recomputed per tile instead of being hoisted out of the tile loop,
@@ -80,24 +84,35 @@ template <class Body>
 __device__ __forceinline__ void for_each_tile(uint32_t* __restrict__ counters, int64_t tiles_m, int64_t tiles_n,
                                               uint16_t* lds, Body&& body) {
     const uint32_t xcd = blockIdx.x & 7;
-    const uint32_t locals = (uint32_t)(pids_for_tiles(tiles_m, tiles_n) >> 3);
+    const uint32_t locals = (uint32_t)(pids_for_tiles(tiles_m, tiles_n) >> 3);  // ids per queue
     // the word sits in the fifth ring slot, which the main loop first writes after its first barrier
     volatile uint32_t* mailbox = reinterpret_cast<volatile uint32_t*>(lds + 4 * BM * BK);
-    uint32_t fetched = 0;
+    constexpr uint32_t NONE = 0xffffffffu;
+    // thread 0 only: the queues of XCDs xcd .. xcd + dry - 1 (mod 8) are known to be empty and
+    // `drawn` came from the queue of XCD xcd + dry
+    uint32_t dry = 0, drawn = 0;
+    auto resolve = [&]() -> uint32_t {
+        for (;;) {
+            if (drawn < locals) return drawn * 8 + ((xcd + dry) & 7);
+            if (++dry == 8) return NONE;
+            drawn = atomicAdd(&counters[(xcd + dry) & 7], 1u);
+        }
+    };
     if (threadIdx.x == 0) {
-        fetched = atomicAdd(&counters[xcd], 1u);
-        *mailbox = fetched;
+        drawn = atomicAdd(&counters[xcd], 1u);
+        *mailbox = resolve();
     }
     __syncthreads();
-    uint32_t local = __builtin_amdgcn_readfirstlane(*mailbox);
-    while (local < locals) {
-        if (threadIdx.x == 0) fetched = atomicAdd(&counters[xcd], 1u);  // in flight while the tile is computed
+    uint32_t pid = __builtin_amdgcn_readfirstlane(*mailbox);
+    while (pid != NONE) {
+        // in flight while the tile is computed
+        if (threadIdx.x == 0 && dry < 8) drawn = atomicAdd(&counters[(xcd + dry) & 7], 1u);
         int64_t tm, tn;
-        if (tile_of_pid((int64_t)local * 8 + xcd, tiles_m, tiles_n, &tm, &tn)) body(tm, tn);
+        if (tile_of_pid((int64_t)pid, tiles_m, tiles_n, &tm, &tn)) body(tm, tn);
         __syncthreads();  // the tile's last use of the LDS is over
-        if (threadIdx.x == 0) *mailbox = fetched;
+        if (threadIdx.x == 0) *mailbox = dry < 8 ? resolve() : NONE;
         __syncthreads();
-        local = __builtin_amdgcn_readfirstlane(*mailbox);
+        pid = __builtin_amdgcn_readfirstlane(*mailbox);
     }
 }
 // fallback used by the stand-alone GEMM entry point, which has no workspace for a counter: one
@@ -521,13 +536,15 @@ __device__ __forceinline__ void copy_staged_tile(const uint16_t* stage, uint16_t
 template <bool CACHE>
 __device__ __forceinline__ void lmhead_fwd_item(const uint16_t* __restrict__ W, const uint16_t* __restrict__ hidden,
                                                 const int64_t* __restrict__ labels, int64_t n_tokens, int64_t hdim,
-                                                int64_t vocab, float c, int64_t tiles_per_split, int64_t n_pad,
-                                                float4* __restrict__ partial, float* __restrict__ zy, int64_t split,
+                                                int64_t vocab, float c, int64_t tiles_per_split, int64_t long_splits,
+                                                int64_t n_pad, float4* __restrict__ partial, float* __restrict__ zy, int64_t split,
                                                 int64_t tt, uint16_t* __restrict__ ecache, int64_t cache_ld,
                                                 int64_t cache_tiles, uint16_t* lds) {
     const int64_t vocab_tiles = (vocab + BM - 1) / BM;
-    const int64_t vt_begin = split * tiles_per_split;
-    int64_t vt_end = vt_begin + tiles_per_split;
+    // the first long_splits splits take tiles_per_split vocabulary tiles each, the others one
+    const bool long_item = split < long_splits;
+    const int64_t vt_begin = long_item ? split * tiles_per_split : long_splits * tiles_per_split + (split - long_splits);
+    int64_t vt_end = vt_begin + (long_item ? tiles_per_split : 1);
     vt_end = vt_end < vocab_tiles ? vt_end : vocab_tiles;
 
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6, wm = wave & 3, wn = wave >> 2;
@@ -617,15 +634,15 @@ template <bool CACHE>
 __global__ void __launch_bounds__(NTHREADS)
     lmhead_fwd_kernel(const uint16_t* __restrict__ W, const uint16_t* __restrict__ hidden,
                       const int64_t* __restrict__ labels, int64_t n_tokens, const int32_t* __restrict__ n_dev,
-                      int64_t hdim, int64_t vocab, float c, int64_t n_splits, int64_t tiles_per_split, int64_t n_pad,
-                      float4* __restrict__ partial, float* __restrict__ zy, uint16_t* __restrict__ ecache,
+                      int64_t hdim, int64_t vocab, float c, int64_t n_splits, int64_t tiles_per_split,
+                      int64_t long_splits, int64_t n_pad, float4* __restrict__ partial, float* __restrict__ zy, uint16_t* __restrict__ ecache,
                       int64_t cache_ld, int64_t cache_tiles, uint32_t* __restrict__ queue) {
     __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
     if (n_dev) n_tokens = *n_dev;  // rows selected on the device: the host only knows an upper bound
     const int64_t token_tiles = (n_tokens + BN - 1) / BN;
     for_each_tile(queue, n_splits, token_tiles, lds, [&](int64_t split, int64_t tt) {
-        lmhead_fwd_item<CACHE>(W, hidden, labels, n_tokens, hdim, vocab, c, tiles_per_split, n_pad, partial, zy, split,
-                               tt, ecache, cache_ld, cache_tiles, lds);
+        lmhead_fwd_item<CACHE>(W, hidden, labels, n_tokens, hdim, vocab, c, tiles_per_split, long_splits, n_pad, partial,
+                               zy, split, tt, ecache, cache_ld, cache_tiles, lds);
     });
 }
 
@@ -1081,7 +1098,7 @@ CachePlan plan_cache(int64_t n_tokens, int64_t vocab, int64_t cache_chunks) {
 }
 
 struct FwdPlan {
-    int64_t token_tiles, vocab_tiles, n_splits, tiles_per_split, n_pad;
+    int64_t token_tiles, vocab_tiles, n_splits, tiles_per_split, long_splits, n_pad;
     size_t off_partial, off_zy, off_queue, total;
     SelectionPlan sel;
 };
@@ -1090,14 +1107,18 @@ FwdPlan plan_fwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_select
     p.token_tiles = (n_tokens + BN - 1) / BN;
     p.vocab_tiles = (vocab + BM - 1) / BM;
     p.n_pad = p.token_tiles * BN;
-    // Work items of 4 vocabulary tiles: the CUs finish the launch up to one work item apart, so the
-    // item is kept short (8 tiles measured 1.6 % slower, 2 tiles no faster: every item also writes
-    // and later merges a set of partial statistics).  Fewer tiles per split only when the problem
-    // is too small to give every CU work otherwise.
+    // Work items of 4 vocabulary tiles (8 tiles measured 1.6 % slower, 2 tiles no faster: every
+    // item also writes and later merges a set of partial statistics).  Fewer tiles per split only
+    // when the problem is too small to give every CU work otherwise.
     int64_t tps = 4;
     while (tps > 1 && ((p.vocab_tiles + tps - 1) / tps) * p.token_tiles < 512) tps /= 2;
     p.tiles_per_split = tps;
-    p.n_splits = (p.vocab_tiles + p.tiles_per_split - 1) / p.tiles_per_split;
+    // The ids are handed out with the vocabulary split as the slow index, so the last splits are
+    // the last work of the launch: they are single tiles, about four per CU, which the workgroups
+    // that run out of long items pick up (the launch then ends within one tile, not one item).
+    const int64_t short_wanted = (4 * 256 + p.token_tiles - 1) / p.token_tiles;
+    p.long_splits = tps > 1 && p.vocab_tiles > short_wanted ? (p.vocab_tiles - short_wanted) / tps : 0;
+    p.n_splits = p.long_splits + (p.vocab_tiles - p.long_splits * tps);
     Carver cv;
     p.off_partial = cv.take((size_t)p.n_splits * p.n_pad * sizeof(float4));
     p.off_zy = cv.take((size_t)p.n_pad * sizeof(float));
@@ -1207,11 +1228,11 @@ void enqueue_fwd(const FwdPlan& p, char* ws, const RowInputs& in, const uint8_t*
     const uint16_t* Wp = static_cast<const uint16_t*>(weight);
     if (cache.chunks > 0)
         hipLaunchKernelGGL(lmhead_fwd_kernel<true>, grid, dim3(NTHREADS), 0, s, Wp, in.hidden, in.labels, n_tokens,
-                           in.n_dev, hidden_dim, vocab, c, p.n_splits, p.tiles_per_split, p.n_pad, partial, zy, ecache,
-                           cache.ld, cache.tiles, queue);
+                           in.n_dev, hidden_dim, vocab, c, p.n_splits, p.tiles_per_split, p.long_splits, p.n_pad, partial, zy,
+                           ecache, cache.ld, cache.tiles, queue);
     else
         hipLaunchKernelGGL(lmhead_fwd_kernel<false>, grid, dim3(NTHREADS), 0, s, Wp, in.hidden, in.labels, n_tokens,
-                           in.n_dev, hidden_dim, vocab, c, p.n_splits, p.tiles_per_split, p.n_pad, partial, zy,
+                           in.n_dev, hidden_dim, vocab, c, p.n_splits, p.tiles_per_split, p.long_splits, p.n_pad, partial, zy,
                            static_cast<uint16_t*>(nullptr), (int64_t)0, (int64_t)0, queue);
     hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
                        zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, logprob,
