@@ -72,6 +72,7 @@ __host__ __device__ inline int64_t pids_for_tiles(int64_t tiles_m, int64_t tiles
 // afterwards.  `counters` are 8 zeroed words; every workgroup leaves each of them raised past the
 // number of ids at most once.
 constexpr int QUEUE_WORDS = 8;
+constexpr int FWD_QUEUE_WORDS = 2 * QUEUE_WORDS;  // the forward hands out its long and its short items from two sets of queues
 // threadIdx.x as a value the optimiser cannot trace: everything derived from it (fragment and
 // epilogue addresses) is then recomputed per tile instead of being hoisted out of the tile loop,
 // where it would stay live through the main loop and push accumulators into scratch
@@ -640,9 +641,15 @@ __global__ void __launch_bounds__(NTHREADS)
     __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
     if (n_dev) n_tokens = *n_dev;  // rows selected on the device: the host only knows an upper bound
     const int64_t token_tiles = (n_tokens + BN - 1) / BN;
-    for_each_tile(queue, n_splits, token_tiles, lds, [&](int64_t split, int64_t tt) {
+    // every long item of every XCD's queue is taken before the first short one: the short items are
+    // there to fill the end of the launch
+    for_each_tile(queue, long_splits, token_tiles, lds, [&](int64_t split, int64_t tt) {
         lmhead_fwd_item<CACHE>(W, hidden, labels, n_tokens, hdim, vocab, c, tiles_per_split, long_splits, n_pad, partial,
                                zy, split, tt, ecache, cache_ld, cache_tiles, lds);
+    });
+    for_each_tile(queue + QUEUE_WORDS, n_splits - long_splits, token_tiles, lds, [&](int64_t split, int64_t tt) {
+        lmhead_fwd_item<CACHE>(W, hidden, labels, n_tokens, hdim, vocab, c, tiles_per_split, long_splits, n_pad, partial,
+                               zy, long_splits + split, tt, ecache, cache_ld, cache_tiles, lds);
     });
 }
 
@@ -1117,12 +1124,14 @@ FwdPlan plan_fwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_select
     // the last work of the launch: they are single tiles, about four per CU, which the workgroups
     // that run out of long items pick up (the launch then ends within one tile, not one item).
     const int64_t short_wanted = (4 * 256 + p.token_tiles - 1) / p.token_tiles;
-    p.long_splits = tps > 1 && p.vocab_tiles > short_wanted ? (p.vocab_tiles - short_wanted) / tps : 0;
+    // whole groups of 8 long splits: the ids of a group of 8 splits are handed out together, and a
+    // long item among the last short ones would be the new ragged end
+    p.long_splits = tps > 1 && p.vocab_tiles > short_wanted ? (p.vocab_tiles - short_wanted) / tps / 8 * 8 : 0;
     p.n_splits = p.long_splits + (p.vocab_tiles - p.long_splits * tps);
     Carver cv;
     p.off_partial = cv.take((size_t)p.n_splits * p.n_pad * sizeof(float4));
     p.off_zy = cv.take((size_t)p.n_pad * sizeof(float));
-    p.off_queue = cv.take(QUEUE_WORDS * sizeof(uint32_t));
+    p.off_queue = cv.take(FWD_QUEUE_WORDS * sizeof(uint32_t));
     if (with_selection) p.sel = plan_selection(cv, p.n_pad, hdim, false);
     p.total = cv.off;
     return p;
@@ -1370,9 +1379,9 @@ extern "C" int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const 
     RowInputs in = {static_cast<const uint16_t*>(hidden), labels, nullptr, nullptr, nullptr, nullptr, nullptr};
     if (row_mask)
         in = launch_selection(p.sel, ws, hidden, labels, nullptr, nullptr, row_mask, false, n_tokens, hidden_dim, queue,
-                              QUEUE_WORDS, s);
+                              FWD_QUEUE_WORDS, s);
     else
-        hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, queue, QUEUE_WORDS);
+        hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, queue, FWD_QUEUE_WORDS);
     enqueue_fwd(p, ws, in, row_mask, weight, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy, lse,
                 static_cast<uint16_t*>(exp_cache), cache, s);
     return oi_launch_status();
@@ -1466,7 +1475,7 @@ extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, co
     uint32_t* bwd_queues = reinterpret_cast<uint32_t*>(ws_bwd + p.bwd.off_queues);
     const int n_queue_words = (int)(3 * p.bwd.n_chunks * QUEUE_WORDS);
     const bool select_clears_queues = n_queue_words <= SELECT_THREADS;
-    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, fwd_queue, QUEUE_WORDS);
+    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, fwd_queue, FWD_QUEUE_WORDS);
     if (!select_clears_queues)
         hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_queue_words + 255) / 256)), dim3(256), 0, s,
                            bwd_queues, n_queue_words);
