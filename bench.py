@@ -42,12 +42,12 @@ PEAK_BF16_TFLOPS = 2500.0
 # profiles/; workloads without a counter run report null.
 MEASURED_TRAFFIC_BYTES = {
     # lmhead_fwd_kernel: L2 misses of the tiled operand re-reads (1.24 GB of unique operands at c3) + the partials
-    "c3": 43.14e9 + 0.19e9,
-    "c4": 40.63e9 + 0.21e9,
-    "c5": 88.61e9 + 0.19e9,
+    "c3": 42.01e9 + 0.20e9,
+    "c4": 40.21e9 + 0.20e9,
+    "c5": 84.05e9 + 0.20e9,
     # lsg_grpo_fused_kernel: one read of the logits (the row waits on the CU for the gradient pass) + one write of
     # dlogits
-    "c2": 16.88e9 + 16.95e9,
+    "c2": 16.88e9 + 16.94e9,
     "c2-two-pass": 16.83e9 + 0.0e9,  # lsg_entropy_fwd_kernel: 1.00x the logits
 }
 
