@@ -396,6 +396,35 @@ int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* la
                        size_t workspace_bytes, void* stream);
 
 /*
+ * Forward + backward for callers that need d_hidden only (a frozen lm_head: the DPO / reward passes of
+ * open_instruct/dpo_utils.py:959-1019 through DPOLMHead when the head's weight takes no gradient, or
+ * any d_weight == NULL use of oi_lmhead_logp_bwd).  With x = z * inv_T * log2 e,
+ *   d_hidden[n] = s_n * sum_{v != label_n} 2^x[n,v] * weight[v]  -  g_n * inv_T * expm1(logprob_n) * weight[label_n],
+ *   s_n = -g_n * inv_T * 2^(-lse_n * log2 e),
+ * and the sum does not depend on the upstream gradient g: oi_lmhead_logp_fwd_wsum computes it together
+ * with logprob / entropy / lse while the logits exist (one chunk of 32768 vocabulary columns at a
+ * time: the chunk's exponentials as bf16 in the workspace, then wsum (+)= E_chunk @ weight_chunk in
+ * fp32), and oi_lmhead_dh_from_wsum turns it into d_hidden in one pass over [n_tokens, hidden_dim].
+ * Matrix work of forward + backward: 4 N H V instead of 6 N H V, nothing is recomputed, nothing of size
+ * [tokens, vocab] exists.  Needs |z * inv_T| < 87 like the cache of exponentials.
+ * wsum: fp32 [n_tokens, hidden_dim], 16-byte aligned, owned by the caller between the two calls; row j
+ * belongs to the j-th selected row (rows in ascending order; every row without a row_mask).  The
+ * backward call takes the same labels / row_mask and the forward's lse and logprob; rows left out
+ * get a zero d_hidden row.  d_hidden: bf16 [n_tokens, hidden_dim], 8-byte aligned.  The workspace of
+ * the backward call is only read with a row_mask (it may be NULL otherwise).
+ */
+size_t oi_lmhead_fwd_wsum_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int with_row_mask);
+int oi_lmhead_logp_fwd_wsum(const void* hidden, const void* weight, const int64_t* labels, const uint8_t* row_mask,
+                            int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob,
+                            float* entropy, float* lse, float* wsum, void* workspace, size_t workspace_bytes,
+                            void* stream);
+size_t oi_lmhead_dh_workspace_bytes(int64_t n_tokens);
+int oi_lmhead_dh_from_wsum(const void* weight, const int64_t* labels, const float* lse, const float* logprob,
+                           const float* grad_logprob, const uint8_t* row_mask, const float* wsum, int64_t n_tokens,
+                           int64_t hidden_dim, int64_t vocab, float inv_temperature, void* d_hidden, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/*
  * The whole GRPO step on hidden states in one call: fused lm_head forward (logprob, entropy),
  * scalar loss with its statistics, and the backward to d_hidden / d_weight, for an upstream
  * gradient of 1 on the loss.  It replaces, for a model that hands out its final hidden states, the

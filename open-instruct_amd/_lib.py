@@ -67,6 +67,10 @@ SIGNATURES: dict[str, tuple] = {
         _I,
         [_P, _P, _P, _P, _P, _P, _I, _I64, _I64, _I64, _F, _P, _P, _I64, _P, _P, _P, _SZ, _P],
     ),
+    "oi_lmhead_fwd_wsum_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I]),
+    "oi_lmhead_logp_fwd_wsum": (_I, [_P, _P, _P, _P, _I64, _I64, _I64, _F, _P, _P, _P, _P, _P, _SZ, _P]),
+    "oi_lmhead_dh_workspace_bytes": (_SZ, [_I64]),
+    "oi_lmhead_dh_from_wsum": (_I, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _F, _P, _P, _SZ, _P]),
     "oi_lmhead_grpo_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I64, _I64]),
     "oi_lmhead_grpo_fwd_bwd": (
         _I,

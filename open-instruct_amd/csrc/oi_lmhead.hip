@@ -534,13 +534,26 @@ __device__ __forceinline__ void copy_staged_tile(const uint16_t* stage, uint16_t
 // CACHE: the first cache_tiles vocabulary tiles also leave 2^(z c) behind as bf16, token-major
 // [n_pad, cache_ld] (bf16 has the exponent range of fp32, so no per-token reference is needed);
 // rows of tokens past the end are zero.
+// What a forward launch covers and where its exponentials go.  Splits [0, long_splits) take
+// tiles_per_split vocabulary tiles each, the others one.  A launch hands out the long splits
+// [first, first + n_first) from one set of queues and then the short splits
+// [long_splits, long_splits + n_second) from a second set.
+// The cache takes the vocabulary tiles [cache_tile0, cache_tile0 + cache_tiles) as columns from 0 on;
+// with skip_label the label's own entry is stored as 0 (the caller adds that term itself).
+struct FwdLaunch {
+    int64_t tiles_per_split, long_splits, first, n_first, n_second;
+    uint16_t* ecache;
+    int64_t cache_ld, cache_tile0, cache_tiles;
+    int skip_label;
+};
+
 template <bool CACHE>
 __device__ __forceinline__ void lmhead_fwd_item(const uint16_t* __restrict__ W, const uint16_t* __restrict__ hidden,
                                                 const int64_t* __restrict__ labels, int64_t n_tokens, int64_t hdim,
-                                                int64_t vocab, float c, int64_t tiles_per_split, int64_t long_splits,
-                                                int64_t n_pad, float4* __restrict__ partial, float* __restrict__ zy, int64_t split,
-                                                int64_t tt, uint16_t* __restrict__ ecache, int64_t cache_ld,
-                                                int64_t cache_tiles, uint16_t* lds) {
+                                                int64_t vocab, float c, const FwdLaunch& fl, int64_t n_pad,
+                                                float4* __restrict__ partial, float* __restrict__ zy, int64_t split,
+                                                int64_t tt, uint16_t* lds) {
+    const int64_t tiles_per_split = fl.tiles_per_split, long_splits = fl.long_splits;
     const int64_t vocab_tiles = (vocab + BM - 1) / BM;
     // the first long_splits splits take tiles_per_split vocabulary tiles each, the others one
     const bool long_item = split < long_splits;
@@ -573,32 +586,42 @@ __device__ __forceinline__ void lmhead_fwd_item(const uint16_t* __restrict__ W, 
         for (int j = 0; j < 4; ++j) {
             // the target logit, when its row falls into this wave's 64 rows
             const int rel = lab[j] - wave_row0;
+            // register of this lane that holds the label's row, -1 when another lane or wave does
+            int label_reg = -1;
             if (rel >= 0 && rel < 64) {
-                const int ri = rel >> 5, rr = rel & 31;
-                if (((rr >> 2) & 1) == (lane >> 5)) {
-                    const int reg = (rr >> 3) * 4 + (rr & 3);
-                    float v = 0.f;
+                const int rr = rel & 31;
+                if (((rr >> 2) & 1) == (lane >> 5)) label_reg = (rel >> 5) * 16 + (rr >> 3) * 4 + (rr & 3);
+            }
+            if (label_reg >= 0) {
+                float v = 0.f;
 #pragma unroll
-                    for (int i = 0; i < 2; ++i)
+                for (int i = 0; i < 2; ++i)
 #pragma unroll
-                        for (int r = 0; r < 16; ++r)
-                            if (i == ri && r == reg) v = acc[i][j][r];
-                    const int64_t n = n0 + acc_col(wn, j, lane);
-                    if (n < n_tokens) zy[n] = v;
-                }
+                    for (int r = 0; r < 16; ++r)
+                        if (i * 16 + r == label_reg) v = acc[i][j][r];
+                const int64_t n = n0 + acc_col(wn, j, lane);
+                if (n < n_tokens) zy[n] = v;
             }
             if (partial_tile)
                 stats_update<true, CACHE>(acc, j, wm, lane, m0, vocab, c, st_m[j], st_s[j], st_t[j]);
             else
                 stats_update<false, CACHE>(acc, j, wm, lane, m0, vocab, c, st_m[j], st_s[j], st_t[j]);
+            if (CACHE && fl.skip_label && label_reg >= 0) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (i * 16 + r == label_reg) acc[i][j][r] = 0.f;
+            }
         }
-        if (CACHE && vt < cache_tiles) {
+        if (CACHE && vt >= fl.cache_tile0 && vt < fl.cache_tile0 + fl.cache_tiles) {
             // the operand ring is free (the product ended with a barrier); the next tile's first loads
             // must wait until the image has been read out again
             stage_tile_bf16(acc, lds, wm, wn, lane);
             __syncthreads();
             const int64_t left = n_tokens - n0;
-            copy_staged_tile(lds, ecache + n0 * cache_ld + vt * BM, cache_ld, tid, (int)(left < BN ? left : BN));
+            copy_staged_tile(lds, fl.ecache + n0 * fl.cache_ld + (vt - fl.cache_tile0) * BM, fl.cache_ld, tid,
+                             (int)(left < BN ? left : BN));
             __syncthreads();
         }
     }
@@ -635,21 +658,20 @@ template <bool CACHE>
 __global__ void __launch_bounds__(NTHREADS)
     lmhead_fwd_kernel(const uint16_t* __restrict__ W, const uint16_t* __restrict__ hidden,
                       const int64_t* __restrict__ labels, int64_t n_tokens, const int32_t* __restrict__ n_dev,
-                      int64_t hdim, int64_t vocab, float c, int64_t n_splits, int64_t tiles_per_split,
-                      int64_t long_splits, int64_t n_pad, float4* __restrict__ partial, float* __restrict__ zy, uint16_t* __restrict__ ecache,
-                      int64_t cache_ld, int64_t cache_tiles, uint32_t* __restrict__ queue) {
+                      int64_t hdim, int64_t vocab, float c, FwdLaunch fl, int64_t n_pad, float4* __restrict__ partial,
+                      float* __restrict__ zy, uint32_t* __restrict__ queue) {
     __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
     if (n_dev) n_tokens = *n_dev;  // rows selected on the device: the host only knows an upper bound
     const int64_t token_tiles = (n_tokens + BN - 1) / BN;
     // every long item of every XCD's queue is taken before the first short one: the short items are
     // there to fill the end of the launch
-    for_each_tile(queue, long_splits, token_tiles, lds, [&](int64_t split, int64_t tt) {
-        lmhead_fwd_item<CACHE>(W, hidden, labels, n_tokens, hdim, vocab, c, tiles_per_split, long_splits, n_pad, partial,
-                               zy, split, tt, ecache, cache_ld, cache_tiles, lds);
+    for_each_tile(queue, fl.n_first, token_tiles, lds, [&](int64_t split, int64_t tt) {
+        lmhead_fwd_item<CACHE>(W, hidden, labels, n_tokens, hdim, vocab, c, fl, n_pad, partial, zy, fl.first + split, tt,
+                               lds);
     });
-    for_each_tile(queue + QUEUE_WORDS, n_splits - long_splits, token_tiles, lds, [&](int64_t split, int64_t tt) {
-        lmhead_fwd_item<CACHE>(W, hidden, labels, n_tokens, hdim, vocab, c, tiles_per_split, long_splits, n_pad, partial,
-                               zy, long_splits + split, tt, ecache, cache_ld, cache_tiles, lds);
+    for_each_tile(queue + QUEUE_WORDS, fl.n_second, token_tiles, lds, [&](int64_t split, int64_t tt) {
+        lmhead_fwd_item<CACHE>(W, hidden, labels, n_tokens, hdim, vocab, c, fl, n_pad, partial, zy,
+                               fl.long_splits + split, tt, lds);
     });
 }
 
@@ -1106,10 +1128,14 @@ CachePlan plan_cache(int64_t n_tokens, int64_t vocab, int64_t cache_chunks) {
 
 struct FwdPlan {
     int64_t token_tiles, vocab_tiles, n_splits, tiles_per_split, long_splits, n_pad;
-    size_t off_partial, off_zy, off_queue, total;
+    int64_t chunk, n_chunks;  // chunked flavour only
+    size_t off_partial, off_zy, off_queue, off_chunk, total;
     SelectionPlan sel;
 };
-FwdPlan plan_fwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_selection) {
+// `chunked`: the launch covers one backward-sized vocabulary chunk at a time (the forward that also
+// accumulates the weighted sum of weight rows): every split is a long one, so that a chunk is a whole
+// number of splits, and there is one set of queues per chunk for the forward and one for the product.
+FwdPlan plan_fwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_selection, bool chunked = false) {
     FwdPlan p;
     p.token_tiles = (n_tokens + BN - 1) / BN;
     p.vocab_tiles = (vocab + BM - 1) / BM;
@@ -1128,10 +1154,19 @@ FwdPlan plan_fwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_select
     // long item among the last short ones would be the new ragged end
     p.long_splits = tps > 1 && p.vocab_tiles > short_wanted ? (p.vocab_tiles - short_wanted) / tps / 8 * 8 : 0;
     p.n_splits = p.long_splits + (p.vocab_tiles - p.long_splits * tps);
+    p.chunk = p.n_chunks = 0;
+    if (chunked) {
+        p.n_splits = p.long_splits = (p.vocab_tiles + tps - 1) / tps;
+        const int64_t v_pad = p.vocab_tiles * BM;
+        p.chunk = v_pad < BWD_VOCAB_CHUNK ? v_pad : BWD_VOCAB_CHUNK;
+        p.n_chunks = (v_pad + p.chunk - 1) / p.chunk;
+    }
     Carver cv;
     p.off_partial = cv.take((size_t)p.n_splits * p.n_pad * sizeof(float4));
     p.off_zy = cv.take((size_t)p.n_pad * sizeof(float));
-    p.off_queue = cv.take(FWD_QUEUE_WORDS * sizeof(uint32_t));
+    p.off_queue = cv.take((chunked ? (size_t)p.n_chunks * (FWD_QUEUE_WORDS + QUEUE_WORDS) : (size_t)FWD_QUEUE_WORDS) *
+                          sizeof(uint32_t));
+    p.off_chunk = chunked ? cv.take((size_t)p.n_pad * p.chunk * 2) : 0;
     if (with_selection) p.sel = plan_selection(cv, p.n_pad, hdim, false);
     p.total = cv.off;
     return p;
@@ -1235,17 +1270,90 @@ void enqueue_fwd(const FwdPlan& p, char* ws, const RowInputs& in, const uint8_t*
     const float c = inv_temperature * OI_LOG2E;
     const dim3 grid(resident_grid(p.n_splits, p.token_tiles));
     const uint16_t* Wp = static_cast<const uint16_t*>(weight);
+    const FwdLaunch fl = {p.tiles_per_split, p.long_splits, 0,        p.long_splits, p.n_splits - p.long_splits,
+                          ecache,            cache.ld,      0,        cache.chunks > 0 ? cache.tiles : 0, 0};
     if (cache.chunks > 0)
         hipLaunchKernelGGL(lmhead_fwd_kernel<true>, grid, dim3(NTHREADS), 0, s, Wp, in.hidden, in.labels, n_tokens,
-                           in.n_dev, hidden_dim, vocab, c, p.n_splits, p.tiles_per_split, p.long_splits, p.n_pad, partial, zy,
-                           ecache, cache.ld, cache.tiles, queue);
+                           in.n_dev, hidden_dim, vocab, c, fl, p.n_pad, partial, zy, queue);
     else
         hipLaunchKernelGGL(lmhead_fwd_kernel<false>, grid, dim3(NTHREADS), 0, s, Wp, in.hidden, in.labels, n_tokens,
-                           in.n_dev, hidden_dim, vocab, c, p.n_splits, p.tiles_per_split, p.long_splits, p.n_pad, partial, zy,
-                           static_cast<uint16_t*>(nullptr), (int64_t)0, (int64_t)0, queue);
+                           in.n_dev, hidden_dim, vocab, c, fl, p.n_pad, partial, zy, queue);
     hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
                        zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, logprob,
                        entropy, lse);
+}
+
+// The forward that also prepares d_hidden.  With x = z c in the log2 domain,
+//   d_hidden[n] = sum_v dZ[n, v] W[v] = s_n sum_{v != y} 2^(x_nv) W[v] - g_n inv_T expm1(logprob_n) W[y_n],
+//   s_n = -g_n inv_T 2^(-lse2_n),
+// and the sum does not depend on the upstream gradient: it is accumulated while the logits exist,
+// one vocabulary chunk at a time (the exponentials of the chunk as bf16 in a chunk-sized buffer, as
+// for the cache of exponentials, with the label's own entry left out; then wsum (+)= E_chunk * W_chunk
+// in fp32).  A backward pass that only needs d_hidden is then one pass over [tokens, hidden]:
+// 4 N H V matrix work for forward + backward instead of 6 N H V, and nothing is recomputed.
+void enqueue_fwd_wsum(const FwdPlan& p, char* ws, const RowInputs& in, const uint8_t* row_mask, const void* weight,
+                      int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob,
+                      float* entropy, float* lse, float* wsum, hipStream_t s) {
+    float4* partial = reinterpret_cast<float4*>(ws + p.off_partial);
+    float* zy = reinterpret_cast<float*>(ws + p.off_zy);
+    uint32_t* queues = reinterpret_cast<uint32_t*>(ws + p.off_queue);
+    uint16_t* chunk_buf = reinterpret_cast<uint16_t*>(ws + p.off_chunk);
+    const float c = inv_temperature * OI_LOG2E;
+    const uint16_t* Wp = static_cast<const uint16_t*>(weight);
+    const int64_t h_tiles = (hidden_dim + BN - 1) / BN;
+    const int64_t v_pad = p.vocab_tiles * BM;
+    const int64_t splits_per_chunk = (p.chunk / BM + p.tiles_per_split - 1) / p.tiles_per_split;
+    for (int64_t ci = 0; ci < p.n_chunks; ++ci) {
+        const int64_t v_begin = ci * p.chunk;
+        const int64_t v_end = v_begin + p.chunk < v_pad ? v_begin + p.chunk : v_pad;
+        const int64_t cols = v_end - v_begin;                                   // multiple of 256
+        const int64_t valid = vocab - v_begin < cols ? vocab - v_begin : cols;  // real rows of W
+        const int64_t first = ci * splits_per_chunk;
+        const int64_t n_first = p.n_splits - first < splits_per_chunk ? p.n_splits - first : splits_per_chunk;
+        uint32_t* q = queues + ci * (FWD_QUEUE_WORDS + QUEUE_WORDS);
+        const FwdLaunch fl = {p.tiles_per_split, p.long_splits, first, n_first, 0, chunk_buf, cols, v_begin / BM, cols / BM, 1};
+        hipLaunchKernelGGL(lmhead_fwd_kernel<true>, dim3(resident_grid(n_first, p.token_tiles)), dim3(NTHREADS), 0, s, Wp,
+                           in.hidden, in.labels, n_tokens, in.n_dev, hidden_dim, vocab, c, fl, p.n_pad, partial, zy, q);
+        const Operand a = {chunk_buf, cols, 0, p.n_pad, cols};
+        const Operand b = {Wp + v_begin * hidden_dim, hidden_dim, 0, hidden_dim, valid};
+        const DynRows dyn = {in.n_dev, 1, nullptr, nullptr, nullptr};
+        hipLaunchKernelGGL((gemm_store_kernel<false, true>), dim3(resident_grid(p.n_pad / BM, h_tiles)), dim3(NTHREADS), 0,
+                           s, a, p.n_pad, b, hidden_dim, round_up(valid, BK), ci == 0 ? 0 : 1, wsum,
+                           static_cast<uint16_t*>(nullptr), hidden_dim, n_tokens, dyn, q + FWD_QUEUE_WORDS);
+    }
+    hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
+                       zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, logprob,
+                       entropy, lse);
+}
+
+// d_hidden row of selected token j (caller row rows[j], or j without a selection) from the weighted
+// sum that the forward left behind; one workgroup per selected row.  The factor s is applied in two
+// halves so that neither leaves the fp32 range.
+__global__ void __launch_bounds__(256)
+    dh_from_wsum_kernel(const float* __restrict__ wsum, const uint16_t* __restrict__ W,
+                        const int64_t* __restrict__ labels, const float* __restrict__ lse,
+                        const float* __restrict__ logprob, const float* __restrict__ grad,
+                        const int32_t* __restrict__ rows, const int32_t* __restrict__ count, int64_t n_tokens,
+                        int64_t hdim, int64_t vocab, float inv_t, uint16_t* __restrict__ d_hidden) {
+    const int64_t j = blockIdx.x;
+    if (j >= (count ? (int64_t)*count : n_tokens)) return;
+    const int64_t n = rows ? (int64_t)rows[j] : j;
+    const float g = grad[n] * inv_t;
+    const float half = __builtin_amdgcn_exp2f(-0.5f * lse[n] * OI_LOG2E);
+    const float sb = -g * half;
+    const float tl = -g * expm1f(logprob[n]);
+    int64_t y = labels[n];
+    y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
+    const float4* src = reinterpret_cast<const float4*>(wsum + j * hdim);
+    const uint2* wy = reinterpret_cast<const uint2*>(W + y * hdim);
+    uint2* dst = reinterpret_cast<uint2*>(d_hidden + n * hdim);
+    for (int64_t c = threadIdx.x; c < hdim / 4; c += blockDim.x) {  // hdim is a multiple of 64
+        const float4 o = src[c];
+        const uint2 w = wy[c];
+        const float r0 = o.x * half * sb + tl * oi_bf16lo_to_f32(w.x), r1 = o.y * half * sb + tl * oi_bf16hi_to_f32(w.x);
+        const float r2 = o.z * half * sb + tl * oi_bf16lo_to_f32(w.y), r3 = o.w * half * sb + tl * oi_bf16hi_to_f32(w.y);
+        dst[c] = make_uint2(oi_pack_bf16x2(r0, r1), oi_pack_bf16x2(r2, r3));
+    }
 }
 
 // backward launches.  Per vocabulary chunk: dZ [n_pad, cols] (token-major, bf16, zero in padded rows
@@ -1384,6 +1492,80 @@ extern "C" int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const 
         hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, queue, FWD_QUEUE_WORDS);
     enqueue_fwd(p, ws, in, row_mask, weight, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy, lse,
                 static_cast<uint16_t*>(exp_cache), cache, s);
+    return oi_launch_status();
+}
+
+extern "C" size_t oi_lmhead_fwd_wsum_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
+                                                     int with_row_mask) {
+    if (n_tokens <= 0 || vocab <= 0 || hidden_dim <= 0) return 0;
+    return plan_fwd(n_tokens, hidden_dim, vocab, with_row_mask != 0, true).total;
+}
+
+extern "C" int oi_lmhead_logp_fwd_wsum(const void* hidden, const void* weight, const int64_t* labels,
+                                       const uint8_t* row_mask, int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
+                                       float inv_temperature, float* logprob, float* entropy, float* lse, float* wsum,
+                                       void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
+    if (rc != OI_OK) return rc;
+    if (n_tokens == 0) return OI_OK;
+    OI_RETURN_IF(!logprob || !lse || !wsum || !workspace, OI_ENULL);
+    OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(wsum, 16), OI_EALIGN);
+    const FwdPlan p = plan_fwd(n_tokens, hidden_dim, vocab, row_mask != nullptr, true);
+    OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
+    char* ws = static_cast<char*>(workspace);
+    uint32_t* queues = reinterpret_cast<uint32_t*>(ws + p.off_queue);
+    const int n_queue_words = (int)(p.n_chunks * (FWD_QUEUE_WORDS + QUEUE_WORDS));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    RowInputs in = {static_cast<const uint16_t*>(hidden), labels, nullptr, nullptr, nullptr, nullptr, nullptr};
+    const bool select_clears_queues = row_mask && n_queue_words <= SELECT_THREADS;
+    if (!select_clears_queues)
+        hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_queue_words + 255) / 256)), dim3(256), 0, s, queues,
+                           n_queue_words);
+    if (row_mask)
+        in = launch_selection(p.sel, ws, hidden, labels, nullptr, nullptr, row_mask, false, n_tokens, hidden_dim, queues,
+                              select_clears_queues ? n_queue_words : 0, s);
+    enqueue_fwd_wsum(p, ws, in, row_mask, weight, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy, lse,
+                     wsum, s);
+    return oi_launch_status();
+}
+
+extern "C" size_t oi_lmhead_dh_workspace_bytes(int64_t n_tokens) {
+    if (n_tokens <= 0) return 0;
+    Carver cv;
+    cv.take((size_t)round_up(n_tokens, 256) * sizeof(int32_t));
+    cv.take(sizeof(int32_t));
+    return cv.off;
+}
+
+extern "C" int oi_lmhead_dh_from_wsum(const void* weight, const int64_t* labels, const float* lse, const float* logprob,
+                                      const float* grad_logprob, const uint8_t* row_mask, const float* wsum,
+                                      int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature,
+                                      void* d_hidden, void* workspace, size_t workspace_bytes, void* stream) {
+    OI_RETURN_IF(n_tokens < 0 || hidden_dim <= 0 || vocab <= 0 || hidden_dim % 64 != 0, OI_EINVAL);
+    OI_RETURN_IF(!(inv_temperature >= 1.0e-6f) || !(inv_temperature <= 1.0e6f), OI_EINVAL);
+    if (n_tokens == 0) return OI_OK;
+    OI_RETURN_IF(!weight || !labels || !lse || !logprob || !grad_logprob || !wsum || !d_hidden, OI_ENULL);
+    OI_RETURN_IF(!oi_aligned(weight, 16) || !oi_aligned(wsum, 16) || !oi_aligned(d_hidden, 8), OI_EALIGN);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int32_t *rows = nullptr, *count = nullptr;
+    if (row_mask) {
+        OI_RETURN_IF(!workspace, OI_ENULL);
+        OI_RETURN_IF(!oi_aligned(workspace, 256), OI_EALIGN);
+        OI_RETURN_IF(workspace_bytes < oi_lmhead_dh_workspace_bytes(n_tokens), OI_EWORKSPACE);
+        // the same ascending selection as in the forward pass, rebuilt from the same mask
+        char* ws = static_cast<char*>(workspace);
+        int32_t* r = reinterpret_cast<int32_t*>(ws);
+        int32_t* c = reinterpret_cast<int32_t*>(ws + (size_t)round_up(n_tokens, 256) * sizeof(int32_t));
+        hipLaunchKernelGGL(select_rows_kernel, dim3(1), dim3(SELECT_THREADS), 0, s, row_mask,
+                           static_cast<const float*>(nullptr), n_tokens, r, c, static_cast<uint32_t*>(nullptr), 0);
+        hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, row_mask,
+                           static_cast<const float*>(nullptr), hidden_dim, static_cast<uint16_t*>(d_hidden));
+        rows = r;
+        count = c;
+    }
+    hipLaunchKernelGGL(dh_from_wsum_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, wsum,
+                       static_cast<const uint16_t*>(weight), labels, lse, logprob, grad_logprob, rows, count, n_tokens,
+                       hidden_dim, vocab, inv_temperature, static_cast<uint16_t*>(d_hidden));
     return oi_launch_status();
 }
 

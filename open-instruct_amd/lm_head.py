@@ -40,7 +40,7 @@ def resolve_cache_chunks(logit_cache_chunks, n_tokens: int, vocab: int, device) 
 class _FusedLMHead(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, weight, labels, mask, inv_temperature, want_entropy, compact_backward=False,
-                cache_chunks=0):
+                cache_chunks=0, dhidden_in_forward="auto"):
         dev = _lib.require_gpu(hidden, weight, labels, mask)
         if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
             raise ValueError("fused lm_head expects bf16 hidden states and weight")
@@ -67,8 +67,24 @@ class _FusedLMHead(torch.autograd.Function):
         cache_chunks = resolve_cache_chunks(cache_chunks, n, v, dev) if wants_grad and n > 0 else 0
         if cache_chunks and compact_backward:
             raise ValueError("compact_backward re-selects rows in the backward pass; it cannot be combined with a cache")
-        cache = None
-        if n > 0:
+        # a backward pass that only needs d_hidden is prepared while the logits exist (no recomputation)
+        if dhidden_in_forward == "auto":
+            dhidden_in_forward = not cache_chunks and not compact_backward
+        wsum_mode = bool(dhidden_in_forward) and ctx.needs_input_grad[0] and not ctx.needs_input_grad[1] and n > 0
+        if wsum_mode and (cache_chunks or compact_backward):
+            raise ValueError("dhidden_in_forward cannot be combined with a cache of exponentials or compact_backward")
+        cache = wsum = None
+        if wsum_mode:
+            lib = _lib.load()
+            wsum = torch.empty(n, h, dtype=torch.float32, device=dev)
+            ws_bytes = lib.oi_lmhead_fwd_wsum_workspace_bytes(n, h, v, int(m is not None))
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            _lib.call(
+                "oi_lmhead_logp_fwd_wsum", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), _lib.ptr(m), n, h, v,
+                inv_temperature, logprob.data_ptr(), _lib.ptr(entropy), lse.data_ptr(), wsum.data_ptr(), ws.data_ptr(),
+                ws_bytes, _lib.stream_of(hid),
+            )  # fmt: skip
+        elif n > 0:
             lib = _lib.load()
             if cache_chunks > 0:
                 cache = torch.empty(lib.oi_lmhead_cache_bytes(n, v, cache_chunks), dtype=torch.uint8, device=dev)
@@ -79,7 +95,7 @@ class _FusedLMHead(torch.autograd.Function):
                 inv_temperature, logprob.data_ptr(), _lib.ptr(entropy), lse.data_ptr(), _lib.ptr(cache),
                 cache_chunks if cache is not None else 0, ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
             )  # fmt: skip
-        ctx.save_for_backward(hid, w, lab, lse, m, cache, logprob)
+        ctx.save_for_backward(hid, w, lab, lse, m, cache, logprob, wsum)
         ctx.inv_temperature = inv_temperature
         ctx.compact_backward = bool(compact_backward)
         ctx.cache_chunks = cache_chunks if cache is not None else 0
@@ -89,14 +105,23 @@ class _FusedLMHead(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_logprob, _grad_entropy):
-        hid, w, lab, lse, m, cache, logprob = ctx.saved_tensors
+        hid, w, lab, lse, m, cache, logprob, wsum = ctx.saved_tensors
         n, h = hid.shape
         v = w.shape[0]
         need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if grad_logprob is None or not (need_h or need_w):
-            return None, None, None, None, None, None, None, None
+            return (None,) * 9
         g = _lib.f32c(grad_logprob)
         d_hidden = torch.empty_like(hid)
+        if wsum is not None:
+            ws_bytes = _lib.load().oi_lmhead_dh_workspace_bytes(n) if m is not None else 0
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=hid.device) if ws_bytes else None
+            _lib.call(
+                "oi_lmhead_dh_from_wsum", w.data_ptr(), lab.data_ptr(), lse.data_ptr(), logprob.data_ptr(), g.data_ptr(),
+                _lib.ptr(m), wsum.data_ptr(), n, h, v, ctx.inv_temperature, d_hidden.data_ptr(), _lib.ptr(ws), ws_bytes,
+                _lib.stream_of(hid),
+            )  # fmt: skip
+            return (d_hidden,) + (None,) * 8
         d_weight = torch.empty_like(w) if need_w else None
         if n > 0:
             selecting = m is not None or ctx.compact_backward
@@ -112,7 +137,7 @@ class _FusedLMHead(torch.autograd.Function):
             )  # fmt: skip
         elif d_weight is not None:
             d_weight.zero_()
-        return (d_hidden if need_h else None), d_weight, None, None, None, None, None, None
+        return (d_hidden if need_h else None), d_weight, None, None, None, None, None, None, None
 
 
 def fused_lm_head_logprobs(
@@ -124,6 +149,7 @@ def fused_lm_head_logprobs(
     return_entropy: bool = False,
     compact_backward: bool = False,
     logit_cache_chunks: int | str = 0,
+    dhidden_in_forward: bool | str = "auto",
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """``log_softmax(hidden @ weight.T / temperature)[labels]`` (+ entropy) per token, fp32.
 
@@ -144,6 +170,13 @@ def fused_lm_head_logprobs(
     columns (2 bytes per cached logit, held until the backward pass) and the backward multiplies
     the cache directly.  With every chunk cached a quarter of the step's matrix work goes away.
     ``"auto"`` caches as many chunks as fit into a quarter of the free device memory.
+
+    ``dhidden_in_forward`` (default ``"auto"``: on whenever ``hidden`` takes a gradient and ``weight``
+    does not, e.g. a frozen lm_head) lets the forward also accumulate, per token, the
+    softmax-weighted sum of the weight rows, which is all the backward to ``hidden`` needs besides
+    the upstream gradient: the backward is then one pass over ``[tokens, hidden]`` and the logits
+    are never recomputed (4·N·H·V matrix work for both passes instead of 6·N·H·V).  It holds an
+    fp32 ``[tokens, hidden]`` tensor between the passes.
     """
     lead = hidden.shape[:-1]
     hid2 = hidden.reshape(-1, hidden.shape[-1])
@@ -153,7 +186,9 @@ def fused_lm_head_logprobs(
         raise ValueError(f"temperature must be positive, got {temperature}")
     if mask is not None and tuple(mask.shape) != tuple(lead):
         raise ValueError(f"mask {tuple(mask.shape)} does not match the rows of hidden {tuple(lead)}")
-    lp, ent = _FusedLMHead.apply(hid2, weight, lab1, mask, inv_t, return_entropy, compact_backward, logit_cache_chunks)
+    lp, ent = _FusedLMHead.apply(
+        hid2, weight, lab1, mask, inv_t, return_entropy, compact_backward, logit_cache_chunks, dhidden_in_forward
+    )
     return lp.reshape(lead), (ent.reshape(lead) if ent is not None else None)
 
 

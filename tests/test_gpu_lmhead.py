@@ -71,9 +71,12 @@ def test_forward_matches_oracle(n, h, v, temperature):
         (130, 192, 300),
     ],
 )
-@pytest.mark.parametrize("want_dw", [True, False])
-def test_backward_matches_oracle(n, h, v, want_dw):
-    print(f"case N={n} H={h} V={v} dW={want_dw}", flush=True)
+@pytest.mark.parametrize("route", ["d_weight", "d_hidden_recomputed", "d_hidden_in_forward"])
+def test_backward_matches_oracle(n, h, v, route):
+    """d_hidden and d_weight by recomputation, d_hidden alone by recomputation, and d_hidden alone
+    from the weighted sum of weight rows that the forward accumulates (the default without d_weight)."""
+    print(f"case N={n} H={h} V={v} route={route}", flush=True)
+    want_dw = route == "d_weight"
     hidden, weight, labels = _case(n, h, v, seed=1, w_scale=3.0 / math.sqrt(h))
     g = torch.Generator().manual_seed(2)
     upstream = torch.randn(n, generator=g)
@@ -84,7 +87,12 @@ def test_backward_matches_oracle(n, h, v, want_dw):
     lp.backward(upstream)
     dh = hidden.to(DEV).requires_grad_(True)
     dw = weight.to(DEV).requires_grad_(want_dw)
-    out, _ = lm_head.fused_lm_head_logprobs(dh, dw, labels.to(DEV), 0.9)
+    out, ent = lm_head.fused_lm_head_logprobs(
+        dh, dw, labels.to(DEV), 0.9, return_entropy=True, dhidden_in_forward=route == "d_hidden_in_forward"
+    )
+    assert (out.detach().cpu() - lp.detach()).abs().max().item() <= TOL
+    exp_ent = o_lm.lm_head_logprobs(hidden, weight, labels, 0.9, True)[1]
+    assert (ent.cpu() - exp_ent).abs().max().item() <= TOL
     out.backward(upstream.to(DEV))
     assert dh.grad.dtype == torch.bfloat16 and dh.grad.shape == hidden.shape
     # bf16 outputs: allow one bf16 rounding of the largest entry on top of the absolute tolerance
@@ -118,6 +126,61 @@ def test_mask_compaction_and_leading_shape():
     assert (lp.cpu()[~mask] == 0).all()
     lp.sum().backward()
     assert (dh.grad.cpu()[~mask] == 0).all() and dh.grad.cpu()[mask].abs().sum() > 0
+
+
+@pytest.mark.parametrize("n,h,v", [(300, 128, 1000), (520, 64, 40000)])
+def test_d_hidden_in_forward_with_mask_and_confident_tokens(n, h, v):
+    """The d_hidden-only route with a row mask (compact rows of the weighted sum, rebuilt selection in
+    the backward) and with tokens whose label has probability close to 1 (their gradient is the small
+    difference 1 - p: the label's term is evaluated from the fp32 logprob, not from bf16 exponentials)."""
+    print(f"case N={n} H={h} V={v}", flush=True)
+    hidden, weight, labels = _case(n, h, v, seed=11, w_scale=2.0 / math.sqrt(h))
+    # make every fifth token confident: its hidden row points along its label's weight row
+    for i in range(0, n, 5):
+        wy = weight[labels[i]].float()
+        hidden[i] = (wy * (math.log(300.0 * v) / wy.pow(2).sum())).bfloat16()  # p(label) around 0.97-0.99
+    g = torch.Generator().manual_seed(12)
+    mask = torch.rand(n, generator=g) > 0.35
+    upstream = torch.randn(n, generator=g)
+    rh = hidden.float().requires_grad_(True)
+    lp, _ = o_lm.lm_head_logprobs(rh, weight.float(), labels, 1.0)
+    (lp * mask).backward(upstream)
+    p_conf = lp.detach()[::5].exp()
+    assert 0.9 < p_conf.min().item() and p_conf.max().item() < 0.9999  # confident, and 1 - p still well inside fp32
+    for route in (True, False):
+        dh = hidden.to(DEV).requires_grad_(True)
+        out, _ = lm_head.fused_lm_head_logprobs(
+            dh, weight.to(DEV), labels.to(DEV), mask=mask.to(DEV), dhidden_in_forward=route
+        )
+        assert ((out.detach().cpu() - lp.detach()) * mask).abs().max().item() <= TOL
+        out.backward(upstream.to(DEV))
+        got = dh.grad.float().cpu()
+        assert (got[~mask] == 0).all()
+        tol = TOL + rh.grad.abs().max().item() * 2**-7
+        assert (got - rh.grad).abs().max().item() <= tol, route
+        # relative, per confident token: the small gradient itself must be right, not only small
+        conf = torch.arange(0, n, 5)
+        conf = conf[mask[conf]]
+        rel = (got[conf] - rh.grad[conf]).norm(dim=1) / rh.grad[conf].norm(dim=1).clamp(min=1e-12)
+        assert rel.max().item() <= 3e-2, (route, rel.max().item())
+
+
+def test_d_hidden_in_forward_is_the_default_without_d_weight():
+    hidden, weight, labels = _case(300, 64, 700, seed=13)
+    grads = {}
+    for route in ("auto", True, False):
+        dh = hidden.to(DEV).requires_grad_(True)
+        out, _ = lm_head.fused_lm_head_logprobs(dh, weight.to(DEV), labels.to(DEV), dhidden_in_forward=route)
+        out.sum().backward()
+        grads[route] = dh.grad.clone()
+    assert torch.equal(grads["auto"], grads[True])  # bit-equal: the same kernels ran
+    assert not torch.equal(grads[True], grads[False])  # the recomputing route rounds differently ...
+    assert (grads[True].float() - grads[False].float()).abs().max().item() <= TOL  # ... and agrees
+    with pytest.raises(ValueError):
+        lm_head.fused_lm_head_logprobs(
+            hidden.to(DEV).requires_grad_(True), weight.to(DEV), labels.to(DEV), dhidden_in_forward=True,
+            logit_cache_chunks=1,
+        )
 
 
 def test_dpo_lm_head_matches_calculate_per_token_logps():

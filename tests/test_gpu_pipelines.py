@@ -419,7 +419,10 @@ def test_grpo_loss_on_hidden_whole_step(loss_fn, axis, denominator, with_old, wa
     # the three-call chain of this package gives the same numbers
     dh2 = d(hidden).requires_grad_(True)
     dw2 = d(weight).requires_grad_(want_dw)
-    lp2, ent2 = lm_head.fused_lm_head_logprobs(dh2, dw2, d(labels), temperature, mask=d(mask), return_entropy=True)
+    # (the recomputing backward on both sides: the one-call entry has no other)
+    lp2, ent2 = lm_head.fused_lm_head_logprobs(
+        dh2, dw2, d(labels), temperature, mask=d(mask), return_entropy=True, dhidden_in_forward=False
+    )
     loss2, stats2 = grpo_utils.grpo_loss_fused(
         lp2, d(old) if with_old else None, d(ref), d(adv), d(mask), cfg, rho_weights=d(rho), entropy=ent2,
         loss_denominator=denominator, axis=axis, dp_scale=2.0,
