@@ -44,7 +44,8 @@ MEASURED_TRAFFIC_BYTES = {
     # lmhead_fwd_kernel: L2 misses of the tiled operand re-reads (1.24 GB of unique operands at c3) + the partials
     "c3": 42.01e9 + 0.20e9,
     "c4": 40.21e9 + 0.20e9,
-    "c5": 84.05e9 + 0.20e9,
+    # oi_lmhead_logp_fwd_wsum: four launches of lmhead_fwd_kernel<true> and four of gemm_store_kernel<false, true>
+    "c5": None,
     # lsg_grpo_fused_kernel: one read of the logits (the row waits on the CU for the gradient pass) + one write of
     # dlogits
     "c2": 16.88e9 + 16.94e9,
@@ -156,6 +157,14 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=Fals
     if one_call:
         info["kernel"] = "oi_lmhead_grpo_fwd_bwd (every launch of the step: forward, loss, dZ, dHidden, dW)"
         info["alg_per_launch"] = 3.0 * flops_fwd
+    if dpo and not cache_chunks:
+        # the weight takes no gradient: the forward call also accumulates the weighted sum of weight rows that
+        # the backward to hidden needs (per vocabulary chunk: statistics + exponentials, then E_chunk @ W_chunk)
+        info["kernel"] = (
+            "oi_lmhead_logp_fwd_wsum (per vocabulary chunk: lmhead_fwd_kernel<true> + gemm_store_kernel<false, true>; "
+            "all of the step's matrix work, nothing is recomputed)"
+        )
+        info["alg_per_launch"] = 2.0 * flops_fwd
     return step, info
 
 

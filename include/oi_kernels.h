@@ -402,7 +402,7 @@ int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* la
  *   d_hidden[n] = s_n * sum_{v != label_n} 2^x[n,v] * weight[v]  -  g_n * inv_T * expm1(logprob_n) * weight[label_n],
  *   s_n = -g_n * inv_T * 2^(-lse_n * log2 e),
  * and the sum does not depend on the upstream gradient g: oi_lmhead_logp_fwd_wsum computes it together
- * with logprob / entropy / lse while the logits exist (one chunk of 32768 vocabulary columns at a
+ * with logprob / entropy / lse while the logits exist (one chunk of 65536 vocabulary columns at a
  * time: the chunk's exponentials as bf16 in the workspace, then wsum (+)= E_chunk @ weight_chunk in
  * fp32), and oi_lmhead_dh_from_wsum turns it into d_hidden in one pass over [n_tokens, hidden_dim].
  * Matrix work of forward + backward: 4 N H V instead of 6 N H V, nothing is recomputed, nothing of size
