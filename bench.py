@@ -45,7 +45,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c3": 42.01e9 + 0.20e9,
     "c4": 40.21e9 + 0.20e9,
     # oi_lmhead_logp_fwd_wsum: four launches of lmhead_fwd_kernel<true> and four of gemm_store_kernel<false, true>
-    "c5": None,
+    "c5": 2 * (42.62e9 + 3.06e9) + 2 * (43.14e9 + 0.75e9),
     # lsg_grpo_fused_kernel: one read of the logits (the row waits on the CU for the gradient pass) + one write of
     # dlogits
     "c2": 16.88e9 + 16.94e9,
