@@ -84,7 +84,7 @@ class EventTimer:
 # ------------------------------------------------------------------------------------------------
 # workloads
 # ------------------------------------------------------------------------------------------------
-def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=False, cache_chunks=0):
+def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=False, cache_chunks=0, token_slabs=False):
     dev = "cuda:0"
     torch.manual_seed(0)
     hidden = torch.randn(n_tokens, hdim, device=dev).bfloat16().requires_grad_(True)
@@ -122,7 +122,7 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=Fals
             with fwd_timer:  # the whole step is one C call here: the timer brackets all of it
                 loss, _, _, _ = oi.grpo_utils.grpo_loss_on_hidden(
                     hidden[None], weight, labels[None], old[None], ref[None], adv[None], mask[None], cfg,
-                    logit_cache_chunks=cache_chunks,
+                    logit_cache_chunks=cache_chunks, token_slabs=token_slabs,
                 )
         elif not dpo:
             with fwd_timer:
@@ -157,6 +157,11 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=Fals
     if one_call:
         info["kernel"] = "oi_lmhead_grpo_fwd_bwd (every launch of the step: forward, loss, dZ, dHidden, dW)"
         info["alg_per_launch"] = 3.0 * flops_fwd
+        if token_slabs:
+            info["kernel"] = (
+                "oi_lmhead_grpo_fwd_bwd in slabs of 8192 selected tokens (per slab: forward with its exponentials kept, "
+                "loss gradient, dHidden, dW; nothing is recomputed)"
+            )
     if dpo and not cache_chunks:
         # the weight takes no gradient: the forward call also accumulates the weighted sum of weight rows that
         # the backward to hidden needs (per vocabulary chunk: statistics + exponentials, then E_chunk @ W_chunk)
@@ -495,7 +500,7 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="c3",
-                    choices=["c1", "c2", "c2-two-pass", "c3", "c3-one-call", "c4", "c5", "pack"])
+                    choices=["c1", "c2", "c2-two-pass", "c3", "c3-one-call", "c3-slabs", "c4", "c5", "pack"])
     ap.add_argument("--cache-chunks", type=int, default=0,
                     help="c3 / c3-one-call / c5 only: keep 2^logit in bf16 for this many vocabulary chunks of 32768 "
                          "columns instead of recomputing them in the backward pass (0 = the headline configuration: "
@@ -527,6 +532,11 @@ def main():
     elif args.workload == "c3-one-call":
         step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02, one_call=True, cache_chunks=args.cache_chunks)
         name = "c3: the same step through the single entry point grpo_loss_on_hidden (oi_lmhead_grpo_fwd_bwd)"
+        dtype = "bf16"
+    elif args.workload == "c3-slabs":
+        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02, one_call=True, token_slabs=True)
+        name = ("c3: the same step through grpo_loss_on_hidden(token_slabs=True): slabs of 8192 selected tokens, a slab's "
+                "exponentials [8192, vocab] bf16 kept between its forward and its backward products, nothing recomputed")
         dtype = "bf16"
     elif args.workload == "c4":
         step, info = make_c4(torch, oi)
@@ -652,6 +662,27 @@ def main():
             }
         }
         del step_c
+        torch.cuda.empty_cache()
+        # the same step in slabs of 8192 selected tokens through the one-call entry: a slab's exponentials are
+        # kept between its forward and its backward products ([8192, vocab] bf16 at a time), nothing is recomputed
+        step_s, info_s = make_fused(torch, oi, 32768, 4096, 128256, 0.02, one_call=True, token_slabs=True)
+        for _ in range(args.warmup):
+            step_s()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step_s()
+        torch.cuda.synchronize()
+        ms_s = (time.perf_counter() - t0) * 1e3 / args.steps
+        line["opt_in_variants"]["token_slabs_one_call"] = {
+            "ms_per_step": ms_s,
+            "tokens_per_s": info_s["tokens"] / (ms_s * 1e-3),
+            "whole_step_frac": info_s["flops_step"] / (ms_s * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            "extra_hbm_bytes": 8192 * 128256 * 2 + 128256 * 4096 * 4,
+            "note": "not the headline configuration: grpo_loss_on_hidden(token_slabs=True), no recomputation, no "
+                    "[tokens, vocab] tensor",
+        }
+        del step_s
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, args.workload)
     print(json.dumps(line), flush=True)

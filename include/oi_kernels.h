@@ -442,6 +442,13 @@ int oi_lmhead_dh_from_wsum(const void* weight, const int64_t* labels, const floa
  * the backward is enqueued straight behind the forward: nothing returns to the host in between.
  * exp_cache / cache_chunks: the optional cache of exponentials described at oi_lmhead_cache_bytes
  * (scratch of this one call here; NULL / 0 = recompute every chunk).
+ * cache_chunks < 0 (exp_cache ignored): the step runs in slabs of -cache_chunks * 4096 selected tokens and
+ * recomputes nothing.  A slab's forward leaves its exponentials (every vocabulary column, bf16) in a slab-sized
+ * buffer inside the workspace, the slab's tokens get their upstream gradient at once, and both
+ * products read the buffer before the next slab overwrites it: d_hidden rows are final, d_weight
+ * accumulates in fp32 over the slabs (deterministic: slab after slab) and is rounded to bf16 once.
+ * 6 N H V of matrix work instead of 8 N H V; the workspace holds [slab, vocab] bf16 and, with
+ * d_weight, an fp32 [vocab, hidden_dim], never anything of size [tokens, vocab].
  */
 size_t oi_lmhead_grpo_workspace_bytes(int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab,
                                       int64_t cache_chunks);

@@ -560,6 +560,7 @@ def grpo_loss_on_hidden(
     axis: int | None = None,
     dp_scale: float = 1.0,
     logit_cache_chunks: int | str = 0,
+    token_slabs: bool | int = False,
 ) -> tuple[torch.Tensor, dict[str, torch.Tensor], torch.Tensor, torch.Tensor]:
     """GRPO loss straight from final hidden states; returns ``(loss, stats, logprobs, entropy)``.
 
@@ -572,7 +573,18 @@ def grpo_loss_on_hidden(
     bf16, ``weight`` ``[V, H]`` bf16, ``labels`` and the side tensors ``[B, T]`` (anything that
     broadcasts).  ``logprobs`` and ``entropy`` are returned detached, 0 off the mask.  Without a
     gradient to compute (``torch.no_grad()``, inputs without ``requires_grad``) only the forward runs.
+
+    ``token_slabs=True`` (or a slab size in tokens, a multiple of 4096; ``True`` = 8192) runs the step in
+    slabs of that many selected tokens without recomputing anything: a
+    slab's forward leaves its exponentials (all vocabulary columns, bf16) in a slab-sized scratch
+    buffer, the slab's tokens get their upstream gradient at once, and both backward products read
+    that buffer before the next slab overwrites it (``d_weight`` accumulates in fp32 over the
+    slabs).  6·N·H·V of matrix work instead of 8·N·H·V; the scratch is ``[slab, vocab]`` bf16 plus an
+    fp32 ``[vocab, hidden]``, never ``[tokens, vocab]``.  Larger slabs are faster (fewer passes over the
+    fp32 ``d_weight``, fewer launch ends).  Not together with ``logit_cache_chunks``.
     """
+    if token_slabs and logit_cache_chunks not in (0, None):
+        raise ValueError("token_slabs keeps its own scratch; it cannot be combined with logit_cache_chunks")
     if axis not in (None, 1, -1):
         raise ValueError("axis must be None or the token axis (1)")
     if loss_denominator is not None and float(loss_denominator) <= 0.0:
@@ -621,9 +633,18 @@ def grpo_loss_on_hidden(
 
     cache_chunks = lm_head.resolve_cache_chunks(logit_cache_chunks, rows * cols, v, dev) if rows * cols > 0 else 0
     cache = None
-    if cache_chunks:
+    if token_slabs:
+        # the C entry's tag for the slab-wise step (minus the slab size in units of 4096 rows); its scratch is
+        # part of the workspace
+        slab_tokens = 8192 if token_slabs is True else int(token_slabs)
+        if slab_tokens < 4096 or slab_tokens % 4096:
+            raise ValueError("token_slabs must be True or a multiple of 4096 tokens")
+        cache_chunks = -(slab_tokens // 4096)
+    elif cache_chunks:
         cache = torch.empty(lib.oi_lmhead_cache_bytes(rows * cols, v, cache_chunks), dtype=torch.uint8, device=dev)
-    ws_bytes = lib.oi_lmhead_grpo_workspace_bytes(rows, cols, h, v, cache_chunks if cache is not None else 0)
+    if cache is None and cache_chunks > 0:
+        cache_chunks = 0
+    ws_bytes = lib.oi_lmhead_grpo_workspace_bytes(rows, cols, h, v, cache_chunks)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     _lib.call(
         "oi_lmhead_grpo_fwd_bwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), m.data_ptr(), _lib.ptr(old_c),

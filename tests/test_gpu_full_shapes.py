@@ -132,6 +132,39 @@ def _check_fused_head(hidden, weight, labels_eff, mask, g_cpu, lp, ent, d_hidden
     assert (per_v <= 2 * REL).all(), per_v.max().item()
 
 
+def test_c3_llama8b_head_grpo_in_token_slabs_full_shape():
+    """The c3 step through grpo_loss_on_hidden(token_slabs=True): three slabs of up to 8192 selected rows,
+    nothing recomputed, d_weight accumulated in fp32 over the slabs."""
+    print("case c3 token slabs N=32768 H=4096 V=128256", flush=True)
+    torch.manual_seed(0)
+    n, h, v = 32768, 4096, 128256
+    hidden = torch.randn(n, h, device=DEV).bfloat16().requires_grad_(True)
+    weight = (torch.randn(v, h, device=DEV) * 0.02).bfloat16().requires_grad_(True)
+    labels = torch.randint(0, v, (n,), device=DEV)
+    mask = torch.rand(n, device=DEV) < 0.7
+    adv = torch.randn(n, device=DEV)
+    cfg = _cfg()
+    with torch.no_grad():
+        lp0, _ = lm_head.fused_lm_head_logprobs(hidden, weight, labels, mask=mask)
+    old = lp0 + 0.05 * torch.randn(n, device=DEV)
+    ref = lp0 + 0.1 * torch.randn(n, device=DEV)
+    loss, stats, lp, ent = grpo_utils.grpo_loss_on_hidden(
+        hidden[None], weight, labels[None], old[None], ref[None], adv[None], mask[None], cfg, token_slabs=True
+    )
+    loss.backward()
+    torch.cuda.synchronize()
+    lp, ent = lp[0], ent[0]
+    assert (lp - lp0).abs().max().item() <= 1e-5
+    lp_leaf = lp.detach().cpu().requires_grad_(True)
+    loss_o, *_ = o_grpo.grpo_token_loss(
+        lp_leaf[None], old.cpu()[None], ref.cpu()[None], adv.cpu()[None], mask.cpu()[None].float(), cfg
+    )
+    loss_o.backward()
+    assert abs(loss.item() - loss_o.item()) <= 1e-5 + 1e-5 * abs(loss_o.item())
+    assert int(stats["num_response_tokens"].item()) == int(mask.sum().item())
+    _check_fused_head(hidden, weight, labels, mask, lp_leaf.grad, lp, ent, hidden.grad, weight.grad, seed=5)
+
+
 @pytest.mark.parametrize("cache_chunks", [0, 4, 1])
 def test_c3_llama8b_head_grpo_full_shape(cache_chunks):
     """hidden bf16 [32768, 4096], W bf16 [128256, 4096], 70 % response rows: fused lm_head + logprob +

@@ -361,6 +361,70 @@ def test_concatenated_forward_olmo_through_dpo_lm_head(packing, average_log_prob
         assert ((got - exp).norm() / exp.norm()).item() <= 2e-2
 
 
+@pytest.mark.parametrize("b,t,h,v,axis,want_dw,slabs", [
+    (3, 130, 128, 40000, None, True, True),  # one slab, two vocabulary chunks
+    (5, 2500, 64, 700, None, True, True),  # two slabs of selected tokens: d_weight accumulates over them
+    (5, 2500, 64, 700, 1, False, 4096),  # three slabs
+    (9, 2000, 64, 300, None, True, True),  # the third slab is short
+    (9, 2000, 64, 300, None, True, 4096),  # five slabs, the last one empty (no selected row reaches it)
+])  # fmt: skip
+def test_grpo_loss_on_hidden_in_token_slabs(b, t, h, v, axis, want_dw, slabs):
+    """The whole step without recomputation (slabs of 8192 selected tokens, the exponentials of one
+    slab at a time) against the oracle chain."""
+    print(f"case b={b} t={t} h={h} v={v} axis={axis} dW={want_dw} slabs={slabs}", flush=True)
+    torch.manual_seed(41)
+    hidden = torch.randn(b, t, h).bfloat16()
+    weight = (torch.randn(v, h) * 3.0 / math.sqrt(h)).bfloat16()
+    labels = torch.randint(0, v, (b, t))
+    mask = torch.rand(b, t) < 0.8
+    mask[1, :] = False
+    adv = torch.randn(b, 1)
+    cfg = make_grpo_config(loss_fn="dapo", beta=0.05, kl_estimator=2, clip_higher=0.28)
+    rh = hidden.float().requires_grad_(True)
+    rw = weight.float().requires_grad_(True)
+    lp_o, ent_o = o_lm.lm_head_logprobs(rh.reshape(b * t, h), rw, labels.reshape(-1), 1.0, True)
+    lp_o, ent_o = lp_o.reshape(b, t), ent_o.reshape(b, t)
+    old = lp_o.detach() + 0.05 * torch.randn(b, t)
+    ref = lp_o.detach() + 0.1 * torch.randn(b, t)
+    loss_o, *_ = o_grpo.grpo_token_loss(lp_o, old, ref, adv.expand(b, t), mask.float(), cfg, axis=axis)
+    torch.nan_to_num(loss_o, nan=0.0).backward()
+    exp_dh, exp_dw = torch.nan_to_num(rh.grad, nan=0.0), torch.nan_to_num(rw.grad, nan=0.0)
+
+    d = lambda x: x.to(DEV)  # noqa: E731
+    dh = d(hidden).requires_grad_(True)
+    dw = d(weight).requires_grad_(want_dw)
+    loss, stats, lp, ent = grpo_utils.grpo_loss_on_hidden(
+        dh, dw, d(labels), d(old), d(ref), d(adv), d(mask), cfg, axis=axis, token_slabs=slabs
+    )
+    loss.backward()
+    assert ((lp.cpu() - lp_o.detach()) * mask).abs().max().item() <= TOL and (lp.cpu()[~mask] == 0).all()
+    assert ((ent.cpu() - ent_o) * mask).abs().max().item() <= TOL and (ent.cpu()[~mask] == 0).all()
+    if axis is None:
+        assert abs(loss.item() - loss_o.item()) <= TOL
+    got = dh.grad.float().cpu()
+    assert (got - exp_dh).abs().max().item() <= _bf16_tol(exp_dh)
+    assert ((got - exp_dh).norm() / exp_dh.norm()).item() <= 2e-2
+    assert (dh.grad.cpu()[~mask] == 0).all()
+    if want_dw:
+        gw = dw.grad.float().cpu()
+        assert (gw - exp_dw).abs().max().item() <= _bf16_tol(exp_dw)
+        assert ((gw - exp_dw).norm() / exp_dw.norm()).item() <= 2e-2
+    else:
+        assert dw.grad is None
+    # the statistics are those of the recomputing step
+    dh2 = d(hidden).requires_grad_(True)
+    loss2, stats2, lp2, _ = grpo_utils.grpo_loss_on_hidden(
+        dh2, d(weight).requires_grad_(want_dw), d(labels), d(old), d(ref), d(adv), d(mask), cfg, axis=axis
+    )
+    # (not to the last bit: a slab's forward merges its vocabulary splits in another order)
+    assert (lp - lp2).abs().max().item() <= 1e-5 and abs(loss.item() - loss2.item()) <= 1e-6
+    for k in stats2:
+        assert torch.allclose(stats[k], stats2[k], rtol=1e-4, atol=1e-6, equal_nan=True), k
+    with pytest.raises(ValueError):
+        grpo_utils.grpo_loss_on_hidden(dh2, d(weight), d(labels), d(old), d(ref), d(adv), d(mask), cfg, token_slabs=True,
+                                       logit_cache_chunks=1)
+
+
 @pytest.mark.parametrize("loss_fn,axis,denominator,with_old,want_dw", [
     ("dapo", None, None, True, True),
     ("dapo", 1, None, True, False),
