@@ -201,6 +201,7 @@ def fused_linear_cross_entropy(
     num_items_in_batch: torch.Tensor | int | float | None = None,
     ignore_index: int = -100,
     logit_cache_chunks: int = 0,
+    token_slabs: bool | int = False,
 ) -> torch.Tensor:
     """Causal-LM cross-entropy of ``hidden @ weight.T`` against next-token labels, scalar fp32.
 
@@ -211,6 +212,13 @@ def fused_linear_cross_entropy(
     or ``sum / num_items_in_batch`` when that count is given (gradient accumulation over several
     micro-batches).  Differentiable with respect to ``hidden`` and ``weight``.
     ``logit_cache_chunks`` as for :func:`fused_lm_head_logprobs`.
+
+    ``token_slabs`` (``True`` = slabs of 8192 kept tokens, or a multiple of 4096) computes the loss and
+    both gradients in one call with nothing recomputed: every token's upstream gradient is the known
+    constant ``-1 / count``, so the step can run slab by slab like
+    :func:`open_instruct_amd.grpo_utils.grpo_loss_on_hidden` (whose ``loss_fn="cispo"`` term with
+    unit advantages, ratio 1 and no KL term *is* the negative log-likelihood); the gradients are
+    handed out by ``loss.backward()``.  Needs a 2-D ``[B, T]`` batch.
     """
     if (labels is None) == (shift_labels is None):
         raise ValueError("pass exactly one of labels / shift_labels")
@@ -220,6 +228,23 @@ def fused_linear_cross_entropy(
     if shift_labels.shape != hidden.shape[:-1]:
         raise ValueError(f"labels {tuple(shift_labels.shape)} do not match hidden {tuple(hidden.shape)}")
     keep = shift_labels != ignore_index
+    if token_slabs:
+        import types
+
+        from . import grpo_utils
+
+        if shift_labels.ndim != 2:
+            raise ValueError("token_slabs needs [B, T] labels")
+        # masked_mean(-logprob, keep, denominator): the CISPO term with advantage 1, ratio 1, beta 0
+        nll = types.SimpleNamespace(loss_fn="cispo", clip_lower=0.0, clip_higher=0.0, beta=0.0, kl_estimator=2)
+        denominator = None
+        if num_items_in_batch is not None:
+            denominator = float(num_items_in_batch)  # a device tensor is read here: the C entry takes a number
+        loss, _, _, _ = grpo_utils.grpo_loss_on_hidden(
+            hidden, weight, shift_labels, None, None, torch.ones((), device=hidden.device), keep, nll,
+            loss_denominator=denominator, token_slabs=token_slabs,
+        )  # fmt: skip
+        return loss
     logps, _ = fused_lm_head_logprobs(hidden, weight, shift_labels, mask=keep, logit_cache_chunks=logit_cache_chunks)
     total = -logps.sum()
     if num_items_in_batch is None:

@@ -253,6 +253,16 @@ def test_fused_linear_cross_entropy_matches_oracle(num_items):
     assert (dh.grad.float().cpu() - rh.grad).abs().max().item() <= TOL + rh.grad.abs().max().item() * 2**-7
     assert (dw.grad.float().cpu() - rw.grad).abs().max().item() <= TOL + rw.grad.abs().max().item() * 2**-7
     assert ((dw.grad.float().cpu() - rw.grad).norm() / rw.grad.norm()).item() <= 2e-2
+    # the same loss and gradients in token slabs (one call, nothing recomputed)
+    dh3 = hidden.to(DEV).requires_grad_(True)
+    dw3 = weight.to(DEV).requires_grad_(True)
+    got3 = lm_head.fused_linear_cross_entropy(dh3, dw3, labels.to(DEV), num_items_in_batch=num_items, token_slabs=True)
+    got3.backward()
+    assert abs(got3.item() - exp.item()) <= TOL
+    assert (dh3.grad.float().cpu() - rh.grad).abs().max().item() <= TOL + rh.grad.abs().max().item() * 2**-7
+    assert (dw3.grad.float().cpu() - rw.grad).abs().max().item() <= TOL + rw.grad.abs().max().item() * 2**-7
+    assert ((dw3.grad.float().cpu() - rw.grad).norm() / rw.grad.norm()).item() <= 2e-2
+    assert ((dh3.grad.float().cpu() - rh.grad).norm() / rh.grad.norm()).item() <= 2e-2
     # already shifted labels give the same loss
     shifted = torch.full_like(labels, -100)
     shifted[:, :-1] = labels[:, 1:]
