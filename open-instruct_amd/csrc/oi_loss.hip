@@ -887,7 +887,7 @@ extern "C" int oi_logprob_diff_stats(const float* local_logprobs, const float* o
     return oi_launch_status();
 }
 
-extern "C" int oi_version(void) { return 1100; }
+extern "C" int oi_version(void) { return 1200; }
 
 extern "C" const char* oi_error_string(int code) {
     switch (code) {
