@@ -822,6 +822,7 @@ __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B,
     A.r0 = m0;
     B.r0 = n0;
     AccTile acc;
+    if (K <= 0 && mode == 1) return;  // nothing to add
     if (K > 0) {
         gemm_tile<A_KM, B_KM>(acc, A, B, K, lds);
     } else {
@@ -1376,9 +1377,9 @@ __global__ void __launch_bounds__(256)
 // cache of exponentials skip the recomputation: the cache itself is the A operand of both products
 // (see cache_rows_prepare_kernel).  The queue words must be zeroed.
 // dw_mode / dw32: how d_weight is stored.  2 (default): this call holds every token, bf16 rows are
-// written directly.  0 / 1 / 3: the tokens come in several calls; dw32 (fp32 [vocab, hidden]) takes
-// the first call's product (0), adds the following ones (1), and the last call (3) writes
-// bf16 d_weight = dw32 + its own product.
+// written directly.  0 / 1: the tokens come in several calls; dw32 (fp32 [vocab, hidden]) takes the
+// first call's product (0) and adds the following ones (1; a call without tokens adds nothing and
+// costs nothing); the caller rounds dw32 to bf16 when the last call is through.
 void enqueue_bwd(const BwdPlan& p, char* ws, const RowInputs& in, const void* weight, int64_t n_tokens,
                  int64_t hidden_dim, int64_t vocab, float inv_temperature, void* d_hidden, void* d_weight,
                  uint16_t* ecache, const CachePlan& cache, hipStream_t s, int dw_mode = 2, float* dw32 = nullptr) {
@@ -1505,6 +1506,15 @@ SlabPlan plan_slabs(int64_t rows, int64_t cols, int64_t hdim, int64_t vocab, boo
     p.off_denoms = cv.take((size_t)rows * sizeof(float));
     p.total = cv.off;
     return p;
+}
+
+// out[8 i .. 8 i + 8) = bf16(in[8 i .. 8 i + 8))
+__global__ void __launch_bounds__(256) f32_to_bf16_kernel(const float* __restrict__ in, int64_t n8, uint16_t* __restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8) return;
+    const float4 a = reinterpret_cast<const float4*>(in)[2 * i], b = reinterpret_cast<const float4*>(in)[2 * i + 1];
+    reinterpret_cast<oi_u32x4*>(out)[i] =
+        oi_u32x4{oi_pack_bf16x2(a.x, a.y), oi_pack_bf16x2(a.z, a.w), oi_pack_bf16x2(b.x, b.y), oi_pack_bf16x2(b.z, b.w)};
 }
 
 // counts[i] = number of selected rows that fall into slab i
@@ -1764,9 +1774,14 @@ int grpo_step_in_slabs(const void* hidden, const void* weight, const int64_t* la
         in.lse = lse_c + r0;
         in.grad = grad_c + r0;
         in.logprob = logprob_c + r0;
-        const int dw_mode = p.n_slabs == 1 ? 2 : (i == 0 ? 0 : (i == p.n_slabs - 1 ? 3 : 1));
+        const int dw_mode = p.n_slabs == 1 ? 2 : (i == 0 ? 0 : 1);
         enqueue_bwd(p.bwd, ws_bwd, in, weight, p.slab, hidden_dim, vocab, inv_temperature, d_hidden, d_weight, ecache,
                     p.cache, s, dw_mode, dw32);
+    }
+    if (dw32) {
+        const int64_t n8 = vocab * hidden_dim / 8;  // hidden_dim is a multiple of 64
+        hipLaunchKernelGGL(f32_to_bf16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, s, dw32, n8,
+                           static_cast<uint16_t*>(d_weight));
     }
     // loss and statistics from all logprobs
     return oi_grpo_fused_fwd(logprob, old_logprobs, ref_logprobs, advantages, mask, rho_weights, entropy, nullptr, nullptr,
