@@ -9,7 +9,9 @@
  * Conventions
  *  - Every pointer is DEVICE memory owned by the caller.  The library never allocates, frees or
  *    keeps a pointer after the call returns.  Scratch memory is passed in as `workspace` and sized
- *    by the matching oi_*_workspace_bytes().
+ *    by the matching oi_*_workspace_bytes().  Workspaces and fp32 accumulators (wsum) must be
+ *    ordinary device allocations (hipMalloc, a torch tensor): the kernels add to them with the
+ *    L2's floating-point atomics, which fine-grained or host-mapped memory does not support.
  *  - Work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the null stream) and the
  *    call returns without waiting for it.
  *  - Return value: 0 on success, a negative OI_E* code for a rejected argument (nothing was
