@@ -530,16 +530,18 @@ def test_grpo_loss_on_hidden_whole_step(loss_fn, axis, denominator, with_old, wa
             assert ((dw5.grad.float().cpu() - exp_dw).norm() / exp_dw.norm()).item() <= 2e-2
 
 
-def test_entry_points_replay_from_a_hip_graph():
+@pytest.mark.parametrize("slabs,t", [(False, 140), (4096, 3000)])
+def test_entry_points_replay_from_a_hip_graph(slabs, t):
     """The C entry points enqueue kernels only (no allocation, no synchronisation, no memset nodes), so a
     caller may capture them in a HIP graph.  Two launch-bound cases: logprob + entropy + masked means on
-    small logits, and the whole GRPO step on hidden states in one call.  Every replay is compared with the
-    eager result on inputs that eager work changed between the replays."""
+    small logits, and the whole GRPO step on hidden states in one call (recomputing, and in two token slabs
+    whose d_weight accumulates through the L2's atomics).  Every replay is compared with the eager result on
+    inputs that eager work changed between the replays."""
     torch.manual_seed(51)
     logits = (torch.randn(4, 128, 8000, device=DEV) * 2.0)
     ids = torch.randint(0, 8000, (4, 128), device=DEV)
     mask = torch.rand(4, 128, device=DEV) > 0.3
-    b, t, h, v = 2, 140, 128, 3000
+    b, h, v = 2, 128, 3000
     hidden = torch.randn(b, t, h, device=DEV).bfloat16().requires_grad_(True)
     weight = (torch.randn(v, h, device=DEV) * 0.2).bfloat16().requires_grad_(True)
     labels = torch.randint(0, v, (b, t), device=DEV)
@@ -556,7 +558,9 @@ def test_entry_points_replay_from_a_hip_graph():
     def grpo_step():
         hidden.grad = None
         weight.grad = None
-        loss, _, lp, _ = grpo_utils.grpo_loss_on_hidden(hidden, weight, labels, None, None, adv, rmask, cfg)
+        loss, _, lp, _ = grpo_utils.grpo_loss_on_hidden(
+            hidden, weight, labels, None, None, adv, rmask, cfg, token_slabs=slabs
+        )
         loss.backward()
         return loss.detach(), hidden.grad, weight.grad
 
