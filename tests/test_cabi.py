@@ -107,6 +107,22 @@ def test_rejected_arguments_return_codes_without_launching():
     assert lib.oi_lmhead_cache_bytes(256, 70000, 1) == 256 * 32768 * 2 and lib.oi_lmhead_cache_bytes(256, 70000, 9) == 256 * 70144 * 2
     assert lib.oi_lmhead_cache_bytes(256, 70000, 0) == 0
     assert lib.oi_lmhead_fwd_workspace_bytes(256, 64, 256, 1) == lib.oi_lmhead_fwd_workspace_bytes(256, 64, 256, 0) + 256 * 4 + 256 + 256 * 64 * 2 + 256 * 8
+    # the forward that also accumulates the weighted sum of weight rows: the plain forward's buffers (one split per
+    # vocabulary tile at this size), one pair of queue sets per vocabulary chunk of 65536 columns and the chunk of
+    # exponentials (2 bytes per token and column)
+    assert lib.oi_lmhead_fwd_wsum_workspace_bytes(0, 64, 10, 0) == 0
+    assert lib.oi_lmhead_fwd_wsum_workspace_bytes(256, 64, 256, 0) == 256 * 16 + 256 * 4 + 256 + 256 * 256 * 2
+    assert lib.oi_lmhead_fwd_wsum_workspace_bytes(256, 64, 70000, 0) >= 256 * 65536 * 2
+    assert lib.oi_lmhead_dh_workspace_bytes(0) == 0 and lib.oi_lmhead_dh_workspace_bytes(300) == 512 * 4 + 256
+    assert lib.oi_lmhead_logp_fwd_wsum(None, None, None, None, 4, 100, 32, 1.0, None, None, None, None, None, 0, None) == -1
+    assert lib.oi_lmhead_logp_fwd_wsum(16, 32, 8, None, 4, 64, 32, 1.0, None, None, None, None, None, 0, None) == -2
+    assert lib.oi_lmhead_dh_from_wsum(None, None, None, None, None, None, None, 4, 100, 32, 1.0, None, None, 0, None) == -1
+    assert lib.oi_lmhead_dh_from_wsum(None, None, None, None, None, None, None, 4, 64, 32, 1.0, None, None, 0, None) == -2
+    assert lib.oi_lmhead_dh_from_wsum(None, None, None, None, None, None, None, 0, 64, 32, 1.0, None, None, 0, None) == 0
+    # the whole step in token slabs (cache_chunks < 0) sizes its own scratch: a slab of exponentials and an fp32 d_weight
+    slabs = lib.oi_lmhead_grpo_workspace_bytes(4, 4096, 64, 1000, -1)
+    assert slabs >= 4096 * 1024 * 2 + 1000 * 64 * 4
+    assert lib.oi_lmhead_grpo_workspace_bytes(4, 4096, 64, 1000, -2) >= slabs + 4096 * 1024 * 2
 
 
 def test_cpu_tensors_are_refused_loudly():
