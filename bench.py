@@ -268,7 +268,7 @@ def make_c1(torch, oi):
     return step, info
 
 
-def make_c4(torch, oi, hdim=4096, vocab=100352, n_seqs=16, budget=32768):
+def make_c4(torch, oi, hdim=4096, vocab=100352, n_seqs=16, budget=32768, token_slabs=False):
     """Packed (padding-free) batch: per-sequence summed logprobs through cu_seqlens plus the GRPO loss
     with masked_mean(axis=1) over the packed row, forward and backward."""
     dev = "cuda:0"
@@ -298,6 +298,20 @@ def make_c4(torch, oi, hdim=4096, vocab=100352, n_seqs=16, budget=32768):
     n_eff = int(mask.sum().item())
     fwd_timer = EventTimer(torch)
 
+    def step_slabs():
+        # the GRPO loss and both gradients in one slab-wise call (nothing recomputed); the per-sequence sums are
+        # taken from the returned logprobs (the loss does not depend on them)
+        hidden.grad = None
+        weight.grad = None
+        with fwd_timer:
+            loss, _, lp, _ = oi.grpo_utils.grpo_loss_on_hidden(
+                hidden[None], weight, shifted.view(1, -1), old[None], ref[None], adv[None], mask[None], cfg, axis=1,
+                token_slabs=True,
+            )
+        oi.padding_free_collator.get_batch_logps(lp.view(1, -1), labels, cu)
+        loss.backward()
+        return loss
+
     def step():
         hidden.grad = None
         weight.grad = None
@@ -320,6 +334,10 @@ def make_c4(torch, oi, hdim=4096, vocab=100352, n_seqs=16, budget=32768):
         "bound": "mfma",
         "timer": fwd_timer,
     }
+    if token_slabs:
+        info["kernel"] = "oi_lmhead_grpo_fwd_bwd in slabs of 8192 selected tokens (nothing is recomputed)"
+        info["alg_per_launch"] = 3.0 * flops_fwd
+        return step_slabs, info
     return step, info
 
 
@@ -379,8 +397,7 @@ def cpu_baseline(torch, workload):
     threads = torch.get_num_threads()
     cfg = _cfg()
     torch.manual_seed(0)
-    if workload == "c3-one-call":
-        workload = "c3"
+    workload = {"c3-one-call": "c3", "c3-slabs": "c3", "c4-slabs": "c4"}.get(workload, workload)
     if workload in ("c3", "c4", "c5"):
         hdim = 8192 if workload == "c5" else 4096
         vocab, n = (100352 if workload == "c4" else 128256), 2048
@@ -500,7 +517,7 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="c3",
-                    choices=["c1", "c2", "c2-two-pass", "c3", "c3-one-call", "c3-slabs", "c4", "c5", "pack"])
+                    choices=["c1", "c2", "c2-two-pass", "c3", "c3-one-call", "c3-slabs", "c4", "c4-slabs", "c5", "pack"])
     ap.add_argument("--cache-chunks", type=int, default=0,
                     help="c3 / c3-one-call / c5 only: keep 2^logit in bf16 for this many vocabulary chunks of 32768 "
                          "columns instead of recomputing them in the backward pass (0 = the headline configuration: "
@@ -541,6 +558,11 @@ def main():
     elif args.workload == "c4":
         step, info = make_c4(torch, oi)
         name = "c4: packed OLMo-2-7B shape, 16 sequences via cu_seqlens, hidden bf16 [N<=32768,4096], W bf16 [100352,4096]; per-sequence logprob sums + GRPO loss masked_mean(axis=1), fwd+bwd"
+        dtype = "bf16"
+    elif args.workload == "c4-slabs":
+        step, info = make_c4(torch, oi, token_slabs=True)
+        name = ("c4 through grpo_loss_on_hidden(token_slabs=True): packed OLMo-2-7B shape, GRPO loss masked_mean(axis=1) "
+                "fwd+bwd in slabs of 8192 tokens with nothing recomputed, per-sequence logprob sums from the returned logprobs")
         dtype = "bf16"
     elif args.workload == "c5":
         step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True, cache_chunks=args.cache_chunks)
@@ -610,7 +632,7 @@ def main():
         roofline["whole_step_frac"] = roofline["whole_step_tflops"] / PEAK_BF16_TFLOPS
         if not args.no_library_gemm:
             hdim = 8192 if args.workload == "c5" else 4096
-            vocab = 100352 if args.workload == "c4" else 128256
+            vocab = 100352 if args.workload in ("c4", "c4-slabs") else 128256
             roofline["library_bf16_gemm_tflops"] = library_gemm_tflops(torch, 32768, hdim, vocab)
     if "bytes_step" in info:
         roofline["whole_step_gbs"] = info["bytes_step"] / (ms_per_step * 1e-3) / 1e9
