@@ -4,15 +4,17 @@ Names and signatures follow open_instruct/dpo_utils.py in the reference (``dpo_l
 ``wpo_loss`` :566-613, ``simpo_loss`` :617-642, ``compute_loss`` :645-686, ``_get_batch_logps``
 :689-712, ``process_batch`` :715-731, ``concatenated_inputs`` :734-763, ``concatenated_forward``
 :826-878, ``separate_forward`` :881-956, ``concatenated_forward_olmo`` :959-1019,
-``build_reference_logprobs_cache`` :405-520 without its multi-process steps).
+``build_reference_logprobs_cache`` :405-520).
 """
 
 from __future__ import annotations
 
+import contextlib
 import pathlib
 from collections.abc import Callable, Iterable
 
 import torch
+import torch.distributed as dist
 
 from . import _lib, lm_head, model_utils, olmo_core_utils, padding_free_collator
 from .padding_free_collator import get_batch_logps_padded
@@ -319,42 +321,71 @@ def build_reference_logprobs_cache(
     forward_fn: Callable,
     full_dataset_size: int,
     device: torch.device,
-    cache_path: pathlib.Path | str | None = None,
+    cache_path: pathlib.Path | str,
+    is_main_process: bool,
+    model_dims=None,
+    use_lora: bool = False,
+    disable_adapter_context: Callable[[], contextlib.AbstractContextManager] | None = None,
     forward_kwargs: dict | None = None,
 ) -> model_utils.TensorCache:
-    """Reference-policy logps of every sample, computed once; open_instruct/dpo_utils.py:405-520.
+    """Reference-policy logps of every sample, computed once; open_instruct/dpo_utils.py:405-520,
+    same parameters in the same order (both reference callers pass them by keyword:
+    open_instruct/dpo_tune_cache.py:522-534, open_instruct/dpo.py:310).
 
     One no-grad pass over ``dataloader``: ``forward_fn(model, batch, average_log_prob=...)`` returns
     ``(chosen_logps, rejected_logps, aux)``, which are scattered to ``batch["index"]``.  Batches
     flagged ``is_padding`` are skipped; an index that no batch covered raises, as in the reference.
-    An existing ``cache_path`` is loaded instead of recomputed, a new cache is written there.
-    This is the one-process form: the reference's barriers and MAX all-reduce across ranks
-    (open_instruct/dpo_utils.py:456,494-495,518) belong to the caller's launcher.
+    An existing ``cache_path`` is loaded instead of recomputed.  ``is_main_process`` gates the
+    directory check and the write of the new cache; with ``use_lora`` the forward runs inside
+    ``disable_adapter_context()`` when one is given; ``model_dims`` only feeds the reference's
+    progress-bar MFU read-out and is accepted and unused.  The barriers and the MAX all-reduce across
+    ranks (open_instruct/dpo_utils.py:456,494-495,518) run when a process group is initialised.
     """
-    cache_path = pathlib.Path(cache_path) if cache_path is not None else None
-    if cache_path is not None and cache_path.exists():
+    del model_dims
+    cache_path = pathlib.Path(cache_path)
+    if cache_path.exists():
         return model_utils.TensorCache.from_disk(cache_path, device=device)
-    was_training = model.training
+    if is_main_process:
+        cache_path.parent.mkdir(parents=True, exist_ok=True)
+        probe = cache_path.parent / f".write_test_{cache_path.stem}"
+        try:
+            probe.touch()
+            probe.unlink()
+        except (OSError, PermissionError) as e:
+            raise RuntimeError(
+                f"Cannot write to cache directory {cache_path.parent}: {e}. "
+                f"Set REFERENCE_LOGPROBS_CACHE_PATH to a writable location."
+            ) from e
+    distributed = dist.is_available() and dist.is_initialized()
+    if distributed:
+        dist.barrier()
     model.eval()
     chosen = torch.full((full_dataset_size,), float("-inf"), dtype=torch.float32, device=device)
     rejected = torch.full((full_dataset_size,), float("-inf"), dtype=torch.float32, device=device)
     with torch.no_grad():
         for batch in dataloader:
-            chosen_logps, rejected_logps, _ = forward_fn(
-                model, batch, average_log_prob=average_log_prob, **(forward_kwargs or {})
-            )
+            adapter_off = disable_adapter_context() if use_lora and disable_adapter_context is not None else None
+            with adapter_off if adapter_off is not None else contextlib.nullcontext():
+                chosen_logps, rejected_logps, _ = forward_fn(
+                    model, batch, average_log_prob=average_log_prob, **(forward_kwargs or {})
+                )
             if batch.get("is_padding", False):
                 continue
             index = batch["index"].to(device).long()
             chosen[index] = chosen_logps.float()
             rejected[index] = rejected_logps.float()
+    if distributed:
+        dist.all_reduce(chosen, op=dist.ReduceOp.MAX)
+        dist.all_reduce(rejected, op=dist.ReduceOp.MAX)
     missing = torch.where((chosen == float("-inf")) | (rejected == float("-inf")))[0]
     if len(missing) > 0:
         raise RuntimeError(
             f"Missing {len(missing)} indices during reference logprobs caching. First 10: {missing[:10].tolist()}"
         )
-    model.train(was_training)
+    model.train()
     cache = model_utils.TensorCache(tensors={"chosen_logps": chosen, "rejected_logps": rejected})
-    if cache_path is not None:
+    if is_main_process:
         cache.to_disk(cache_path)
+    if distributed:
+        dist.barrier()
     return cache

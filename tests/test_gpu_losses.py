@@ -566,7 +566,7 @@ def test_vllm_local_debug_metrics_parity(shape):
         grpo_utils.vllm_local_debug_stats(local.to(DEV), vllm.to(DEV)[..., :-1], mask.to(DEV))
 
 
-def test_reference_cache_build_through_concatenated_forward():
+def test_reference_cache_build_through_concatenated_forward(tmp_path):
     """open_instruct/dpo_utils.py:405-520 over open_instruct/dpo_utils.py:826-878 with a stub model:
     the cache holds, per dataset index, what a direct oracle evaluation of that sample gives."""
     g = torch.Generator().manual_seed(24)
@@ -592,8 +592,11 @@ def test_reference_cache_build_through_concatenated_forward():
     samples = [sample(i) for i in (2, 0, 3, 1)]
     batches = [{k: val.to(DEV) for k, val in s.items()} for s in samples]
     cache = dpo_utils.build_reference_logprobs_cache(
-        Model(), batches, False, dpo_utils.concatenated_forward, n_samples, torch.device(DEV)
-    )
+        model=Model(), dataloader=batches, average_log_prob=False, forward_fn=dpo_utils.concatenated_forward,
+        full_dataset_size=n_samples, device=torch.device(DEV), cache_path=tmp_path / "reference_logps.pt",
+        is_main_process=True, model_dims=None,
+    )  # fmt: skip
+    assert (tmp_path / "reference_logps.pt").exists()
     for s in samples:
         i = int(s["index"])
         for side in ("chosen", "rejected"):

@@ -1,5 +1,7 @@
 """Host-side plumbing that needs no GPU: row layouts, reshapes, label shifts, batch concatenation."""
 
+import contextlib
+
 import pytest
 import torch
 
@@ -141,21 +143,66 @@ def test_tensor_cache_roundtrip_and_reference_cache_builder(tmp_path):
         {"index": torch.tensor([1, 3])},
         {"index": torch.tensor([0, 0]), "is_padding": True},
     ]
+    # called as open_instruct/dpo_tune_cache.py:522-534 calls it (every argument by keyword)
     built = dpo_utils.build_reference_logprobs_cache(
-        model, batches, True, forward_fn, 4, torch.device("cpu"), tmp_path / "ref.pt", forward_kwargs={"scale": 2.0}
+        model=model,
+        dataloader=batches,
+        average_log_prob=True,
+        forward_fn=forward_fn,
+        full_dataset_size=4,
+        device=torch.device("cpu"),
+        cache_path=tmp_path / "deep" / "ref.pt",
+        is_main_process=True,
+        model_dims=object(),
+        use_lora=False,
+        disable_adapter_context=None,
     )
-    assert built.tensors["chosen_logps"].tolist() == [0.0, 2.0, 4.0, 6.0]
-    assert built.tensors["rejected_logps"].tolist() == [0.0, -2.0, -4.0, -6.0]
+    assert built.tensors["chosen_logps"].tolist() == [0.0, 1.0, 2.0, 3.0]
+    assert built.tensors["rejected_logps"].tolist() == [0.0, -1.0, -2.0, -3.0]
     assert calls == [(False, True, False)] * 3 and model.training
-    assert (tmp_path / "ref.pt").exists()
+    assert (tmp_path / "deep" / "ref.pt").exists()
     # an existing file is loaded, not recomputed
     n_calls = len(calls)
     loaded = dpo_utils.build_reference_logprobs_cache(
-        model, batches, True, forward_fn, 4, torch.device("cpu"), tmp_path / "ref.pt"
+        model, batches, True, forward_fn, 4, torch.device("cpu"), tmp_path / "deep" / "ref.pt", True, None
     )
     assert len(calls) == n_calls and torch.equal(loaded.tensors["chosen_logps"], built.tensors["chosen_logps"])
+    # the keyword dictionary of open_instruct/dpo.py:310 (`model=..., **cache_kwargs`), extra forward arguments
+    # included; a process that is not the main one computes the cache and writes nothing
+    cache_kwargs = dict(
+        dataloader=batches, average_log_prob=False, forward_fn=forward_fn, full_dataset_size=4,
+        device=torch.device("cpu"), cache_path=tmp_path / "other" / "ref.pt", is_main_process=False,
+        model_dims=None, forward_kwargs={"scale": 2.0},
+    )  # fmt: skip
+    model.eval()
+    quiet = dpo_utils.build_reference_logprobs_cache(model=model, **cache_kwargs)
+    assert quiet.tensors["chosen_logps"].tolist() == [0.0, 2.0, 4.0, 6.0] and model.training
+    assert not (tmp_path / "other").exists()
+    # with LoRA the forward runs inside the context that switches the adapter off
+    entered = []
+
+    @contextlib.contextmanager
+    def adapter_off():
+        entered.append("in")
+        yield
+        entered.append("out")
+
+    dpo_utils.build_reference_logprobs_cache(
+        model, batches, False, forward_fn, 4, torch.device("cpu"), tmp_path / "lora.pt", True, None,
+        use_lora=True, disable_adapter_context=adapter_off,
+    )  # fmt: skip
+    assert entered == ["in", "out"] * 3
+    entered.clear()
+    dpo_utils.build_reference_logprobs_cache(
+        model, batches, False, forward_fn, 4, torch.device("cpu"), tmp_path / "nolora.pt", True, None,
+        use_lora=False, disable_adapter_context=adapter_off,
+    )  # fmt: skip
+    assert entered == []
     with pytest.raises(RuntimeError, match="Missing 1 indices"):
-        dpo_utils.build_reference_logprobs_cache(model, batches[:2], False, forward_fn, 5, torch.device("cpu"))
+        dpo_utils.build_reference_logprobs_cache(
+            model, batches[:2], False, forward_fn, 5, torch.device("cpu"), tmp_path / "miss.pt", True, None
+        )
+    assert not (tmp_path / "miss.pt").exists()
 
 
 def test_collation_of_packed_rows_for_workers():
