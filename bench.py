@@ -6,11 +6,15 @@ Prints ONE JSON line.  A "step" is one pass of the hot path (forward + backward)
 synthetic inputs that already live in HBM.  Workloads are the BASELINE configs:
 
   c3 (default, the headline metric): fused lm_head + logprob + entropy + GRPO loss, fwd + bwd, at
-      Llama-3.1-8B shape: hidden bf16 [32768, 4096], W bf16 [128256, 4096], 70 % response tokens.
+      Llama-3.1-8B shape: hidden bf16 [32768, 4096], W bf16 [128256, 4096], 70 % response tokens,
+      through grpo_loss_on_hidden as it runs by default (slabs of tokens, nothing recomputed);
+      c3-recompute is the same step through the three differentiable calls whose backward recomputes
+      the logits, c3-one-call-recompute the recomputing form of the one-call entry.
   c2: GRPO loss on materialised bf16 logits [64, 1024, 128256], fwd + bwd (HBM-bound), single pass;
       c2-two-pass keeps the reference's order of operations (the logits are read twice).
   c1: logprob + entropy + masked_mean on fp32 logits [4, 512, 32000], forward only.
-  c4: packed batch at OLMo-2-7B shape (16 sequences, cu_seqlens, V=100352), per-sequence sums + GRPO loss.
+  c4: packed batch at OLMo-2-7B shape (16 sequences, cu_seqlens, V=100352), per-sequence sums + GRPO loss
+      (c4-recompute: through the three differentiable calls).
   c5: DPO at Llama-3.1-70B head shape: hidden [32768, 8192], W [128256, 8192], bwd to dHidden only.
 
 `roofline` describes the dominant kernel of the workload, timed with HIP events on the stream it
@@ -42,8 +46,8 @@ PEAK_BF16_TFLOPS = 2500.0
 # profiles/; workloads without a counter run report null.
 MEASURED_TRAFFIC_BYTES = {
     # lmhead_fwd_kernel: L2 misses of the tiled operand re-reads (1.24 GB of unique operands at c3) + the partials
-    "c3": 42.01e9 + 0.20e9,
-    "c4": 40.21e9 + 0.20e9,
+    "c3-recompute": 42.01e9 + 0.20e9,
+    "c4-recompute": 40.21e9 + 0.20e9,
     # oi_lmhead_logp_fwd_wsum: four launches of lmhead_fwd_kernel<true> and four of gemm_store_kernel<false, true>
     "c5": 2 * (42.62e9 + 3.06e9) + 2 * (43.14e9 + 0.75e9),
     # lsg_grpo_fused_kernel: one read of the logits (the row waits on the CU for the gradient pass) + one write of
@@ -84,7 +88,37 @@ class EventTimer:
 # ------------------------------------------------------------------------------------------------
 # workloads
 # ------------------------------------------------------------------------------------------------
-def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=False, cache_chunks=0, token_slabs=False):
+class KernelProbe:
+    """Times one tile kernel of the slab-wise entry points through the library's own event probe (the
+    call launches several kernels, so events around the call would time all of them)."""
+
+    def __init__(self, oi, kernel):
+        self.oi, self.kernel, self.samples = oi, kernel, []
+
+    def __enter__(self):
+        self.oi._lib.call("oi_lmhead_probe_arm", self.kernel)
+        return self
+
+    def __exit__(self, *exc):
+        import ctypes
+
+        ms = (ctypes.c_float * 256)()
+        n = ctypes.c_int(0)
+        self.oi._lib.call("oi_lmhead_probe_read", ms, 256, ctypes.byref(n))
+        self.samples += [ms[i] for i in range(min(n.value, 256))]
+
+    def reset(self):
+        self.samples = []
+
+    def mean_ms(self, skip_below_ms=0.05):
+        """Average over the launches that had rows to work on (a pass past the last slab takes microseconds)."""
+        real = [x for x in self.samples if x >= skip_below_ms]
+        return sum(real) / max(1, len(real))
+
+
+def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, route="slabs"):
+    """route: "slabs" = grpo_loss_on_hidden as it runs by default, "one-call-recompute" = the same entry with
+    token_slabs=False, "recompute" = fused_lm_head_logprobs -> grpo_loss_fused -> backward."""
     dev = "cuda:0"
     torch.manual_seed(0)
     hidden = torch.randn(n_tokens, hdim, device=dev).bfloat16().requires_grad_(True)
@@ -114,33 +148,35 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=Fals
         ref_r = torch.randn(seqs // 2, device=dev) * 50 - 400
         n_eff = int(mask.sum().item())
     fwd_timer = EventTimer(torch)
+    probe = KernelProbe(oi, 2)  # the d_weight product: the largest share of the slab-wise step
 
     def step():
         hidden.grad = None
         weight.grad = None
-        if one_call:
-            with fwd_timer:  # the whole step is one C call here: the timer brackets all of it
-                loss, _, _, _ = oi.grpo_utils.grpo_loss_on_hidden(
-                    hidden[None], weight, labels[None], old[None], ref[None], adv[None], mask[None], cfg,
-                    logit_cache_chunks=cache_chunks, token_slabs=token_slabs,
-                )
-        elif not dpo:
+        if dpo:
             with fwd_timer:
-                lp, ent = oi.fused_lm_head_logprobs(
-                    hidden, weight, labels, mask=mask, return_entropy=True, logit_cache_chunks=cache_chunks
-                )
-            loss, _ = oi.grpo_utils.grpo_loss_fused(
-                lp[None], old[None], ref[None], adv[None], mask[None], cfg, entropy=ent[None]
-            )
-        else:
-            with fwd_timer:
-                lp, _ = oi.fused_lm_head_logprobs(
-                    hidden, weight, shifted.view(-1), mask=mask, logit_cache_chunks=cache_chunks
-                )
+                lp, _ = oi.fused_lm_head_logprobs(hidden, weight, shifted.view(-1), mask=mask)
             logps = oi.padding_free_collator.get_batch_logps(lp.view(1, -1), labels, cu)
             bs = logps.shape[0] // 2
             losses, _, _ = oi.dpo_utils.dpo_loss(logps[:bs], logps[bs:], ref_c, ref_r, beta=0.1)
             loss = losses.mean()
+        elif route == "slabs":
+            with probe:
+                loss, _, _, _ = oi.grpo_utils.grpo_loss_on_hidden(
+                    hidden[None], weight, labels[None], old[None], ref[None], adv[None], mask[None], cfg
+                )
+        elif route == "one-call-recompute":
+            with fwd_timer:  # the whole step is one C call here: the timer brackets all of it
+                loss, _, _, _ = oi.grpo_utils.grpo_loss_on_hidden(
+                    hidden[None], weight, labels[None], old[None], ref[None], adv[None], mask[None], cfg,
+                    token_slabs=False,
+                )
+        else:
+            with fwd_timer:
+                lp, ent = oi.fused_lm_head_logprobs(hidden, weight, labels, mask=mask, return_entropy=True)
+            loss, _ = oi.grpo_utils.grpo_loss_fused(
+                lp[None], old[None], ref[None], adv[None], mask[None], cfg, entropy=ent[None]
+            )
         loss.backward()
         return loss
 
@@ -154,15 +190,7 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=Fals
         "bound": "mfma",
         "timer": fwd_timer,
     }
-    if one_call:
-        info["kernel"] = "oi_lmhead_grpo_fwd_bwd (every launch of the step: forward, loss, dZ, dHidden, dW)"
-        info["alg_per_launch"] = 3.0 * flops_fwd
-        if token_slabs:
-            info["kernel"] = (
-                "oi_lmhead_grpo_fwd_bwd in slabs of 8192 selected tokens (per slab: forward with its exponentials kept, "
-                "loss gradient, dHidden, dW; nothing is recomputed)"
-            )
-    if dpo and not cache_chunks:
+    if dpo:
         # the weight takes no gradient: the forward call also accumulates the weighted sum of weight rows that
         # the backward to hidden needs (per vocabulary chunk: statistics + exponentials, then E_chunk @ W_chunk)
         info["kernel"] = (
@@ -170,6 +198,18 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, one_call=Fals
             "all of the step's matrix work, nothing is recomputed)"
         )
         info["alg_per_launch"] = 2.0 * flops_fwd
+    elif route == "slabs":
+        slab = oi.grpo_utils.DEFAULT_SLAB_TOKENS
+        n_slabs = max(1, -(-n_eff // slab))
+        info["kernel"] = (
+            f"gemm_store_kernel<true, true> (d_weight product of a slab of {-(-n_eff // n_slabs)} selected tokens, added to the "
+            f"fp32 d_weight; {n_slabs} such launches per step, timed one by one through the library's event probe)"
+        )
+        info["alg_per_launch"] = flops_fwd / n_slabs
+        info["timer"] = probe
+    elif route == "one-call-recompute":
+        info["kernel"] = "oi_lmhead_grpo_fwd_bwd, recomputing (every launch of the step: forward, loss, dZ, dHidden, dW)"
+        info["alg_per_launch"] = 3.0 * flops_fwd
     return step, info
 
 
@@ -268,7 +308,7 @@ def make_c1(torch, oi):
     return step, info
 
 
-def make_c4(torch, oi, hdim=4096, vocab=100352, n_seqs=16, budget=32768, token_slabs=False):
+def make_c4(torch, oi, hdim=4096, vocab=100352, n_seqs=16, budget=32768, route="slabs"):
     """Packed (padding-free) batch: per-sequence summed logprobs through cu_seqlens plus the GRPO loss
     with masked_mean(axis=1) over the packed row, forward and backward."""
     dev = "cuda:0"
@@ -297,16 +337,16 @@ def make_c4(torch, oi, hdim=4096, vocab=100352, n_seqs=16, budget=32768, token_s
     ref = lp0 + 0.1 * torch.randn(n_tokens, device=dev)
     n_eff = int(mask.sum().item())
     fwd_timer = EventTimer(torch)
+    probe = KernelProbe(oi, 2)
 
     def step_slabs():
         # the GRPO loss and both gradients in one slab-wise call (nothing recomputed); the per-sequence sums are
         # taken from the returned logprobs (the loss does not depend on them)
         hidden.grad = None
         weight.grad = None
-        with fwd_timer:
+        with probe:
             loss, _, lp, _ = oi.grpo_utils.grpo_loss_on_hidden(
-                hidden[None], weight, shifted.view(1, -1), old[None], ref[None], adv[None], mask[None], cfg, axis=1,
-                token_slabs=True,
+                hidden[None], weight, shifted.view(1, -1), old[None], ref[None], adv[None], mask[None], cfg, axis=1
             )
         oi.padding_free_collator.get_batch_logps(lp.view(1, -1), labels, cu)
         loss.backward()
@@ -334,9 +374,15 @@ def make_c4(torch, oi, hdim=4096, vocab=100352, n_seqs=16, budget=32768, token_s
         "bound": "mfma",
         "timer": fwd_timer,
     }
-    if token_slabs:
-        info["kernel"] = "oi_lmhead_grpo_fwd_bwd in slabs of 8192 selected tokens (nothing is recomputed)"
-        info["alg_per_launch"] = 3.0 * flops_fwd
+    if route == "slabs":
+        slab = oi.grpo_utils.DEFAULT_SLAB_TOKENS
+        n_slabs = max(1, -(-n_eff // slab))
+        info["kernel"] = (
+            f"gemm_store_kernel<true, true> (d_weight product of a slab of {-(-n_eff // n_slabs)} selected tokens, added to the "
+            f"fp32 d_weight; {n_slabs} such launches per step, timed one by one through the library's event probe)"
+        )
+        info["alg_per_launch"] = flops_fwd / n_slabs
+        info["timer"] = probe
         return step_slabs, info
     return step, info
 
@@ -397,12 +443,37 @@ def cpu_baseline(torch, workload):
     threads = torch.get_num_threads()
     cfg = _cfg()
     torch.manual_seed(0)
-    workload = {"c3-one-call": "c3", "c3-slabs": "c3", "c4-slabs": "c4"}.get(workload, workload)
-    if workload in ("c3", "c4", "c5"):
-        hdim = 8192 if workload == "c5" else 4096
+    workload = {"c3-recompute": "c3", "c3-one-call-recompute": "c3", "c4-recompute": "c4"}.get(workload, workload)
+    if workload == "c5":
+        # one chosen / rejected pair of 2 x 1024 tokens (of the 8 pairs of 2 x 2048), prompts masked out
+        from oracle import dpo as o_dpo
+
+        hdim, vocab, per = 8192, 128256, 1024
+        n = 2 * per
+        hidden = torch.randn(n, hdim).bfloat16().requires_grad_(True)
+        weight = (torch.randn(vocab, hdim) * 0.01).bfloat16()
+        labels = torch.randint(0, vocab, (2, per))
+        prompt = torch.randint(64, 513, (2,))
+        labels[torch.arange(per).unsqueeze(0) < prompt.unsqueeze(1)] = -100
+        ref_c, ref_r = torch.randn(1) * 50 - 400, torch.randn(1) * 50 - 400
+
+        def run():
+            hidden.grad = None
+            # reference order: bf16 lm_head GEMM, fp32 log_softmax + gather of the shifted labels, per-sequence
+            # sums, sigmoid DPO loss, backward to the hidden states
+            z = torch.nn.functional.linear(hidden, weight).view(2, per, vocab)
+            per_token = o_lp.calculate_per_token_logps(z, labels)
+            logps = o_red.get_batch_logps_padded(per_token, labels)
+            losses, _, _ = o_dpo.dpo_loss(logps[:1], logps[1:], ref_c, ref_r, 0.1)
+            losses.mean().backward()
+
+        sample = (f"one pair of 2 x {per} tokens (of 8 pairs of 2 x 2048) at full H={hdim}, V={vocab}, W ~ N(0, 0.01); "
+                  "fwd + bwd to the hidden states; bf16 GEMM + fp32 log_softmax + sigmoid DPO loss")
+    elif workload in ("c3", "c4"):
+        hdim = 4096
         vocab, n = (100352 if workload == "c4" else 128256), 2048
         hidden = torch.randn(n, hdim).bfloat16().requires_grad_(True)
-        weight = (torch.randn(vocab, hdim) * 0.02).bfloat16().requires_grad_(workload != "c5")
+        weight = (torch.randn(vocab, hdim) * 0.02).bfloat16().requires_grad_(True)
         labels = torch.randint(0, vocab, (n,))
         mask = torch.rand(n) < 0.7
         adv, noise = torch.randn(n), torch.randn(n)
@@ -517,15 +588,14 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="c3",
-                    choices=["c1", "c2", "c2-two-pass", "c3", "c3-one-call", "c3-slabs", "c4", "c4-slabs", "c5", "pack"])
-    ap.add_argument("--cache-chunks", type=int, default=0,
-                    help="c3 / c3-one-call / c5 only: keep 2^logit in bf16 for this many vocabulary chunks of 32768 "
-                         "columns instead of recomputing them in the backward pass (0 = the headline configuration: "
-                         "nothing of size [tokens, vocab] is stored)")
+                    choices=["c1", "c2", "c2-two-pass", "c3", "c3-recompute", "c3-one-call-recompute", "c4",
+                             "c4-recompute", "c5", "pack"])
+    ap.add_argument("--slab-tokens", type=int, default=0,
+                    help="c3 / c4 only: slab size of the no-recompute step (0 = the package's default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-library-gemm", action="store_true",
                     help="skip the reference points beside the measurement: the vendor bf16 GEMM of the same shape and, "
-                         "for c3, the timing of the opt-in cache of exponentials")
+                         "for c3, the timing of the recomputing route")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -542,30 +612,36 @@ def main():
         sys.exit(2)
     oi._lib.load()
 
+    if args.slab_tokens:
+        oi.grpo_utils.DEFAULT_SLAB_TOKENS = args.slab_tokens
+    slab_note = f"slabs of at most {oi.grpo_utils.DEFAULT_SLAB_TOKENS} selected tokens, nothing recomputed, no [tokens, vocab] tensor"
     if args.workload == "c3":
-        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02, cache_chunks=args.cache_chunks)
-        name = "c3: fused lm_head+logprob+entropy+GRPO loss fwd+bwd, hidden bf16 [32768,4096], W bf16 [128256,4096], 70% response tokens (rows selected on the device)"
+        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02)
+        name = ("c3: fused lm_head+logprob+entropy+GRPO loss fwd+bwd, hidden bf16 [32768,4096], W bf16 [128256,4096], 70% "
+                f"response tokens (rows selected on the device), through grpo_loss_on_hidden as it runs by default: {slab_note}")
         dtype = "bf16"
-    elif args.workload == "c3-one-call":
-        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02, one_call=True, cache_chunks=args.cache_chunks)
-        name = "c3: the same step through the single entry point grpo_loss_on_hidden (oi_lmhead_grpo_fwd_bwd)"
+    elif args.workload == "c3-recompute":
+        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02, route="recompute")
+        name = ("c3 through the three differentiable calls fused_lm_head_logprobs -> grpo_loss_fused -> backward: the "
+                "backward recomputes the logits one vocabulary chunk at a time (8 N H V executed for 6 N H V credited)")
         dtype = "bf16"
-    elif args.workload == "c3-slabs":
-        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02, one_call=True, token_slabs=True)
-        name = ("c3: the same step through grpo_loss_on_hidden(token_slabs=True): slabs of 8192 selected tokens, a slab's "
-                "exponentials [8192, vocab] bf16 kept between its forward and its backward products, nothing recomputed")
+    elif args.workload == "c3-one-call-recompute":
+        step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02, route="one-call-recompute")
+        name = "c3 through grpo_loss_on_hidden(token_slabs=False): the recomputing step from one C call"
         dtype = "bf16"
     elif args.workload == "c4":
         step, info = make_c4(torch, oi)
-        name = "c4: packed OLMo-2-7B shape, 16 sequences via cu_seqlens, hidden bf16 [N<=32768,4096], W bf16 [100352,4096]; per-sequence logprob sums + GRPO loss masked_mean(axis=1), fwd+bwd"
+        name = ("c4: packed OLMo-2-7B shape, 16 sequences via cu_seqlens, hidden bf16 [N<=32768,4096], W bf16 [100352,4096]; "
+                "GRPO loss masked_mean(axis=1) fwd+bwd through grpo_loss_on_hidden as it runs by default "
+                f"({slab_note}), per-sequence logprob sums from the returned logprobs")
         dtype = "bf16"
-    elif args.workload == "c4-slabs":
-        step, info = make_c4(torch, oi, token_slabs=True)
-        name = ("c4 through grpo_loss_on_hidden(token_slabs=True): packed OLMo-2-7B shape, GRPO loss masked_mean(axis=1) "
-                "fwd+bwd in slabs of 8192 tokens with nothing recomputed, per-sequence logprob sums from the returned logprobs")
+    elif args.workload == "c4-recompute":
+        step, info = make_c4(torch, oi, route="recompute")
+        name = ("c4 through the three differentiable calls: per-sequence logprob sums + GRPO loss masked_mean(axis=1), "
+                "fwd+bwd, recomputing backward")
         dtype = "bf16"
     elif args.workload == "c5":
-        step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True, cache_chunks=args.cache_chunks)
+        step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True)
         name = "c5: fused lm_head+per-sequence logprob sums+sigmoid DPO loss, hidden bf16 [32768,8192], W bf16 [128256,8192], bwd to dHidden only"
         dtype = "bf16"
     elif args.workload == "c2":
@@ -585,11 +661,6 @@ def main():
         name = "c1: logprob+entropy+masked_mean on fp32 logits [4,512,32000], forward"
         dtype = "f32"
 
-    if args.cache_chunks:
-        if args.workload not in ("c3", "c3-one-call", "c5"):
-            print("--cache-chunks applies to c3, c3-one-call and c5")
-            sys.exit(2)
-        name += f" [NOT the headline configuration: 2^logit of {args.cache_chunks} vocabulary chunk(s) kept in bf16 for the backward pass]"
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_(0, 255)
         dst = torch.empty_like(src)
@@ -632,7 +703,7 @@ def main():
         roofline["whole_step_frac"] = roofline["whole_step_tflops"] / PEAK_BF16_TFLOPS
         if not args.no_library_gemm:
             hdim = 8192 if args.workload == "c5" else 4096
-            vocab = 100352 if args.workload in ("c4", "c4-slabs") else 128256
+            vocab = 100352 if args.workload in ("c4", "c4-recompute") else 128256
             roofline["library_bf16_gemm_tflops"] = library_gemm_tflops(torch, 32768, hdim, vocab)
     if "bytes_step" in info:
         roofline["whole_step_gbs"] = info["bytes_step"] / (ms_per_step * 1e-3) / 1e9
@@ -659,52 +730,34 @@ def main():
         },
         "roofline": roofline,
     }
-    if args.workload == "c3" and not args.cache_chunks and not args.no_library_gemm:
-        # reported beside the headline figure, never as `value`: the same step with 2^logit of all four
-        # vocabulary chunks kept in bf16 between the passes (8.4 GB) instead of being recomputed
+    if args.workload == "c3" and not args.no_library_gemm:
+        # reported beside the headline figure: the same step through the three differentiable calls, whose
+        # backward recomputes the logits (what a caller gets who needs the autograd seam between forward and loss)
         del step
         torch.cuda.empty_cache()
-        step_c, info_c = make_fused(torch, oi, 32768, 4096, 128256, 0.02, cache_chunks=4)
+        step_r, info_r = make_fused(torch, oi, 32768, 4096, 128256, 0.02, route="recompute")
         for _ in range(args.warmup):
-            step_c()
+            step_r()
         torch.cuda.synchronize()
+        info_r["timer"].reset()
         t0 = time.perf_counter()
         for _ in range(args.steps):
-            step_c()
+            step_r()
         torch.cuda.synchronize()
-        ms_c = (time.perf_counter() - t0) * 1e3 / args.steps
-        line["opt_in_variants"] = {
-            "cache_of_exponentials_4_chunks": {
-                "ms_per_step": ms_c,
-                "tokens_per_s": info_c["tokens"] / (ms_c * 1e-3),
-                "whole_step_frac": info_c["flops_step"] / (ms_c * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
-                "extra_hbm_bytes": 8.4e9,
-                "note": "not the headline configuration: the backward multiplies stored exponentials instead of "
-                        "recomputing the logits",
+        ms_r = (time.perf_counter() - t0) * 1e3 / args.steps
+        fwd_ms = info_r["timer"].mean_ms()
+        line["other_routes"] = {
+            "recompute_three_calls": {
+                "ms_per_step": ms_r,
+                "tokens_per_s": info_r["tokens"] / (ms_r * 1e-3),
+                "whole_step_frac": info_r["flops_step"] / (ms_r * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                "forward_kernel_ms": fwd_ms,
+                "forward_kernel_frac": info_r["alg_per_launch"] / (fwd_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                "note": "fused_lm_head_logprobs -> grpo_loss_fused -> backward: the backward recomputes the logits "
+                        "(8 N H V executed, 6 N H V credited)",
             }
         }
-        del step_c
-        torch.cuda.empty_cache()
-        # the same step in slabs of 8192 selected tokens through the one-call entry: a slab's exponentials are
-        # kept between its forward and its backward products ([8192, vocab] bf16 at a time), nothing is recomputed
-        step_s, info_s = make_fused(torch, oi, 32768, 4096, 128256, 0.02, one_call=True, token_slabs=True)
-        for _ in range(args.warmup):
-            step_s()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step_s()
-        torch.cuda.synchronize()
-        ms_s = (time.perf_counter() - t0) * 1e3 / args.steps
-        line["opt_in_variants"]["token_slabs_one_call"] = {
-            "ms_per_step": ms_s,
-            "tokens_per_s": info_s["tokens"] / (ms_s * 1e-3),
-            "whole_step_frac": info_s["flops_step"] / (ms_s * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
-            "extra_hbm_bytes": 8192 * 128256 * 2 + 128256 * 4096 * 4,
-            "note": "not the headline configuration: grpo_loss_on_hidden(token_slabs=True), no recomputation, no "
-                    "[tokens, vocab] tensor",
-        }
-        del step_s
+        del step_r
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, args.workload)
     print(json.dumps(line), flush=True)

@@ -353,25 +353,7 @@ int oi_pack_sequences(const int64_t* q_tokens, const int64_t* q_offsets, const i
 size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int with_row_mask);
 int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* labels, const uint8_t* row_mask,
                        int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob,
-                       float* entropy, float* lse, void* exp_cache, int64_t cache_chunks, void* workspace,
-                       size_t workspace_bytes, void* stream);
-
-/*
- * Optional cache of exponentials (cache_chunks > 0; 0 = off, the default of the Python mirror: the
- * backward then recomputes every chunk and nothing of size [tokens, vocab] exists).  It trades memory
- * for the recomputation: the forward also stores 2^(z * inv_T * log2 e) in bf16 (whose exponent
- * range is that of fp32, so no per-token reference is needed) for the first cache_chunks chunks of
- * 32768 vocabulary columns, token-major, oi_lmhead_cache_bytes() bytes at exp_cache (16-byte aligned,
- * owned by the caller, handed unchanged to the backward call of the same rows).  For a cached chunk
- * the backward multiplies the cache itself: dZ[n, v] = s_n (e'[n, v] - 1[v = label_n] 2^lse2_n) with
- * the per-token factor s_n = -g_n inv_T 2^(-lse2_n) moved out of the products (a row factor of
- * d_hidden, a factor of the hidden rows in d_weight), and the label's entry replaced by
- * 2^lse2_n * expm1(logprob_n).  Costs 2 bytes per cached logit (8.4 GB for all four chunks at
- * 32768 x 128256), saves a quarter of the step's matrix work when every chunk is cached.  Needs
- * |z * inv_T| < 87 (2^126); the rounding of a cached entry is the bf16 rounding that a dZ entry
- * undergoes anyway.
- */
-size_t oi_lmhead_cache_bytes(int64_t n_tokens, int64_t vocab, int64_t cache_chunks);
+                       float* entropy, float* lse, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Backward: recomputes the logits tile by tile,
@@ -381,49 +363,65 @@ size_t oi_lmhead_cache_bytes(int64_t n_tokens, int64_t vocab, int64_t cache_chun
  * Vocabulary is processed in chunks of 32768 columns; only one chunk of dZ (bf16, token-major)
  * lives in the workspace at a time, next to the fp32 accumulator of d_hidden.  Both products
  * read weight, hidden and dZ where they lie (no transposed copies), so the workspace is the same
- * with and without d_weight (cached chunks are multiplied as one chunk; with every chunk cached
- * neither the dZ chunk nor the fp32 accumulator is part of the workspace).  row_mask as in the forward (rows left out get a zero d_hidden row
+ * with and without d_weight.  row_mask as in the forward (rows left out get a zero d_hidden row
  * and add nothing to d_weight); skip_zero_grad_rows != 0 also leaves out rows whose grad_logprob is
- * exactly 0, which changes no result (not together with a cache, whose rows are the forward's).
+ * exactly 0, which changes no result.
  * d_hidden and d_weight must be 4-byte aligned.  logprob is the forward's output for the same rows:
  * the label's entry of dZ is taken from it as -grad * inv_T * expm1(logprob), which stays exact
  * where the label's probability is close to 1.
  */
 size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int want_d_weight,
-                                     int with_row_selection, int64_t cache_chunks);
+                                     int with_row_selection);
 int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
                        const float* grad_logprob, const uint8_t* row_mask, int skip_zero_grad_rows, int64_t n_tokens,
-                       int64_t hidden_dim, int64_t vocab, float inv_temperature, const float* logprob,
-                       void* exp_cache, int64_t cache_chunks, void* d_hidden, void* d_weight, void* workspace,
-                       size_t workspace_bytes, void* stream);
+                       int64_t hidden_dim, int64_t vocab, float inv_temperature, const float* logprob, void* d_hidden,
+                       void* d_weight, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Kept exponentials (what the two entry-point families below share).  The forward evaluates
+ * 2^(x[n,v] - max) for its statistics anyway (x = z * inv_T * log2 e); where a backward pass follows
+ * that can use them, it also stores them, as bf16, relative to a per-token reference exponent:
+ *   e'[n, v] = 2^(x[n,v] - xref[n]),   xref[n] = x[n, label_n]  (a dot product taken beforehand),
+ * so that dZ[n, v] = s_n * (e'[n, v] - 1[v = label_n] * 2^(lse2_n - xref[n])) with the per-token
+ * factor s_n = -g_n * inv_T * 2^(xref[n] - lse2_n) moved out of the products and the label's entry
+ * rebuilt from the fp32 logprob.  Relative to the label's own logit the stored numbers and the
+ * factor stay inside the bf16 / fp32 range whatever the magnitude of the logits and the
+ * temperature, as long as the token's largest logit is less than 64 binary orders (44 nats) above
+ * its label's.  A token beyond that (a label of probability below about e^-44), or whose logits hold
+ * a NaN, is flagged on the device and served by the recomputing backward instead, inside the same
+ * call and without a host read: results are those of the reference's exact log_softmax
+ * (open_instruct/padding_free_collator.py:10-16, open_instruct/model_utils.py:587-600) either way.
+ */
 
 /*
  * Forward + backward for callers that need d_hidden only (a frozen lm_head: the DPO / reward passes of
  * open_instruct/dpo_utils.py:959-1019 through DPOLMHead when the head's weight takes no gradient, or
- * any d_weight == NULL use of oi_lmhead_logp_bwd).  With x = z * inv_T * log2 e,
- *   d_hidden[n] = s_n * sum_{v != label_n} 2^x[n,v] * weight[v]  -  g_n * inv_T * expm1(logprob_n) * weight[label_n],
- *   s_n = -g_n * inv_T * 2^(-lse_n * log2 e),
+ * any d_weight == NULL use of oi_lmhead_logp_bwd).  With e' and xref as above,
+ *   d_hidden[n] = s_n * sum_{v != label_n} e'[n,v] * weight[v]  -  g_n * inv_T * expm1(logprob_n) * weight[label_n],
  * and the sum does not depend on the upstream gradient g: oi_lmhead_logp_fwd_wsum computes it together
  * with logprob / entropy / lse while the logits exist (one chunk of 65536 vocabulary columns at a
  * time: the chunk's exponentials as bf16 in the workspace, then wsum (+)= E_chunk @ weight_chunk in
  * fp32), and oi_lmhead_dh_from_wsum turns it into d_hidden in one pass over [n_tokens, hidden_dim].
  * Matrix work of forward + backward: 4 N H V instead of 6 N H V, nothing is recomputed, nothing of size
- * [tokens, vocab] exists.  Needs |z * inv_T| < 87 like the cache of exponentials.
- * wsum: fp32 [n_tokens, hidden_dim], 16-byte aligned, owned by the caller between the two calls; row j
- * belongs to the j-th selected row (rows in ascending order; every row without a row_mask).  The
- * backward call takes the same labels / row_mask and the forward's lse and logprob; rows left out
- * get a zero d_hidden row.  d_hidden: bf16 [n_tokens, hidden_dim], 8-byte aligned.  The workspace of
- * the backward call is only read with a row_mask (it may be NULL otherwise).
+ * [tokens, vocab] exists.
+ * wsum: fp32 [n_tokens, hidden_dim], 16-byte aligned; xref: fp32 [n_tokens]; unsafe: one byte per
+ * token (set for flagged tokens): all three are outputs of the forward call that the caller holds
+ * until the backward call.  Row j of wsum / xref belongs to the j-th selected row (rows in ascending
+ * order; every row without a row_mask), unsafe is indexed like the caller's rows.  The backward call
+ * takes the same hidden / labels / row_mask and the forward's lse and logprob; rows left out get a zero
+ * d_hidden row, flagged rows are recomputed (the workspace holds the recomputing backward's buffers,
+ * which are only touched for such rows).  d_hidden: bf16 [n_tokens, hidden_dim], 8-byte aligned.
  */
 size_t oi_lmhead_fwd_wsum_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab, int with_row_mask);
 int oi_lmhead_logp_fwd_wsum(const void* hidden, const void* weight, const int64_t* labels, const uint8_t* row_mask,
                             int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob,
-                            float* entropy, float* lse, float* wsum, void* workspace, size_t workspace_bytes,
-                            void* stream);
-size_t oi_lmhead_dh_workspace_bytes(int64_t n_tokens);
-int oi_lmhead_dh_from_wsum(const void* weight, const int64_t* labels, const float* lse, const float* logprob,
-                           const float* grad_logprob, const uint8_t* row_mask, const float* wsum, int64_t n_tokens,
-                           int64_t hidden_dim, int64_t vocab, float inv_temperature, void* d_hidden, void* workspace,
+                            float* entropy, float* lse, float* wsum, float* xref, uint8_t* unsafe, void* workspace,
+                            size_t workspace_bytes, void* stream);
+size_t oi_lmhead_dh_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab);
+int oi_lmhead_dh_from_wsum(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
+                           const float* logprob, const float* grad_logprob, const uint8_t* row_mask, const float* wsum,
+                           const float* xref, const uint8_t* unsafe, int64_t n_tokens, int64_t hidden_dim,
+                           int64_t vocab, float inv_temperature, void* d_hidden, void* workspace,
                            size_t workspace_bytes, void* stream);
 
 /*
@@ -442,25 +440,44 @@ int oi_lmhead_dh_from_wsum(const void* weight, const int64_t* labels, const floa
  * [rows, cols], 0 off the mask.  d_weight NULL skips that product.  A token's upstream gradient
  * depends only on its own logprob once the denominators are known, and those come from the mask, so
  * the backward is enqueued straight behind the forward: nothing returns to the host in between.
- * exp_cache / cache_chunks: the optional cache of exponentials described at oi_lmhead_cache_bytes
- * (scratch of this one call here; NULL / 0 = recompute every chunk).
- * cache_chunks < 0 (exp_cache ignored): the step runs in slabs of -cache_chunks * 4096 selected tokens and
- * recomputes nothing.  A slab's forward leaves its exponentials (every vocabulary column, bf16) in a slab-sized
- * buffer inside the workspace, the slab's tokens get their upstream gradient at once, and both
- * products read the buffer before the next slab overwrites it: d_hidden rows are final, d_weight
- * accumulates in fp32 over the slabs (deterministic: slab after slab) and is rounded to bf16 once.
- * 6 N H V of matrix work instead of 8 N H V; the workspace holds [slab, vocab] bf16 and, with
- * d_weight, an fp32 [vocab, hidden_dim], never anything of size [tokens, vocab].
+ *
+ * slab_tokens == 0: one forward over all selected rows, then the recomputing backward of
+ * oi_lmhead_logp_bwd (8 N H V of matrix work).
+ * slab_tokens > 0 (rounded up to a multiple of 256): the step runs in slabs of at most that many
+ * selected tokens and recomputes nothing.  The selected rows are split on the device into the fewest
+ * equal slabs; a slab's forward leaves its kept exponentials (every vocabulary column, bf16, see
+ * above) in a slab-sized buffer inside the workspace, the slab's tokens get their upstream gradient
+ * at once, and both products read the buffer before the next slab overwrites it: d_hidden rows are
+ * final, d_weight accumulates in fp32 over the slabs (deterministic: slab after slab) and is rounded
+ * to bf16 once.  6 N H V of matrix work instead of 8 N H V; the workspace holds [slab, vocab] bf16 and,
+ * with d_weight and more than one slab, an fp32 [vocab, hidden_dim], never anything of size
+ * [tokens, vocab].  Flagged tokens (see above) are recomputed after the last slab.
+ * oi_lmhead_grpo_workspace_bytes takes the same slab_tokens and whether d_weight is wanted.
  */
 size_t oi_lmhead_grpo_workspace_bytes(int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab,
-                                      int64_t cache_chunks);
+                                      int want_d_weight, int64_t slab_tokens);
 int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, const int64_t* labels, const uint8_t* mask,
                            const float* old_logprobs, const float* ref_logprobs, const float* advantages,
                            const float* rho_weights, int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab,
                            float inv_temperature, int loss_fn, float ratio_lo, float ratio_hi, int kl_estimator,
                            float beta, int axis_mode, float denominator, float scale, float* logprob, float* entropy,
-                           float* out_stats, void* d_hidden, void* d_weight, void* exp_cache, int64_t cache_chunks,
-                           void* workspace, size_t workspace_bytes, void* stream);
+                           float* out_stats, void* d_hidden, void* d_weight, int64_t slab_tokens, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/*
+ * Timing probe of the slab-wise entry points (no reference counterpart; it exists for the
+ * measurement harness, which has to time one kernel inside a call that launches several).  Between
+ * oi_lmhead_probe_arm(kernel) and oi_lmhead_probe_read the slab-wise calls of this process record a
+ * pair of HIP events, on the stream of the call, around every launch of the chosen tile kernel:
+ * 0 = the forward that keeps its exponentials, 1 = the d_hidden product, 2 = the d_weight product
+ * (at most 256 launches; later ones are not recorded).  oi_lmhead_probe_read waits for the recorded
+ * events, writes the duration of each recorded launch in milliseconds to ms[0 .. min(n, capacity)),
+ * the number of recorded launches to *n_launches, and disarms the probe.  Launches whose slab is
+ * empty are recorded too (they take a few microseconds).  Not thread-safe; do not arm it around a
+ * call that is captured into a graph.
+ */
+int oi_lmhead_probe_arm(int kernel);
+int oi_lmhead_probe_read(float* ms, int capacity, int* n_launches);
 
 /*
  * The bf16 MFMA main loop of the lm_head kernels as a plain product (no reference counterpart;

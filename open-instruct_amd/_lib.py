@@ -60,22 +60,20 @@ SIGNATURES: dict[str, tuple] = {
     "oi_dpo_sigmoid_bwd": (_I, [_P, _P, _P, _P, _P, _P, _I64, _F, _F, _F, _P, _P, _P]),
     "oi_pack_sequences": (_I, [_P] * 9 + [_I64, _I64, _I] + [_P] * 8),
     "oi_lmhead_fwd_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I]),
-    "oi_lmhead_logp_fwd": (_I, [_P, _P, _P, _P, _I64, _I64, _I64, _F, _P, _P, _P, _P, _I64, _P, _SZ, _P]),
-    "oi_lmhead_cache_bytes": (_SZ, [_I64, _I64, _I64]),
-    "oi_lmhead_bwd_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I, _I, _I64]),
-    "oi_lmhead_logp_bwd": (
-        _I,
-        [_P, _P, _P, _P, _P, _P, _I, _I64, _I64, _I64, _F, _P, _P, _I64, _P, _P, _P, _SZ, _P],
-    ),
+    "oi_lmhead_logp_fwd": (_I, [_P, _P, _P, _P, _I64, _I64, _I64, _F, _P, _P, _P, _P, _SZ, _P]),
+    "oi_lmhead_bwd_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I, _I]),
+    "oi_lmhead_logp_bwd": (_I, [_P, _P, _P, _P, _P, _P, _I, _I64, _I64, _I64, _F, _P, _P, _P, _P, _SZ, _P]),
     "oi_lmhead_fwd_wsum_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I]),
-    "oi_lmhead_logp_fwd_wsum": (_I, [_P, _P, _P, _P, _I64, _I64, _I64, _F, _P, _P, _P, _P, _P, _SZ, _P]),
-    "oi_lmhead_dh_workspace_bytes": (_SZ, [_I64]),
-    "oi_lmhead_dh_from_wsum": (_I, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _F, _P, _P, _SZ, _P]),
-    "oi_lmhead_grpo_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I64, _I64]),
+    "oi_lmhead_logp_fwd_wsum": (_I, [_P, _P, _P, _P, _I64, _I64, _I64, _F, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "oi_lmhead_dh_workspace_bytes": (_SZ, [_I64, _I64, _I64]),
+    "oi_lmhead_dh_from_wsum": (_I, [_P] * 10 + [_I64, _I64, _I64, _F, _P, _P, _SZ, _P]),
+    "oi_lmhead_grpo_workspace_bytes": (_SZ, [_I64, _I64, _I64, _I64, _I, _I64]),
     "oi_lmhead_grpo_fwd_bwd": (
         _I,
-        [_P] * 8 + [_I64, _I64, _I64, _I64, _F, _I, _F, _F, _I, _F, _I, _F, _F] + [_P] * 6 + [_I64, _P, _SZ, _P],
+        [_P] * 8 + [_I64, _I64, _I64, _I64, _F, _I, _F, _F, _I, _F, _I, _F, _F] + [_P] * 5 + [_I64, _P, _SZ, _P],
     ),
+    "oi_lmhead_probe_arm": (_I, [_I]),
+    "oi_lmhead_probe_read": (_I, [_P, _I, _P]),
     "oi_gemm_bf16_tn": (_I, [_P, _I64, _I64, _P, _I64, _I64, _I64, _P, _P, _I64, _I, _P]),
     "oi_gemm_bf16_layouts": (_I, [_P, _I64, _I, _P, _I64, _I, _I64, _I64, _I64, _P, _P, _I64, _I, _P]),
 }

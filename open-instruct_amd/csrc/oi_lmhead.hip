@@ -92,6 +92,9 @@ __device__ __forceinline__ void for_each_tile(uint32_t* __restrict__ counters, i
     // thread 0 only: the queues of XCDs xcd .. xcd + dry - 1 (mod 8) are known to be empty and
     // `drawn` came from the queue of XCD xcd + dry
     uint32_t dry = 0, drawn = 0;
+    // a kernel may run several of these loops back to back over the same word: every wave must have
+    // read the previous loop's last value before thread 0 writes this loop's first one
+    __syncthreads();
     auto resolve = [&]() -> uint32_t {
         for (;;) {
             if (drawn < locals) return drawn * 8 + ((xcd + dry) & 7);
@@ -456,12 +459,16 @@ __device__ __forceinline__ void merge_stats(float ma, float sa, float ta, float 
 // Fold the 32 logits that one lane holds for token column j of a finished tile into the running
 // statistics.  PARTIAL handles the last vocabulary tile: rows past the vocabulary are skipped by
 // predicate (weight exactly 0) instead of through a sentinel value.
-// KEEP leaves 2^x in place of every logit (0 for rows past the vocabulary): the exponentials of the
-// statistics times 2^max, for the cache of exponentials that the backward pass can use in place of
-// a recomputation.
+// KEEP leaves 2^(x - ref) in place of every logit (0 for rows past the vocabulary): the exponentials
+// of the statistics times 2^(max - ref), which the backward products can use in place of a
+// recomputation.  `ref` is the token's reference exponent (the scaled logit of its own label, known
+// before the tile is computed): relative to it the kept numbers stay inside the bf16 range whatever
+// the magnitude of the logits, as long as the token's largest logit is less than KEEP_MAX_LOG2
+// binary orders above its label's (tokens beyond that are flagged by the merge kernel and take the
+// recomputing backward).
 template <bool PARTIAL, bool KEEP>
 __device__ __forceinline__ void stats_update(AccTile& acc, int j, int wm, int lane, int64_t m0, int64_t vocab, float c,
-                                             float& st_m, float& st_s, float& st_t) {
+                                             float ref, float& st_m, float& st_s, float& st_t) {
     // the maximum is taken over the unscaled logits (c > 0) and every exponent is one fma: the new
     // maximum is the rounded product max(z) * c while the exponents are rounded once, so the largest
     // term is 2^(a few ulp) rather than exactly 1, far below the accuracy of the sums
@@ -476,7 +483,7 @@ __device__ __forceinline__ void stats_update(AccTile& acc, int j, int wm, int la
     const float alpha = __builtin_amdgcn_exp2f(shift);
     float s = st_s * alpha;
     float t = alpha * fmaf(shift, st_s, st_t);
-    const float pow2_max = KEEP ? __builtin_amdgcn_exp2f(fminf(mn, 126.f)) : 0.f;
+    const float pow2_max = KEEP ? __builtin_amdgcn_exp2f(fminf(mn - ref, 126.f)) : 0.f;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -531,9 +538,8 @@ __device__ __forceinline__ void copy_staged_tile(const uint16_t* stage, uint16_t
 // ---------------------------------------------------------------------------------------------
 // forward: per-token softmax statistics over the vocabulary tiles of one split
 // ---------------------------------------------------------------------------------------------
-// CACHE: the first cache_tiles vocabulary tiles also leave 2^(z c) behind as bf16, token-major
-// [n_pad, cache_ld] (bf16 has the exponent range of fp32, so no per-token reference is needed);
-// rows of tokens past the end are zero.
+// CACHE: the vocabulary tiles [cache_tile0, cache_tile0 + cache_tiles) also leave 2^(z c - xref[n])
+// behind as bf16, token-major [n_pad, cache_ld]; rows of tokens past the end are zero.
 // What a forward launch covers and where its exponentials go.  Splits [0, long_splits) take
 // tiles_per_split vocabulary tiles each, the others one.  A launch hands out the long splits
 // [first, first + n_first) from one set of queues and then the short splits
@@ -545,6 +551,7 @@ struct FwdLaunch {
     uint16_t* ecache;
     int64_t cache_ld, cache_tile0, cache_tiles;
     int skip_label;
+    const float* xref;  // per token: the exponent that the kept exponentials are relative to (null: 0)
 };
 
 template <bool CACHE>
@@ -564,7 +571,7 @@ __device__ __forceinline__ void lmhead_fwd_item(const uint16_t* __restrict__ W, 
     const int tid = opaque_tid(), lane = tid & 63, wave = tid >> 6, wm = wave & 3, wn = wave >> 2;
     const int64_t n0 = tt * BN;
 
-    float st_m[4], st_s[4], st_t[4];
+    float st_m[4], st_s[4], st_t[4], ref[4];
     int lab[4];  // vocabulary ids fit 32 bits (vocab <= 2^22)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -574,6 +581,7 @@ __device__ __forceinline__ void lmhead_fwd_item(const uint16_t* __restrict__ W, 
         const int64_t n = n0 + acc_col(wn, j, lane);
         int64_t y = n < n_tokens ? labels[n] : 0;
         lab[j] = (int)(y < 0 ? 0 : (y >= vocab ? vocab - 1 : y));
+        ref[j] = (CACHE && fl.xref && n < n_tokens) ? fl.xref[n] : 0.f;
     }
 
     for (int64_t vt = vt_begin; vt < vt_end; ++vt) {
@@ -603,9 +611,9 @@ __device__ __forceinline__ void lmhead_fwd_item(const uint16_t* __restrict__ W, 
                 if (n < n_tokens) zy[n] = v;
             }
             if (partial_tile)
-                stats_update<true, CACHE>(acc, j, wm, lane, m0, vocab, c, st_m[j], st_s[j], st_t[j]);
+                stats_update<true, CACHE>(acc, j, wm, lane, m0, vocab, c, ref[j], st_m[j], st_s[j], st_t[j]);
             else
-                stats_update<false, CACHE>(acc, j, wm, lane, m0, vocab, c, st_m[j], st_s[j], st_t[j]);
+                stats_update<false, CACHE>(acc, j, wm, lane, m0, vocab, c, ref[j], st_m[j], st_s[j], st_t[j]);
             if (CACHE && fl.skip_label && label_reg >= 0) {
 #pragma unroll
                 for (int i = 0; i < 2; ++i)
@@ -675,16 +683,26 @@ __global__ void __launch_bounds__(NTHREADS)
     });
 }
 
+// A token whose largest scaled logit lies more than this many binary orders above its reference
+// exponent is not served from kept exponentials (they would leave the bf16 range, or the factor
+// that undoes the reference would): 2^64 leaves room for the fp32 sums over the vocabulary above it
+// and for the per-token factor 2^(ref - lse2) >= 2^-(64 + 22) below it.
+constexpr float KEEP_MAX_LOG2 = 64.f;
+
 // Merges the partial statistics of token n over the vocabulary splits.  With a row selection
 // (`rows` non-null) token n of the compacted batch is row rows[n] of the caller's tensors, the count
 // comes from the device, and the rows that were left out are written as zeros: the grid covers
 // n_total rows, thread i handles compacted token i and caller row i.
+// `unsafe` (one byte per caller row, optional, cleared by the caller beforehand): set for a token
+// whose kept exponentials cannot be trusted (its maximum is too far above xref[n], or is not a
+// number); never cleared here, so marks that the caller has put there survive.
 __global__ void lmhead_fwd_combine_kernel(const float4* __restrict__ partial, const float* __restrict__ zy,
                                           int64_t n_tokens, const int32_t* __restrict__ n_dev,
                                           const int32_t* __restrict__ rows, const uint8_t* __restrict__ row_mask,
-                                          int64_t n_total, int64_t n_splits, int64_t n_pad, float inv_t,
+                                          int64_t n_total, int64_t n_splits, int64_t n_pad, float inv_t, float c,
                                           float* __restrict__ logprob, float* __restrict__ entropy,
-                                          float* __restrict__ lse_out) {
+                                          float* __restrict__ lse_out, const float* __restrict__ xref,
+                                          uint8_t* __restrict__ unsafe) {
     const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (n_dev) n_tokens = *n_dev;
     if (row_mask && n < n_total && !row_mask[n]) {
@@ -700,11 +718,15 @@ __global__ void lmhead_fwd_combine_kernel(const float4* __restrict__ partial, co
     }
     const double ln2 = 0.69314718055994530942;
     const double log2s = log2((double)s);
-    const double lse = ((double)m + log2s) * ln2;
+    // the statistics are in units of x = z * c with the fp32 constant c the tile kernel multiplied by:
+    // back to nats through that very constant (inv_t / c, not the literal ln 2), so that the logprob of
+    // a token whose label holds all of the probability comes out as 0 at any size of the logits
+    const double lse = ((double)m + log2s) * ((double)inv_t / (double)c);
     const int64_t o = rows ? rows[n] : n;
     logprob[o] = (float)((double)zy[n] * (double)inv_t - lse);
     if (entropy) entropy[o] = (float)((log2s - (double)t / (double)s) * ln2);
     if (lse_out) lse_out[o] = (float)lse;
+    if (unsafe && !(m - (xref ? xref[n] : 0.f) <= KEEP_MAX_LOG2)) unsafe[o] = 1;  // a NaN maximum is flagged too
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -808,6 +830,7 @@ __global__ void __launch_bounds__(NTHREADS)
 // ---------------------------------------------------------------------------------------------
 // mode 0: out_f32  = acc          mode 1: out_f32 += acc
 // mode 2: out_bf16 = acc          mode 3: out_bf16 = out_f32 + acc   (last chunk of d_hidden)
+// mode 4: out_bf16 += acc         (rows added to a d_weight that was already rounded)
 // A, B: operands without their tile origin (r0 is filled in here); the product has M x N
 // entries, of which rows below m_valid are stored.  K == 0 stores zeros.  With `out_rows`, row r
 // of a bf16 result goes to row out_rows[r] of out_bf16 (the fp32 accumulator stays compact).
@@ -822,7 +845,7 @@ __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B,
     A.r0 = m0;
     B.r0 = n0;
     AccTile acc;
-    if (K <= 0 && mode == 1) return;  // nothing to add
+    if (K <= 0 && (mode == 1 || mode == 4)) return;  // nothing to add
     if (K > 0) {
         gemm_tile<A_KM, B_KM>(acc, A, B, K, lds);
     } else {
@@ -858,8 +881,10 @@ __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B,
                     float lo = odd ? recv : own0, hi = odd ? own1 : recv;
                     if (!row_ok || col >= N) continue;
                     if (scale_a) {
-                        lo = lo * sa * sb;
-                        hi = hi * sa * sb;
+                        // a row whose factor is exactly 0 is 0 whatever its sum holds (the sums of
+                        // rows that were taken out may have left the fp32 range)
+                        lo = sb == 0.f ? 0.f : lo * sa * sb;
+                        hi = sb == 0.f ? 0.f : hi * sa * sb;
                     }
                     const int64_t o = row * ldo + col, d = dst_row * ldo + col;
                     if (col + 1 < N) {
@@ -867,10 +892,15 @@ __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B,
                             const float2 part = *reinterpret_cast<const float2*>(out_f32 + o);
                             lo += part.x;
                             hi += part.y;
+                        } else if (mode == 4) {
+                            const uint32_t prev = *reinterpret_cast<const uint32_t*>(out_bf16 + d);
+                            lo += oi_bf16lo_to_f32(prev);
+                            hi += oi_bf16hi_to_f32(prev);
                         }
                         *reinterpret_cast<uint32_t*>(out_bf16 + d) = oi_pack_bf16x2(lo, hi);
                     } else {
                         if (mode == 3) lo += out_f32[o];
+                        else if (mode == 4) lo += oi_bf16lo_to_f32((uint32_t)out_bf16[d]);
                         out_bf16[d] = (uint16_t)oi_f32_to_bf16_bits(lo);
                     }
                 }
@@ -889,7 +919,7 @@ __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B,
                 if (row >= m_valid) continue;
                 const int64_t o = row * ldo + col;
                 float v = acc[i][j][r];
-                if (scale_a) v = v * scale_a[row] * scale_b[row];
+                if (scale_a) v = scale_b[row] == 0.f ? 0.f : v * scale_a[row] * scale_b[row];
                 if (mode == 1) {
                     // the addition is done by the L2 (no load to wait for: 8.2 -> 6.9 ms per d_weight slab product);
                     // every element has one writer per launch and the launches follow each other on
@@ -898,8 +928,13 @@ __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B,
                     continue;
                 }
                 if (mode == 3) v += out_f32[o];
-                if (mode == 0) out_f32[o] = v;
-                else out_bf16[(out_rows ? (int64_t)out_rows[row] : row) * ldo + col] = (uint16_t)oi_f32_to_bf16_bits(v);
+                if (mode == 0) {
+                    out_f32[o] = v;
+                    continue;
+                }
+                const int64_t d = (out_rows ? (int64_t)out_rows[row] : row) * ldo + col;
+                if (mode == 4) v += oi_bf16lo_to_f32((uint32_t)out_bf16[d]);
+                out_bf16[d] = (uint16_t)oi_f32_to_bf16_bits(v);
             }
         }
 }
@@ -954,6 +989,10 @@ inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 __global__ void zero_words_kernel(uint32_t* __restrict__ p, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0u;
+}
+__global__ void zero_bytes_kernel(uint8_t* __restrict__ p, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1022,50 +1061,111 @@ __global__ void __launch_bounds__(256)
     }
 }
 
-// Backward from the cache of exponentials e'[n, v] = 2^(x_nv), x = z c:
-//   dZ[n, v] = g_n inv_T (1[v = y_n] - 2^(x_nv - lse2_n)) = s_n (e'[n, v] - 1[v = y_n] 2^lse2_n),
-//   s_n = -g_n inv_T 2^(-lse2_n).
-// The per-token factor leaves the products: d_hidden[n] = s_n (e'[n, :] W) (a row factor in the
-// store epilogue) and d_weight = e'^T (s h) (the hidden rows are scaled once).  This kernel writes
-// the two halves of s_n (so that neither leaves the fp32 range) and replaces the label's entry of
-// the cache by 2^x_y - 2^lse2 = 2^lse2 expm1(logprob), evaluated in fp32 from the forward's result.
-__global__ void cache_rows_prepare_kernel(const float* __restrict__ lse, const float* __restrict__ grad,
-                                          const float* __restrict__ logprob, const int64_t* __restrict__ labels,
-                                          const int32_t* __restrict__ n_dev, int64_t n_tokens, float inv_t,
-                                          int64_t vocab, uint16_t* __restrict__ ecache, int64_t cache_ld,
-                                          float* __restrict__ scale_a, float* __restrict__ scale_b) {
-    const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+// xref[j] = c * <hidden[j, :], W[label_j, :]>: the scaled logit of token j's own label, the exponent
+// that the token's kept exponentials are relative to.  It needs to be close to the token's largest
+// scaled logit, not equal to it (the same number is taken out again wherever the exponentials are
+// used), so the summation order of this dot product does not matter.  One wave per token.
+__global__ void __launch_bounds__(256)
+    label_ref_kernel(const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ W,
+                     const int64_t* __restrict__ labels, const int32_t* __restrict__ n_dev, int64_t n_tokens,
+                     int64_t hdim, int64_t vocab, float c, float* __restrict__ xref) {
+    const int lane = threadIdx.x & 63;
+    const int64_t j = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (n_dev) n_tokens = *n_dev;
-    if (n >= n_tokens) return;
-    const float l2 = lse[n] * OI_LOG2E;
-    const float half = __builtin_amdgcn_exp2f(-0.5f * l2);
-    scale_a[n] = half;
-    scale_b[n] = -grad[n] * inv_t * half;
-    int64_t y = labels[n];
+    if (j >= n_tokens) return;
+    int64_t y = labels[j];
     y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
-    if (y < cache_ld)
-        ecache[n * cache_ld + y] =
-            (uint16_t)oi_f32_to_bf16_bits(__builtin_amdgcn_exp2f(fminf(l2, 126.f)) * expm1f(logprob[n]));
+    const oi_u32x4* a = reinterpret_cast<const oi_u32x4*>(hidden + j * hdim);
+    const oi_u32x4* b = reinterpret_cast<const oi_u32x4*>(W + y * hdim);
+    float acc = 0.f;
+    for (int64_t p = lane; p < hdim / 8; p += OI_WAVE) {  // hdim is a multiple of 64
+        const oi_u32x4 av = a[p], bv = b[p];
+        const uint32_t aw[4] = {av.x, av.y, av.z, av.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            acc = fmaf(oi_bf16lo_to_f32(aw[k]), oi_bf16lo_to_f32(bw[k]), acc);
+            acc = fmaf(oi_bf16hi_to_f32(aw[k]), oi_bf16hi_to_f32(bw[k]), acc);
+        }
+    }
+    acc = oi_wave_sum(acc);
+    if (lane == 0) xref[j] = acc * c;
 }
 
-// scaled[n, :] = (hidden[n, :] * a_n) * b_n in bf16, one workgroup per row
+// Which rows a slab pass works on: rows order[offset .. offset + count) of a row index that lives
+// on the device.  Written by a planning kernel, read by every kernel of the pass.
+struct SlabMeta {
+    int32_t offset, count;
+};
+
+// Workgroup j copies row order[meta->offset + j] into the slab's own buffers: the hidden-state row
+// (hdim bf16, 16-byte pieces), its label, its row number and, when given, its logsumexp, upstream
+// gradient and logprob.
 __global__ void __launch_bounds__(256)
-    scale_rows_kernel(const uint16_t* __restrict__ hidden, const float* __restrict__ scale_a,
-                      const float* __restrict__ scale_b, const int32_t* __restrict__ n_dev, int64_t n_tokens,
-                      int64_t hdim, uint16_t* __restrict__ scaled) {
-    const int64_t n = blockIdx.x;
-    if (n_dev) n_tokens = *n_dev;
-    if (n >= n_tokens) return;
-    const float a = scale_a[n], b = scale_b[n];
-    const oi_u32x4* from = reinterpret_cast<const oi_u32x4*>(hidden + n * hdim);
-    oi_u32x4* to = reinterpret_cast<oi_u32x4*>(scaled + n * hdim);
+    gather_slab_kernel(const uint16_t* __restrict__ hidden, const int64_t* __restrict__ labels,
+                       const float* __restrict__ lse, const float* __restrict__ grad,
+                       const float* __restrict__ logprob, const int32_t* __restrict__ order,
+                       const SlabMeta* __restrict__ meta, int64_t hdim, uint16_t* __restrict__ hidden_s,
+                       int64_t* __restrict__ labels_s, int32_t* __restrict__ rows_s, float* __restrict__ lse_s,
+                       float* __restrict__ grad_s, float* __restrict__ logprob_s) {
+    const int64_t j = blockIdx.x;
+    if (j >= meta->count) return;
+    const int64_t src = order[meta->offset + j];
+    const oi_u32x4* from = reinterpret_cast<const oi_u32x4*>(hidden + src * hdim);
+    oi_u32x4* to = reinterpret_cast<oi_u32x4*>(hidden_s + j * hdim);
+    for (int64_t c = threadIdx.x; c < hdim / 8; c += blockDim.x) to[c] = from[c];
+    if (threadIdx.x == 0) {
+        labels_s[j] = labels[src];
+        rows_s[j] = (int32_t)src;
+        if (lse_s) lse_s[j] = lse[src];
+        if (grad_s) grad_s[j] = grad[src];
+        if (logprob_s) logprob_s[j] = logprob[src];
+    }
+}
+
+// Backward products straight from the kept exponentials e'[n, v] = 2^(x_nv - ref_n), x = z c:
+//   dZ[n, v] = g_n inv_T (1[v = y_n] - 2^(x_nv - lse2_n)) = s_n (e'[n, v] - 1[v = y_n] 2^(lse2_n - ref_n)),
+//   s_n = -g_n inv_T 2^(ref_n - lse2_n).
+// The per-token factor leaves the products: d_hidden[n] = s_n (e'[n, :] W) (a row factor in the
+// store epilogue) and d_weight = e'^T (s h) (the hidden rows are scaled once).  Workgroup j prepares
+// token j of a slab (caller row rows_s[j]): the two halves of s_n (so that neither leaves the fp32
+// range), the label's entry of the slab's exponentials, replaced by
+// 2^(x_y - ref) - 2^(lse2 - ref) = 2^(lse2 - ref) expm1(logprob) from the forward's fp32 logprob
+// (exact where the label's probability is close to 1), and, when d_weight is wanted, the scaled
+// hidden row.  A token flagged in `unsafe` gets factors of exactly 0: it adds nothing to either
+// product here and takes the recomputing backward afterwards.
+__global__ void __launch_bounds__(256)
+    slab_prepare_kernel(const float* __restrict__ lse, const float* __restrict__ grad,
+                        const float* __restrict__ logprob, const uint8_t* __restrict__ unsafe,
+                        const int32_t* __restrict__ rows_s, const int64_t* __restrict__ labels_s,
+                        const float* __restrict__ xref_s, const SlabMeta* __restrict__ meta, float inv_t,
+                        int64_t vocab, int64_t hdim, uint16_t* __restrict__ ecache, int64_t cache_ld,
+                        const uint16_t* __restrict__ hidden_s, float* __restrict__ scale_a,
+                        float* __restrict__ scale_b, uint16_t* __restrict__ scaled_hidden) {
+    const int64_t j = blockIdx.x;
+    if (j >= meta->count) return;
+    const int64_t src = rows_s[j];
+    const bool dead = unsafe[src] != 0;
+    const float l2 = lse[src] * OI_LOG2E - xref_s[j];  // log2 of the sum of the kept numbers of this token
+    const float half = dead ? 0.f : __builtin_amdgcn_exp2f(-0.5f * l2);
+    const float a = half, b = -grad[src] * inv_t * half;
+    if (threadIdx.x == 0) {
+        scale_a[j] = a;
+        scale_b[j] = b;
+        int64_t y = labels_s[j];
+        y = y < 0 ? 0 : (y >= vocab ? vocab - 1 : y);
+        ecache[j * cache_ld + y] =
+            (uint16_t)oi_f32_to_bf16_bits(__builtin_amdgcn_exp2f(fminf(l2, 126.f)) * expm1f(logprob[src]));
+    }
+    if (!scaled_hidden) return;
+    const oi_u32x4* from = reinterpret_cast<const oi_u32x4*>(hidden_s + j * hdim);
+    oi_u32x4* to = reinterpret_cast<oi_u32x4*>(scaled_hidden + j * hdim);
     for (int64_t c = threadIdx.x; c < hdim / 8; c += blockDim.x) {
         const oi_u32x4 v = from[c];
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
         uint32_t o[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k)
-            o[k] = oi_pack_bf16x2(oi_bf16lo_to_f32(w[k]) * a * b, oi_bf16hi_to_f32(w[k]) * a * b);
+            o[k] = dead ? 0u : oi_pack_bf16x2(oi_bf16lo_to_f32(w[k]) * a * b, oi_bf16hi_to_f32(w[k]) * a * b);
         to[c] = oi_u32x4{o[0], o[1], o[2], o[3]};
     }
 }
@@ -1079,6 +1179,28 @@ __global__ void __launch_bounds__(256)
     uint32_t* row = reinterpret_cast<uint32_t*>(out + i * hdim);  // hdim is a multiple of 64
     for (int64_t c = threadIdx.x; c < hdim / 2; c += blockDim.x) row[c] = 0u;
 }
+
+// Timing probe for the measurement harness: while armed, the slab-wise entry points record a pair
+// of HIP events around every launch of one of their three tile kernels (which one is chosen when the
+// probe is armed), on the stream of the call.  Off by default and between arm / read; not meant for
+// calls that are being captured into a graph.
+struct Probe {
+    int kernel = -1;  // 0 forward with kept exponentials, 1 d_hidden product, 2 d_weight product; -1 = off
+    int used = 0;
+    static constexpr int MAX_LAUNCHES = 256;
+    hipEvent_t ev[2 * MAX_LAUNCHES];
+};
+Probe g_probe;
+struct ProbeScope {
+    bool on;
+    hipStream_t s;
+    ProbeScope(int kernel, hipStream_t stream) : on(g_probe.kernel == kernel && g_probe.used < Probe::MAX_LAUNCHES), s(stream) {
+        if (on) (void)hipEventRecord(g_probe.ev[2 * g_probe.used], s);
+    }
+    ~ProbeScope() {
+        if (on) (void)hipEventRecord(g_probe.ev[2 * g_probe.used++ + 1], s);
+    }
+};
 
 // Workgroups of a queue-driven launch: one per CU of the current device (each takes a whole CU's
 // LDS), a multiple of 8 so that every XCD gets the same number, and no more than there are tiles.
@@ -1119,28 +1241,18 @@ SelectionPlan plan_selection(Carver& cv, int64_t n_pad, int64_t hdim, bool backw
     return p;
 }
 
-// The cache of exponentials: 2^(z c) in bf16 for the first `chunks` vocabulary chunks of the
-// backward pass, token-major [n_pad, ld].
-struct CachePlan {
-    int64_t chunks, ld, tiles;
-    size_t bytes;
+// Where the forward leaves the exponentials it computes anyway (all null / 0: nowhere)
+struct KeepPlan {
+    uint16_t* buf;        // bf16 [n_pad, ld], token-major
+    int64_t ld, tiles;    // columns of the buffer, and as vocabulary tiles
+    const float* xref;    // per token: the exponent the kept numbers are relative to
+    uint8_t* unsafe;      // per caller row: set when the kept numbers of that token cannot be used
 };
-CachePlan plan_cache(int64_t n_tokens, int64_t vocab, int64_t cache_chunks) {
-    const int64_t n_pad = (n_tokens + 255) / 256 * 256, v_pad = (vocab + 255) / 256 * 256;
-    const int64_t chunk = v_pad < BWD_VOCAB_CHUNK ? v_pad : BWD_VOCAB_CHUNK;
-    const int64_t n_chunks = (v_pad + chunk - 1) / chunk;
-    CachePlan c;
-    c.chunks = cache_chunks < 0 ? 0 : (cache_chunks > n_chunks ? n_chunks : cache_chunks);
-    c.ld = c.chunks * chunk < v_pad ? c.chunks * chunk : v_pad;
-    c.tiles = c.ld / BM;
-    c.bytes = (size_t)n_pad * c.ld * 2;
-    return c;
-}
 
 struct FwdPlan {
     int64_t token_tiles, vocab_tiles, n_splits, tiles_per_split, long_splits, n_pad;
     int64_t chunk, n_chunks;  // chunked flavour only
-    size_t off_partial, off_zy, off_queue, off_chunk, total;
+    size_t off_partial, off_zy, off_queue, off_chunk, off_xref, total;
     SelectionPlan sel;
 };
 // `chunked`: the launch covers one backward-sized vocabulary chunk at a time (the forward that also
@@ -1178,6 +1290,7 @@ FwdPlan plan_fwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_select
     p.off_queue = cv.take((chunked ? (size_t)p.n_chunks * (FWD_QUEUE_WORDS + QUEUE_WORDS) : (size_t)FWD_QUEUE_WORDS) *
                           sizeof(uint32_t));
     p.off_chunk = chunked ? cv.take((size_t)p.n_pad * p.chunk * 2) : 0;
+    p.off_xref = 0;
     if (with_selection) p.sel = plan_selection(cv, p.n_pad, hdim, false);
     p.total = cv.off;
     return p;
@@ -1185,31 +1298,21 @@ FwdPlan plan_fwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_select
 
 struct BwdPlan {
     int64_t n_pad, v_pad, chunk, n_chunks;
-    size_t off_dz, off_dh32, off_queues, off_scale_a, off_scale_b, off_scaled_hidden, total;
+    size_t off_dz, off_dh32, off_queues, total;
     SelectionPlan sel;
 };
-BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_selection, int64_t cache_chunks = 0) {
+BwdPlan plan_bwd(int64_t n_tokens, int64_t hdim, int64_t vocab, bool with_selection) {
     BwdPlan p;
     p.n_pad = round_up(n_tokens, 256);
     p.v_pad = round_up(vocab, 256);
     p.chunk = p.v_pad < BWD_VOCAB_CHUNK ? p.v_pad : BWD_VOCAB_CHUNK;
     p.n_chunks = (p.v_pad + p.chunk - 1) / p.chunk;
-    const bool with_cache = cache_chunks > 0;
-    // with every chunk in the cache nothing is recomputed and d_hidden is stored once: neither the
-    // dZ chunk nor the fp32 accumulator is needed
-    const bool all_cached = cache_chunks >= p.n_chunks;
     Carver cv;
-    p.off_dz = cv.take(all_cached ? 0 : (size_t)p.n_pad * p.chunk * 2);
-    p.off_dh32 = cv.take(all_cached ? 0 : (size_t)n_tokens * hdim * 4);
+    p.off_dz = cv.take((size_t)p.n_pad * p.chunk * 2);
+    p.off_dh32 = cv.take((size_t)n_tokens * hdim * 4);
     // one set of work-queue counters per tile-kernel launch (three per vocabulary chunk)
     p.off_queues = cv.take((size_t)(3 * p.n_chunks) * QUEUE_WORDS * sizeof(uint32_t));
     if (with_selection) p.sel = plan_selection(cv, p.n_pad, hdim, true);
-    p.off_scale_a = p.off_scale_b = p.off_scaled_hidden = 0;
-    if (with_cache) {
-        p.off_scale_a = cv.take((size_t)p.n_pad * sizeof(float));
-        p.off_scale_b = cv.take((size_t)p.n_pad * sizeof(float));
-        p.off_scaled_hidden = cv.take((size_t)p.n_pad * hdim * 2);
-    }
     p.total = cv.off;
     return p;
 }
@@ -1271,40 +1374,53 @@ __global__ void gather_f32_kernel(const float* __restrict__ lse, const float* __
     logprob_c[j] = logprob[src];
 }
 
+void launch_label_ref(const RowInputs& in, const void* weight, int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
+                      float inv_temperature, float* xref, hipStream_t s) {
+    hipLaunchKernelGGL(label_ref_kernel, dim3((unsigned)((n_tokens + 3) / 4)), dim3(256), 0, s, in.hidden,
+                       static_cast<const uint16_t*>(weight), in.labels, in.n_dev, n_tokens, hidden_dim, vocab,
+                       inv_temperature * OI_LOG2E, xref);
+}
+
 // forward launches: tile kernel + merge of the partial statistics.  `queue` must be zeroed.
+// `keep`: where the exponentials of every vocabulary tile go as well (buf null: nowhere).
 void enqueue_fwd(const FwdPlan& p, char* ws, const RowInputs& in, const uint8_t* row_mask, const void* weight,
                  int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob,
-                 float* entropy, float* lse, uint16_t* ecache, const CachePlan& cache, hipStream_t s) {
+                 float* entropy, float* lse, const KeepPlan& keep, hipStream_t s) {
     float4* partial = reinterpret_cast<float4*>(ws + p.off_partial);
     float* zy = reinterpret_cast<float*>(ws + p.off_zy);
     uint32_t* queue = reinterpret_cast<uint32_t*>(ws + p.off_queue);
     const float c = inv_temperature * OI_LOG2E;
     const dim3 grid(resident_grid(p.n_splits, p.token_tiles));
     const uint16_t* Wp = static_cast<const uint16_t*>(weight);
-    const FwdLaunch fl = {p.tiles_per_split, p.long_splits, 0,        p.long_splits, p.n_splits - p.long_splits,
-                          ecache,            cache.ld,      0,        cache.chunks > 0 ? cache.tiles : 0, 0};
-    if (cache.chunks > 0)
+    const FwdLaunch fl = {p.tiles_per_split, p.long_splits, 0, p.long_splits, p.n_splits - p.long_splits,
+                          keep.buf, keep.ld, 0, keep.buf ? keep.tiles : 0, 0, keep.xref};
+    if (keep.buf) {
+        const ProbeScope probe(0, s);
         hipLaunchKernelGGL(lmhead_fwd_kernel<true>, grid, dim3(NTHREADS), 0, s, Wp, in.hidden, in.labels, n_tokens,
                            in.n_dev, hidden_dim, vocab, c, fl, p.n_pad, partial, zy, queue);
-    else
+    } else
         hipLaunchKernelGGL(lmhead_fwd_kernel<false>, grid, dim3(NTHREADS), 0, s, Wp, in.hidden, in.labels, n_tokens,
                            in.n_dev, hidden_dim, vocab, c, fl, p.n_pad, partial, zy, queue);
     hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
-                       zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, logprob,
-                       entropy, lse);
+                       zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, c, logprob,
+                       entropy, lse, keep.buf ? keep.xref : static_cast<const float*>(nullptr),
+                       keep.buf ? keep.unsafe : static_cast<uint8_t*>(nullptr));
 }
 
-// The forward that also prepares d_hidden.  With x = z c in the log2 domain,
-//   d_hidden[n] = sum_v dZ[n, v] W[v] = s_n sum_{v != y} 2^(x_nv) W[v] - g_n inv_T expm1(logprob_n) W[y_n],
-//   s_n = -g_n inv_T 2^(-lse2_n),
+// The forward that also prepares d_hidden.  With x = z c in the log2 domain and a per-token
+// reference exponent ref_n (the scaled logit of the token's own label),
+//   d_hidden[n] = sum_v dZ[n, v] W[v]
+//               = s_n sum_{v != y} 2^(x_nv - ref_n) W[v] - g_n inv_T expm1(logprob_n) W[y_n],
+//   s_n = -g_n inv_T 2^(ref_n - lse2_n),
 // and the sum does not depend on the upstream gradient: it is accumulated while the logits exist,
-// one vocabulary chunk at a time (the exponentials of the chunk as bf16 in a chunk-sized buffer, as
-// for the cache of exponentials, with the label's own entry left out; then wsum (+)= E_chunk * W_chunk
-// in fp32).  A backward pass that only needs d_hidden is then one pass over [tokens, hidden]:
-// 4 N H V matrix work for forward + backward instead of 6 N H V, and nothing is recomputed.
+// one vocabulary chunk at a time (the exponentials of the chunk as bf16 in a chunk-sized buffer,
+// with the label's own entry left out; then wsum (+)= E_chunk * W_chunk in fp32).  A backward pass
+// that only needs d_hidden is then one pass over [tokens, hidden]: 4 N H V matrix work for forward +
+// backward instead of 6 N H V, and nothing is recomputed.  Tokens whose largest logit is too far
+// above their label's are flagged in `unsafe`; their sums are not used (the backward recomputes them).
 void enqueue_fwd_wsum(const FwdPlan& p, char* ws, const RowInputs& in, const uint8_t* row_mask, const void* weight,
                       int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature, float* logprob,
-                      float* entropy, float* lse, float* wsum, hipStream_t s) {
+                      float* entropy, float* lse, float* wsum, float* xref, uint8_t* unsafe, hipStream_t s) {
     float4* partial = reinterpret_cast<float4*>(ws + p.off_partial);
     float* zy = reinterpret_cast<float*>(ws + p.off_zy);
     uint32_t* queues = reinterpret_cast<uint32_t*>(ws + p.off_queue);
@@ -1314,6 +1430,7 @@ void enqueue_fwd_wsum(const FwdPlan& p, char* ws, const RowInputs& in, const uin
     const int64_t h_tiles = (hidden_dim + BN - 1) / BN;
     const int64_t v_pad = p.vocab_tiles * BM;
     const int64_t splits_per_chunk = (p.chunk / BM + p.tiles_per_split - 1) / p.tiles_per_split;
+    launch_label_ref(in, weight, n_tokens, hidden_dim, vocab, inv_temperature, xref, s);
     for (int64_t ci = 0; ci < p.n_chunks; ++ci) {
         const int64_t v_begin = ci * p.chunk;
         const int64_t v_end = v_begin + p.chunk < v_pad ? v_begin + p.chunk : v_pad;
@@ -1322,7 +1439,8 @@ void enqueue_fwd_wsum(const FwdPlan& p, char* ws, const RowInputs& in, const uin
         const int64_t first = ci * splits_per_chunk;
         const int64_t n_first = p.n_splits - first < splits_per_chunk ? p.n_splits - first : splits_per_chunk;
         uint32_t* q = queues + ci * (FWD_QUEUE_WORDS + QUEUE_WORDS);
-        const FwdLaunch fl = {p.tiles_per_split, p.long_splits, first, n_first, 0, chunk_buf, cols, v_begin / BM, cols / BM, 1};
+        const FwdLaunch fl = {p.tiles_per_split, p.long_splits, first, n_first, 0, chunk_buf, cols, v_begin / BM,
+                              cols / BM, 1, xref};
         hipLaunchKernelGGL(lmhead_fwd_kernel<true>, dim3(resident_grid(n_first, p.token_tiles)), dim3(NTHREADS), 0, s, Wp,
                            in.hidden, in.labels, n_tokens, in.n_dev, hidden_dim, vocab, c, fl, p.n_pad, partial, zy, q);
         const Operand a = {chunk_buf, cols, 0, p.n_pad, cols};
@@ -1333,15 +1451,17 @@ void enqueue_fwd_wsum(const FwdPlan& p, char* ws, const RowInputs& in, const uin
                            static_cast<uint16_t*>(nullptr), hidden_dim, n_tokens, dyn, q + FWD_QUEUE_WORDS);
     }
     hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
-                       zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, logprob,
-                       entropy, lse);
+                       zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, c, logprob,
+                       entropy, lse, static_cast<const float*>(xref), unsafe);
 }
 
 // d_hidden row of selected token j (caller row rows[j], or j without a selection) from the weighted
 // sum that the forward left behind; one workgroup per selected row.  The factor s is applied in two
-// halves so that neither leaves the fp32 range.
+// halves so that neither leaves the fp32 range.  Rows flagged in `unsafe` are left alone (the
+// recomputing backward writes them).
 __global__ void __launch_bounds__(256)
-    dh_from_wsum_kernel(const float* __restrict__ wsum, const uint16_t* __restrict__ W,
+    dh_from_wsum_kernel(const float* __restrict__ wsum, const float* __restrict__ xref,
+                        const uint8_t* __restrict__ unsafe, const uint16_t* __restrict__ W,
                         const int64_t* __restrict__ labels, const float* __restrict__ lse,
                         const float* __restrict__ logprob, const float* __restrict__ grad,
                         const int32_t* __restrict__ rows, const int32_t* __restrict__ count, int64_t n_tokens,
@@ -1349,8 +1469,9 @@ __global__ void __launch_bounds__(256)
     const int64_t j = blockIdx.x;
     if (j >= (count ? (int64_t)*count : n_tokens)) return;
     const int64_t n = rows ? (int64_t)rows[j] : j;
+    if (unsafe[n]) return;
     const float g = grad[n] * inv_t;
-    const float half = __builtin_amdgcn_exp2f(-0.5f * lse[n] * OI_LOG2E);
+    const float half = __builtin_amdgcn_exp2f(0.5f * (xref[j] - lse[n] * OI_LOG2E));
     const float sb = -g * half;
     const float tl = -g * expm1f(logprob[n]);
     int64_t y = labels[n];
@@ -1367,69 +1488,49 @@ __global__ void __launch_bounds__(256)
     }
 }
 
-// backward launches.  Per vocabulary chunk: dZ [n_pad, cols] (token-major, bf16, zero in padded rows
-// and columns), then both products straight from W and the (selected) hidden rows, which enter as
-// k-major operands:
+// The recomputing backward.  Per vocabulary chunk: dZ [n_pad, cols] (token-major, bf16, zero in padded
+// rows and columns), then both products straight from W and the (selected) hidden rows, which enter
+// as k-major operands:
 //   d_hidden[n, h] (+)= sum_v dZ[n, v] * W[v_begin + v, h]      A k-contiguous, B k-major
 //   d_weight[v_begin + v, h] = sum_n dZ[n, v] * hidden[n, h]    A k-major,      B k-major
 // The sums stop at the last real vocabulary row / token (rounded up to a k-tile, whose missing
-// rows are read from the last real one and meet zeros of dZ).  Chunks that the forward left in the
-// cache of exponentials skip the recomputation: the cache itself is the A operand of both products
-// (see cache_rows_prepare_kernel).  The queue words must be zeroed.
+// rows are read from the last real one and meet zeros of dZ).  The queue words must be zeroed.
 // dw_mode / dw32: how d_weight is stored.  2 (default): this call holds every token, bf16 rows are
 // written directly.  0 / 1: the tokens come in several calls; dw32 (fp32 [vocab, hidden]) takes the
 // first call's product (0) and adds the following ones (1; a call without tokens adds nothing and
-// costs nothing); the caller rounds dw32 to bf16 when the last call is through.
+// costs nothing); the caller rounds dw32 to bf16 when the last call is through.  4: the product is
+// added to bf16 rows that an earlier call wrote.
 void enqueue_bwd(const BwdPlan& p, char* ws, const RowInputs& in, const void* weight, int64_t n_tokens,
                  int64_t hidden_dim, int64_t vocab, float inv_temperature, void* d_hidden, void* d_weight,
-                 uint16_t* ecache, const CachePlan& cache, hipStream_t s, int dw_mode = 2, float* dw32 = nullptr) {
+                 hipStream_t s, int dw_mode = 2, float* dw32 = nullptr) {
     uint16_t* dz = reinterpret_cast<uint16_t*>(ws + p.off_dz);
     float* dh32 = reinterpret_cast<float*>(ws + p.off_dh32);
     uint32_t* queues = reinterpret_cast<uint32_t*>(ws + p.off_queues);
     const uint16_t* Wp = static_cast<const uint16_t*>(weight);
     const float c = inv_temperature * OI_LOG2E;
     const int64_t h_tiles = (hidden_dim + BN - 1) / BN;
-    float* scale_a = reinterpret_cast<float*>(ws + p.off_scale_a);
-    float* scale_b = reinterpret_cast<float*>(ws + p.off_scale_b);
-    uint16_t* scaled_hidden = reinterpret_cast<uint16_t*>(ws + p.off_scaled_hidden);
-    if (cache.chunks > 0) {
-        hipLaunchKernelGGL(cache_rows_prepare_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, in.lse,
-                           in.grad, in.logprob, in.labels, in.n_dev, n_tokens, inv_temperature, vocab, ecache, cache.ld,
-                           scale_a, scale_b);
-        if (d_weight)
-            hipLaunchKernelGGL(scale_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, in.hidden, scale_a, scale_b,
-                               in.n_dev, n_tokens, hidden_dim, scaled_hidden);
-    }
-    // The cached chunks need no dZ buffer between the recomputation and the products, so they are
-    // multiplied as ONE chunk (fewer, longer tiles; d_hidden is stored once instead of accumulated).
-    for (int64_t ci = cache.chunks > 0 ? cache.chunks - 1 : 0; ci < p.n_chunks; ++ci) {
-        const bool merged = cache.chunks > 0 && ci == cache.chunks - 1;
-        const int64_t v_begin = merged ? 0 : ci * p.chunk;
+    for (int64_t ci = 0; ci < p.n_chunks; ++ci) {
+        const int64_t v_begin = ci * p.chunk;
         const int64_t v_end = (ci + 1) * p.chunk < p.v_pad ? (ci + 1) * p.chunk : p.v_pad;
-        const int64_t cols = v_end - v_begin;                                                // multiple of 256
-        const int64_t valid = vocab - v_begin < cols ? vocab - v_begin : cols;               // real rows of W
-        const bool cached = ci < cache.chunks;
+        const int64_t cols = v_end - v_begin;                                   // multiple of 256
+        const int64_t valid = vocab - v_begin < cols ? vocab - v_begin : cols;  // real rows of W
         uint32_t* q = queues + ci * 3 * QUEUE_WORDS;
-        if (!cached)
-            hipLaunchKernelGGL(lmhead_dz_kernel, dim3(resident_grid(cols / BM, p.n_pad / BN)), dim3(NTHREADS), 0, s, Wp,
-                               in.hidden, in.labels, in.lse, in.grad, in.logprob, n_tokens, in.n_dev, hidden_dim, vocab, c,
-                               inv_temperature, v_begin, cols, p.n_pad, dz, q);
-        // the A operand of both products: this chunk's dZ, or this chunk's columns of the cache
-        const uint16_t* a_ptr = cached ? ecache + v_begin : dz;
-        const int64_t a_ld = cached ? cache.ld : cols;
-        const bool first = v_begin == 0, last = ci == p.n_chunks - 1;
+        hipLaunchKernelGGL(lmhead_dz_kernel, dim3(resident_grid(cols / BM, p.n_pad / BN)), dim3(NTHREADS), 0, s, Wp,
+                           in.hidden, in.labels, in.lse, in.grad, in.logprob, n_tokens, in.n_dev, hidden_dim, vocab, c,
+                           inv_temperature, v_begin, cols, p.n_pad, dz, q);
+        const bool first = ci == 0, last = ci == p.n_chunks - 1;
         const int mode = last ? (first ? 2 : 3) : (first ? 0 : 1);
         {
-            const Operand a = {a_ptr, a_ld, 0, p.n_pad, cols};
+            const Operand a = {dz, cols, 0, p.n_pad, cols};
             const Operand b = {Wp + v_begin * hidden_dim, hidden_dim, 0, hidden_dim, valid};
-            const DynRows dyn = {in.n_dev, 1, in.rows, cached ? scale_a : nullptr, cached ? scale_b : nullptr};
+            const DynRows dyn = {in.n_dev, 1, in.rows, nullptr, nullptr};
             hipLaunchKernelGGL((gemm_store_kernel<false, true>), dim3(resident_grid(p.n_pad / BM, h_tiles)),
                                dim3(NTHREADS), 0, s, a, p.n_pad, b, hidden_dim, round_up(valid, BK), mode, dh32,
                                static_cast<uint16_t*>(d_hidden), hidden_dim, n_tokens, dyn, q + QUEUE_WORDS);
         }
         if (d_weight) {
-            const Operand a = {a_ptr, a_ld, 0, cols, p.n_pad};
-            const Operand b = {cached ? scaled_hidden : in.hidden, hidden_dim, 0, hidden_dim, n_tokens};
+            const Operand a = {dz, cols, 0, cols, p.n_pad};
+            const Operand b = {in.hidden, hidden_dim, 0, hidden_dim, n_tokens};
             const DynRows dyn = {in.n_dev, 2, nullptr, nullptr, nullptr};
             hipLaunchKernelGGL((gemm_store_kernel<true, true>), dim3(resident_grid(cols / BM, h_tiles)),
                                dim3(NTHREADS), 0, s, a, cols, b, hidden_dim, round_up(n_tokens, BK), dw_mode,
@@ -1440,6 +1541,37 @@ void enqueue_bwd(const BwdPlan& p, char* ws, const RowInputs& in, const void* we
     }
 }
 
+// Both backward products of a slab from its kept exponentials (see slab_prepare_kernel): the whole
+// vocabulary as one chunk, d_hidden rows stored once through the slab's row numbers, d_weight
+// stored / accumulated as dw_mode says (see enqueue_bwd).  `queues`: 2 * QUEUE_WORDS zeroed words.
+void enqueue_products_from_exponentials(const uint16_t* ecache, int64_t cache_ld, int64_t slab_pad,
+                                        const int32_t* count, const int32_t* rows_s, const float* scale_a,
+                                        const float* scale_b, const uint16_t* scaled_hidden, const void* weight,
+                                        int64_t hidden_dim, int64_t vocab, void* d_hidden, void* d_weight,
+                                        int dw_mode, float* dw32, uint32_t* queues, hipStream_t s) {
+    const uint16_t* Wp = static_cast<const uint16_t*>(weight);
+    const int64_t h_tiles = (hidden_dim + BN - 1) / BN;
+    {
+        const ProbeScope probe(1, s);
+        const Operand a = {ecache, cache_ld, 0, slab_pad, cache_ld};
+        const Operand b = {Wp, hidden_dim, 0, hidden_dim, vocab};
+        const DynRows dyn = {count, 1, rows_s, scale_a, scale_b};
+        hipLaunchKernelGGL((gemm_store_kernel<false, true>), dim3(resident_grid(slab_pad / BM, h_tiles)),
+                           dim3(NTHREADS), 0, s, a, slab_pad, b, hidden_dim, round_up(vocab, BK), 2,
+                           static_cast<float*>(nullptr), static_cast<uint16_t*>(d_hidden), hidden_dim, slab_pad, dyn,
+                           queues);
+    }
+    if (d_weight) {
+        const ProbeScope probe(2, s);
+        const Operand a = {ecache, cache_ld, 0, cache_ld, slab_pad};
+        const Operand b = {scaled_hidden, hidden_dim, 0, hidden_dim, slab_pad};
+        const DynRows dyn = {count, 2, nullptr, nullptr, nullptr};
+        hipLaunchKernelGGL((gemm_store_kernel<true, true>), dim3(resident_grid(cache_ld / BM, h_tiles)),
+                           dim3(NTHREADS), 0, s, a, cache_ld, b, hidden_dim, round_up(slab_pad, BK), dw_mode, dw32,
+                           static_cast<uint16_t*>(d_weight), hidden_dim, vocab, dyn, queues + QUEUE_WORDS);
+    }
+}
+
 // workspace of the whole-step entry point: forward and backward regions side by side (they share
 // one row selection), the statistics partials, and the per-token vectors that connect the stages
 struct StepPlan {
@@ -1447,11 +1579,11 @@ struct StepPlan {
     BwdPlan bwd;
     size_t off_fwd, off_bwd, off_stats, off_lse, off_grad, off_denoms, total;
 };
-StepPlan plan_step(int64_t rows, int64_t cols, int64_t hdim, int64_t vocab, int64_t cache_chunks) {
+StepPlan plan_step(int64_t rows, int64_t cols, int64_t hdim, int64_t vocab) {
     StepPlan p;
     const int64_t n = rows * cols;
     p.fwd = plan_fwd(n, hdim, vocab, false);
-    p.bwd = plan_bwd(n, hdim, vocab, true, cache_chunks);
+    p.bwd = plan_bwd(n, hdim, vocab, true);
     Carver cv;
     p.off_fwd = cv.take(p.fwd.total);
     p.off_bwd = cv.take(p.bwd.total);
@@ -1463,49 +1595,80 @@ StepPlan plan_step(int64_t rows, int64_t cols, int64_t hdim, int64_t vocab, int6
     return p;
 }
 
-// The whole step in slabs of tokens, with nothing recomputed: the selected rows are taken
-// slab_units * SLAB_UNIT at a time; a slab's forward leaves its exponentials (every vocabulary chunk, bf16) in
-// a slab-sized buffer, the slab's tokens get their upstream gradient at once (it depends only on
-// the token's own logprob and on denominators that come from the mask), and both products read the
-// buffer before the next slab overwrites it: d_hidden rows are final, d_weight accumulates in fp32
-// over the slabs.  6 N H V of matrix work instead of 8 N H V; the buffer holds
-// [slab, vocabulary], never [tokens, vocabulary].  Every slab costs a pass over the fp32 d_weight and
-// leaves the ends of its launches ragged (measured at the Llama-3.1-8B shape, 22942 selected rows:
-// 72.7 ms per step with slabs of 4096 rows, 63.2 with 8192, 59.5 with 16384; 77.3 recomputing).
-constexpr int64_t SLAB_UNIT = 4096;  // a slab is a multiple of this many rows (256 d_hidden tiles at H = 4096)
+// ---------------------------------------------------------------------------------------------
+// The whole step in slabs of tokens, with nothing recomputed
+// ---------------------------------------------------------------------------------------------
+// The selected rows are taken a slab at a time (at most `cap` rows; the slabs of a call are made
+// equal on the device, where the selected count lives).  A slab's forward leaves its exponentials
+// (every vocabulary column, bf16, relative to each token's own reference exponent) in a slab-sized
+// buffer, the slab's tokens get their upstream gradient at once (the caller of run_slab_passes says
+// how: for the GRPO loss it depends only on the token's own logprob and on denominators that come
+// from the mask), and both products read the buffer before the next slab overwrites it: d_hidden
+// rows are final, d_weight accumulates in fp32 over the slabs.  6 N H V of matrix work instead of
+// 8 N H V; the buffer holds [slab, vocabulary], never [tokens, vocabulary].  Tokens that the
+// forward flags (largest logit too far above the label's) add nothing in their slab and are served
+// by one recomputing backward over the flagged rows after the last slab, so the results do not
+// depend on the size of the logits.  Every slab costs a pass over the fp32 d_weight and leaves the
+// ends of its launches ragged.
+constexpr int64_t SLAB_UNIT = 256;  // a slab capacity is a multiple of this many rows (a token tile)
+constexpr int SLAB_QUEUE_WORDS = FWD_QUEUE_WORDS + 2 * QUEUE_WORDS;
 struct SlabPlan {
-    int64_t slab, n_slabs, n_pad;
-    FwdPlan fwd;
-    BwdPlan bwd;
-    CachePlan cache;
-    SelectionPlan sel;
-    size_t off_fwd, off_bwd, off_sel, off_counts, off_cache, off_dw32, off_stats, off_lse, off_grad, off_denoms, total;
+    int64_t cap, n_passes, n_pad, v_pad;
+    FwdPlan fwd;     // of one slab
+    BwdPlan repair;  // the recomputing backward over all rows (for the flagged ones)
+    size_t off_fwd, off_order, off_count, off_meta, off_unsafe, off_keep, off_repair, off_hidden_s, off_labels_s,
+        off_rows_s, off_xref_s, off_scale_a, off_scale_b, off_scaled_hidden, off_queues, off_dw32, off_stats, off_lse,
+        off_grad, off_denoms, total;
 };
-SlabPlan plan_slabs(int64_t rows, int64_t cols, int64_t hdim, int64_t vocab, bool want_dw, int64_t slab_units) {
+SlabPlan plan_slabs(int64_t n, int64_t stats_rows, int64_t stats_cols, int64_t hdim, int64_t vocab, bool want_dw,
+                    int64_t slab_tokens, int64_t n_passes_override = 0) {
     SlabPlan p;
-    const int64_t n = rows * cols;
     p.n_pad = round_up(n, 256);
-    const int64_t slab_tokens = (slab_units < 1 ? 1 : (slab_units > 256 ? 256 : slab_units)) * SLAB_UNIT;
-    p.slab = p.n_pad < slab_tokens ? p.n_pad : slab_tokens;
-    p.n_slabs = (p.n_pad + p.slab - 1) / p.slab;
-    const int64_t all_chunks = (round_up(vocab, 256) + BWD_VOCAB_CHUNK - 1) / BWD_VOCAB_CHUNK;
-    p.fwd = plan_fwd(p.slab, hdim, vocab, false);
-    p.bwd = plan_bwd(p.slab, hdim, vocab, false, all_chunks);
-    p.cache = plan_cache(p.slab, vocab, all_chunks);
+    p.v_pad = round_up(vocab, 256);
+    const int64_t cap = round_up(slab_tokens < SLAB_UNIT ? SLAB_UNIT : slab_tokens, SLAB_UNIT);
+    p.cap = p.n_pad < cap ? p.n_pad : cap;
+    p.n_passes = n_passes_override > 0 ? n_passes_override : (p.n_pad + p.cap - 1) / p.cap;
+    p.fwd = plan_fwd(p.cap, hdim, vocab, false);
+    p.repair = plan_bwd(n, hdim, vocab, true);
     Carver cv;
     p.off_fwd = cv.take(p.fwd.total);
-    p.off_bwd = cv.take(p.bwd.total);
-    p.off_sel = cv.off;
-    p.sel = plan_selection(cv, p.n_slabs * p.slab, hdim, true);
-    p.off_counts = cv.take((size_t)p.n_slabs * sizeof(int32_t));
-    p.off_cache = cv.take(p.cache.bytes);
-    p.off_dw32 = cv.take(want_dw && p.n_slabs > 1 ? (size_t)vocab * hdim * sizeof(float) : 0);
-    p.off_stats = cv.take(oi_grpo_fused_workspace_bytes(rows, cols));
+    p.off_order = cv.take((size_t)p.n_pad * sizeof(int32_t));
+    p.off_count = cv.take(sizeof(int32_t));
+    p.off_meta = cv.take((size_t)p.n_passes * sizeof(SlabMeta));
+    p.off_unsafe = cv.take((size_t)p.n_pad);
+    // the slab's exponentials and, after the last slab, the workspace of the repair share one region
+    const size_t keep_bytes = (size_t)p.cap * p.v_pad * 2;
+    p.off_keep = p.off_repair = cv.take(keep_bytes > p.repair.total ? keep_bytes : p.repair.total);
+    p.off_hidden_s = cv.take((size_t)p.cap * hdim * 2);
+    p.off_labels_s = cv.take((size_t)p.cap * sizeof(int64_t));
+    p.off_rows_s = cv.take((size_t)p.cap * sizeof(int32_t));
+    p.off_xref_s = cv.take((size_t)p.cap * sizeof(float));
+    p.off_scale_a = cv.take((size_t)p.cap * sizeof(float));
+    p.off_scale_b = cv.take((size_t)p.cap * sizeof(float));
+    p.off_scaled_hidden = cv.take(want_dw ? (size_t)p.cap * hdim * 2 : 0);
+    p.off_queues = cv.take((size_t)SLAB_QUEUE_WORDS * sizeof(uint32_t));
+    p.off_dw32 = cv.take(want_dw && p.n_passes > 1 ? (size_t)vocab * hdim * sizeof(float) : 0);
+    p.off_stats = cv.take(oi_grpo_fused_workspace_bytes(stats_rows, stats_cols));
     p.off_lse = cv.take((size_t)n * sizeof(float));
     p.off_grad = cv.take((size_t)n * sizeof(float));
-    p.off_denoms = cv.take((size_t)rows * sizeof(float));
+    p.off_denoms = cv.take((size_t)stats_rows * sizeof(float));
     p.total = cv.off;
     return p;
+}
+
+// Equal slabs: the selected rows split into the fewest slabs of at most `cap` rows, all of the same
+// size (a multiple of 256 rows, the last one takes what is left); passes past the last slab are empty.
+__global__ void plan_equal_slabs_kernel(const int32_t* __restrict__ count, int cap, int n_passes,
+                                        SlabMeta* __restrict__ meta) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_passes) return;
+    const int n = *count;
+    const int k = n > 0 ? (n + cap - 1) / cap : 1;
+    int size = ((n + k - 1) / k + 255) / 256 * 256;
+    size = size > cap ? cap : size;
+    const int left = n - i * size;
+    meta[i].offset = i * size;
+    meta[i].count = left < 0 ? 0 : (left > size ? size : left);
 }
 
 // out[8 i .. 8 i + 8) = bf16(in[8 i .. 8 i + 8))
@@ -1515,14 +1678,6 @@ __global__ void __launch_bounds__(256) f32_to_bf16_kernel(const float* __restric
     const float4 a = reinterpret_cast<const float4*>(in)[2 * i], b = reinterpret_cast<const float4*>(in)[2 * i + 1];
     reinterpret_cast<oi_u32x4*>(out)[i] =
         oi_u32x4{oi_pack_bf16x2(a.x, a.y), oi_pack_bf16x2(a.z, a.w), oi_pack_bf16x2(b.x, b.y), oi_pack_bf16x2(b.z, b.w)};
-}
-
-// counts[i] = number of selected rows that fall into slab i
-__global__ void slab_counts_kernel(const int32_t* __restrict__ count, int slab, int n_slabs, int32_t* __restrict__ counts) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n_slabs) return;
-    const int left = *count - i * slab;
-    counts[i] = left < 0 ? 0 : (left > slab ? slab : left);
 }
 
 // the per-token outputs of rows that take no part are zero
@@ -1535,19 +1690,101 @@ __global__ void zero_unselected_f32_kernel(const uint8_t* __restrict__ mask, int
     if (c) c[i] = 0.f;
 }
 
-int check_cache(const void* exp_cache, int64_t cache_chunks) {
-    OI_RETURN_IF(cache_chunks < 0, OI_EINVAL);
-    OI_RETURN_IF(cache_chunks > 0 && !exp_cache, OI_ENULL);
-    OI_RETURN_IF(!oi_aligned(exp_cache, 16), OI_EALIGN);
-    return OI_OK;
+// What a slab-wise step is made of besides the passes themselves
+struct SlabStep {
+    const void *hidden, *weight;
+    const int64_t* labels;       // per caller row, as the kernels score them
+    const uint8_t* mask;         // per caller row: the rows that are multiplied
+    int64_t n_tokens, hidden_dim, vocab;
+    float inv_temperature;
+    float *logprob, *entropy;    // per caller row (entropy may be null)
+    void *d_hidden, *d_weight;   // d_weight may be null
+};
+
+// Runs the slab passes of `st` over the row index order[0 .. *count) that `plan_rows` leaves in the
+// workspace together with the passes' SlabMeta.  `upstream(final)` must enqueue kernels that leave
+// every caller row's d loss / d logprob in the workspace's grad vector, given the logprobs computed
+// so far (the rows of the slabs up to the current one; with `final` set, all rows).
+template <class PlanRows, class Upstream>
+int run_slab_passes(const SlabPlan& p, char* ws, const SlabStep& st, hipStream_t s, PlanRows&& plan_rows,
+                    Upstream&& upstream) {
+    const int64_t n = st.n_tokens, hdim = st.hidden_dim, vocab = st.vocab;
+    char* ws_fwd = ws + p.off_fwd;
+    int32_t* order = reinterpret_cast<int32_t*>(ws + p.off_order);
+    int32_t* count = reinterpret_cast<int32_t*>(ws + p.off_count);
+    SlabMeta* meta = reinterpret_cast<SlabMeta*>(ws + p.off_meta);
+    uint8_t* unsafe = reinterpret_cast<uint8_t*>(ws + p.off_unsafe);
+    uint16_t* keep_buf = reinterpret_cast<uint16_t*>(ws + p.off_keep);
+    uint16_t* hidden_s = reinterpret_cast<uint16_t*>(ws + p.off_hidden_s);
+    int64_t* labels_s = reinterpret_cast<int64_t*>(ws + p.off_labels_s);
+    int32_t* rows_s = reinterpret_cast<int32_t*>(ws + p.off_rows_s);
+    float* xref_s = reinterpret_cast<float*>(ws + p.off_xref_s);
+    float* scale_a = reinterpret_cast<float*>(ws + p.off_scale_a);
+    float* scale_b = reinterpret_cast<float*>(ws + p.off_scale_b);
+    uint16_t* scaled_hidden = st.d_weight ? reinterpret_cast<uint16_t*>(ws + p.off_scaled_hidden) : nullptr;
+    uint32_t* queues = reinterpret_cast<uint32_t*>(ws + p.off_queues);
+    float* dw32 = st.d_weight && p.n_passes > 1 ? reinterpret_cast<float*>(ws + p.off_dw32) : nullptr;
+    float* lse = reinterpret_cast<float*>(ws + p.off_lse);
+    float* grad = reinterpret_cast<float*>(ws + p.off_grad);
+    const uint16_t* hid = static_cast<const uint16_t*>(st.hidden);
+
+    hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((p.n_pad / 4 + 255) / 256)), dim3(256), 0, s,
+                       reinterpret_cast<uint32_t*>(unsafe), (int)(p.n_pad / 4));
+    plan_rows(order, count, meta);
+    hipLaunchKernelGGL(zero_unselected_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, st.mask, n,
+                       st.logprob, st.entropy, lse);
+    hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n), dim3(256), 0, s, st.mask,
+                       static_cast<const float*>(nullptr), hdim, static_cast<uint16_t*>(st.d_hidden));
+    for (int64_t i = 0; i < p.n_passes; ++i) {
+        const int32_t* cnt = &meta[i].count;
+        hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, queues, SLAB_QUEUE_WORDS);
+        hipLaunchKernelGGL(gather_slab_kernel, dim3((unsigned)p.cap), dim3(256), 0, s, hid, st.labels,
+                           static_cast<const float*>(nullptr), static_cast<const float*>(nullptr),
+                           static_cast<const float*>(nullptr), order, meta + i, hdim, hidden_s, labels_s, rows_s,
+                           static_cast<float*>(nullptr), static_cast<float*>(nullptr), static_cast<float*>(nullptr));
+        const RowInputs in = {hidden_s, labels_s, nullptr, nullptr, rows_s, cnt, nullptr};
+        launch_label_ref(in, st.weight, p.cap, hdim, vocab, st.inv_temperature, xref_s, s);
+        const KeepPlan keep = {keep_buf, p.v_pad, p.v_pad / BM, xref_s, unsafe};
+        // the forward's own queue words are the first FWD_QUEUE_WORDS of `queues`
+        FwdPlan fp = p.fwd;
+        fp.off_queue = (size_t)(reinterpret_cast<char*>(queues) - ws_fwd);
+        enqueue_fwd(fp, ws_fwd, in, nullptr, st.weight, p.cap, hdim, vocab, st.inv_temperature, st.logprob, st.entropy,
+                    lse, keep, s);
+        const int rc = upstream(false);
+        if (rc != OI_OK) return rc;
+        hipLaunchKernelGGL(slab_prepare_kernel, dim3((unsigned)p.cap), dim3(256), 0, s, lse, grad, st.logprob, unsafe,
+                           rows_s, labels_s, xref_s, meta + i, st.inv_temperature, vocab, hdim, keep_buf, p.v_pad,
+                           hidden_s, scale_a, scale_b, scaled_hidden);
+        const int dw_mode = p.n_passes == 1 ? 2 : (i == 0 ? 0 : 1);
+        enqueue_products_from_exponentials(keep_buf, p.v_pad, p.cap, cnt, rows_s, scale_a, scale_b, scaled_hidden,
+                                           st.weight, hdim, vocab, st.d_hidden, st.d_weight, dw_mode, dw32,
+                                           queues + FWD_QUEUE_WORDS, s);
+    }
+    // the flagged rows, if any: one recomputing backward over them (its workspace takes the place of
+    // the exponentials), added to what the slabs left in d_weight
+    {
+        const int rc = upstream(true);
+        if (rc != OI_OK) return rc;
+        char* ws_rep = ws + p.off_repair;
+        uint32_t* rq = reinterpret_cast<uint32_t*>(ws_rep + p.repair.off_queues);
+        const int n_words = (int)(3 * p.repair.n_chunks * QUEUE_WORDS);
+        const bool select_clears = n_words <= SELECT_THREADS;
+        if (!select_clears)
+            hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_words + 255) / 256)), dim3(256), 0, s, rq, n_words);
+        const RowInputs in = launch_selection(p.repair.sel, ws_rep, st.hidden, st.labels, lse, grad, unsafe, false, n,
+                                              hdim, rq, select_clears ? n_words : 0, s, st.logprob);
+        enqueue_bwd(p.repair, ws_rep, in, st.weight, n, hdim, vocab, st.inv_temperature, st.d_hidden, st.d_weight, s,
+                    dw32 ? 1 : 4, dw32);
+    }
+    if (dw32) {
+        const int64_t n8 = vocab * hdim / 8;  // hidden_dim is a multiple of 64
+        hipLaunchKernelGGL(f32_to_bf16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, s, dw32, n8,
+                           static_cast<uint16_t*>(st.d_weight));
+    }
+    return oi_launch_status();
 }
 
 }  // namespace
-
-extern "C" size_t oi_lmhead_cache_bytes(int64_t n_tokens, int64_t vocab, int64_t cache_chunks) {
-    if (n_tokens <= 0 || vocab <= 0 || cache_chunks <= 0) return 0;
-    return plan_cache(n_tokens, vocab, cache_chunks).bytes;
-}
 
 extern "C" size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
                                                 int with_row_mask) {
@@ -1557,18 +1794,15 @@ extern "C" size_t oi_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden
 
 extern "C" int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const int64_t* labels,
                                   const uint8_t* row_mask, int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
-                                  float inv_temperature, float* logprob, float* entropy, float* lse, void* exp_cache,
-                                  int64_t cache_chunks, void* workspace, size_t workspace_bytes, void* stream) {
+                                  float inv_temperature, float* logprob, float* entropy, float* lse, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
     int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
-    if (rc != OI_OK) return rc;
-    rc = check_cache(exp_cache, cache_chunks);
     if (rc != OI_OK) return rc;
     if (n_tokens == 0) return OI_OK;
     OI_RETURN_IF(!logprob || !workspace, OI_ENULL);
     OI_RETURN_IF(!oi_aligned(workspace, 256), OI_EALIGN);
     const FwdPlan p = plan_fwd(n_tokens, hidden_dim, vocab, row_mask != nullptr);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
-    const CachePlan cache = plan_cache(n_tokens, vocab, cache_chunks);
     char* ws = static_cast<char*>(workspace);
     uint32_t* queue = reinterpret_cast<uint32_t*>(ws + p.off_queue);
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -1579,7 +1813,7 @@ extern "C" int oi_lmhead_logp_fwd(const void* hidden, const void* weight, const 
     else
         hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, queue, FWD_QUEUE_WORDS);
     enqueue_fwd(p, ws, in, row_mask, weight, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy, lse,
-                static_cast<uint16_t*>(exp_cache), cache, s);
+                KeepPlan{nullptr, 0, 0, nullptr, nullptr}, s);
     return oi_launch_status();
 }
 
@@ -1592,12 +1826,13 @@ extern "C" size_t oi_lmhead_fwd_wsum_workspace_bytes(int64_t n_tokens, int64_t h
 extern "C" int oi_lmhead_logp_fwd_wsum(const void* hidden, const void* weight, const int64_t* labels,
                                        const uint8_t* row_mask, int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
                                        float inv_temperature, float* logprob, float* entropy, float* lse, float* wsum,
-                                       void* workspace, size_t workspace_bytes, void* stream) {
+                                       float* xref, uint8_t* unsafe, void* workspace, size_t workspace_bytes,
+                                       void* stream) {
     int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
     if (rc != OI_OK) return rc;
     if (n_tokens == 0) return OI_OK;
-    OI_RETURN_IF(!logprob || !lse || !wsum || !workspace, OI_ENULL);
-    OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(wsum, 16), OI_EALIGN);
+    OI_RETURN_IF(!logprob || !lse || !wsum || !xref || !unsafe || !workspace, OI_ENULL);
+    OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(wsum, 16) || !oi_aligned(xref, 4), OI_EALIGN);
     const FwdPlan p = plan_fwd(n_tokens, hidden_dim, vocab, row_mask != nullptr, true);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     char* ws = static_cast<char*>(workspace);
@@ -1612,38 +1847,55 @@ extern "C" int oi_lmhead_logp_fwd_wsum(const void* hidden, const void* weight, c
     if (row_mask)
         in = launch_selection(p.sel, ws, hidden, labels, nullptr, nullptr, row_mask, false, n_tokens, hidden_dim, queues,
                               select_clears_queues ? n_queue_words : 0, s);
+    hipLaunchKernelGGL(zero_bytes_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, unsafe, n_tokens);
     enqueue_fwd_wsum(p, ws, in, row_mask, weight, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy, lse,
-                     wsum, s);
+                     wsum, xref, unsafe, s);
     return oi_launch_status();
 }
 
-extern "C" size_t oi_lmhead_dh_workspace_bytes(int64_t n_tokens) {
-    if (n_tokens <= 0) return 0;
+namespace {
+// workspace of oi_lmhead_dh_from_wsum: the row index of the mask, and the recomputing backward for
+// the rows that the forward flagged
+struct DhPlan {
+    BwdPlan repair;
+    size_t off_rows, off_count, off_repair, total;
+};
+DhPlan plan_dh(int64_t n_tokens, int64_t hdim, int64_t vocab) {
+    DhPlan p;
+    p.repair = plan_bwd(n_tokens, hdim, vocab, true);
     Carver cv;
-    cv.take((size_t)round_up(n_tokens, 256) * sizeof(int32_t));
-    cv.take(sizeof(int32_t));
-    return cv.off;
+    p.off_rows = cv.take((size_t)round_up(n_tokens, 256) * sizeof(int32_t));
+    p.off_count = cv.take(sizeof(int32_t));
+    p.off_repair = cv.take(p.repair.total);
+    p.total = cv.off;
+    return p;
+}
+}  // namespace
+
+extern "C" size_t oi_lmhead_dh_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab) {
+    if (n_tokens <= 0 || hidden_dim <= 0 || vocab <= 0) return 0;
+    return plan_dh(n_tokens, hidden_dim, vocab).total;
 }
 
-extern "C" int oi_lmhead_dh_from_wsum(const void* weight, const int64_t* labels, const float* lse, const float* logprob,
-                                      const float* grad_logprob, const uint8_t* row_mask, const float* wsum,
-                                      int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature,
-                                      void* d_hidden, void* workspace, size_t workspace_bytes, void* stream) {
-    OI_RETURN_IF(n_tokens < 0 || hidden_dim <= 0 || vocab <= 0 || hidden_dim % 64 != 0, OI_EINVAL);
-    OI_RETURN_IF(!(inv_temperature >= 1.0e-6f) || !(inv_temperature <= 1.0e6f), OI_EINVAL);
+extern "C" int oi_lmhead_dh_from_wsum(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
+                                      const float* logprob, const float* grad_logprob, const uint8_t* row_mask,
+                                      const float* wsum, const float* xref, const uint8_t* unsafe, int64_t n_tokens,
+                                      int64_t hidden_dim, int64_t vocab, float inv_temperature, void* d_hidden,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
+    if (rc != OI_OK) return rc;
     if (n_tokens == 0) return OI_OK;
-    OI_RETURN_IF(!weight || !labels || !lse || !logprob || !grad_logprob || !wsum || !d_hidden, OI_ENULL);
-    OI_RETURN_IF(!oi_aligned(weight, 16) || !oi_aligned(wsum, 16) || !oi_aligned(d_hidden, 8), OI_EALIGN);
+    OI_RETURN_IF(!lse || !logprob || !grad_logprob || !wsum || !xref || !unsafe || !d_hidden || !workspace, OI_ENULL);
+    OI_RETURN_IF(!oi_aligned(wsum, 16) || !oi_aligned(d_hidden, 8) || !oi_aligned(workspace, 256), OI_EALIGN);
+    const DhPlan p = plan_dh(n_tokens, hidden_dim, vocab);
+    OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    char* ws = static_cast<char*>(workspace);
     const int32_t *rows = nullptr, *count = nullptr;
     if (row_mask) {
-        OI_RETURN_IF(!workspace, OI_ENULL);
-        OI_RETURN_IF(!oi_aligned(workspace, 256), OI_EALIGN);
-        OI_RETURN_IF(workspace_bytes < oi_lmhead_dh_workspace_bytes(n_tokens), OI_EWORKSPACE);
         // the same ascending selection as in the forward pass, rebuilt from the same mask
-        char* ws = static_cast<char*>(workspace);
-        int32_t* r = reinterpret_cast<int32_t*>(ws);
-        int32_t* c = reinterpret_cast<int32_t*>(ws + (size_t)round_up(n_tokens, 256) * sizeof(int32_t));
+        int32_t* r = reinterpret_cast<int32_t*>(ws + p.off_rows);
+        int32_t* c = reinterpret_cast<int32_t*>(ws + p.off_count);
         hipLaunchKernelGGL(select_rows_kernel, dim3(1), dim3(SELECT_THREADS), 0, s, row_mask,
                            static_cast<const float*>(nullptr), n_tokens, r, c, static_cast<uint32_t*>(nullptr), 0);
         hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, row_mask,
@@ -1651,37 +1903,42 @@ extern "C" int oi_lmhead_dh_from_wsum(const void* weight, const int64_t* labels,
         rows = r;
         count = c;
     }
-    hipLaunchKernelGGL(dh_from_wsum_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, wsum,
+    hipLaunchKernelGGL(dh_from_wsum_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, wsum, xref, unsafe,
                        static_cast<const uint16_t*>(weight), labels, lse, logprob, grad_logprob, rows, count, n_tokens,
                        hidden_dim, vocab, inv_temperature, static_cast<uint16_t*>(d_hidden));
+    // the flagged rows (a subset of the mask's), recomputed; normally none
+    char* ws_rep = ws + p.off_repair;
+    uint32_t* rq = reinterpret_cast<uint32_t*>(ws_rep + p.repair.off_queues);
+    const int n_words = (int)(3 * p.repair.n_chunks * QUEUE_WORDS);
+    const bool select_clears = n_words <= SELECT_THREADS;
+    if (!select_clears)
+        hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_words + 255) / 256)), dim3(256), 0, s, rq, n_words);
+    const RowInputs in = launch_selection(p.repair.sel, ws_rep, hidden, labels, lse, grad_logprob, unsafe, false,
+                                          n_tokens, hidden_dim, rq, select_clears ? n_words : 0, s, logprob);
+    enqueue_bwd(p.repair, ws_rep, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, nullptr, s);
     return oi_launch_status();
 }
 
 extern "C" size_t oi_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_dim, int64_t vocab,
-                                                int want_d_weight, int with_row_selection, int64_t cache_chunks) {
+                                                int want_d_weight, int with_row_selection) {
     if (n_tokens <= 0 || hidden_dim <= 0 || vocab <= 0) return 0;
     (void)want_d_weight;
-    return plan_bwd(n_tokens, hidden_dim, vocab, with_row_selection != 0, cache_chunks).total;
+    return plan_bwd(n_tokens, hidden_dim, vocab, with_row_selection != 0).total;
 }
 
 extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const int64_t* labels, const float* lse,
                                   const float* grad_logprob, const uint8_t* row_mask, int skip_zero_grad_rows,
                                   int64_t n_tokens, int64_t hidden_dim, int64_t vocab, float inv_temperature,
-                                  const float* logprob, void* exp_cache, int64_t cache_chunks, void* d_hidden,
-                                  void* d_weight, void* workspace, size_t workspace_bytes, void* stream) {
+                                  const float* logprob, void* d_hidden, void* d_weight, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
     int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
-    if (rc != OI_OK) return rc;
-    rc = check_cache(exp_cache, cache_chunks);
     if (rc != OI_OK) return rc;
     if (n_tokens == 0) return OI_OK;
     OI_RETURN_IF(!lse || !grad_logprob || !logprob || !d_hidden || !workspace, OI_ENULL);
-    // a cache written for the rows of a mask can only be read back for the same rows
-    OI_RETURN_IF(cache_chunks > 0 && skip_zero_grad_rows, OI_EINVAL);
     // bf16 results are stored as pairs (4-byte words)
     OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 4) || !oi_aligned(d_weight, 4), OI_EALIGN);
     const bool selecting = row_mask != nullptr || skip_zero_grad_rows != 0;
-    const CachePlan cache = plan_cache(n_tokens, vocab, cache_chunks);
-    const BwdPlan p = plan_bwd(n_tokens, hidden_dim, vocab, selecting, cache.chunks);
+    const BwdPlan p = plan_bwd(n_tokens, hidden_dim, vocab, selecting);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     hipStream_t s = static_cast<hipStream_t>(stream);
     char* ws = static_cast<char*>(workspace);
@@ -1700,53 +1957,33 @@ extern "C" int oi_lmhead_logp_bwd(const void* hidden, const void* weight, const 
         hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, row_mask,
                            zero_grad_probe, hidden_dim, static_cast<uint16_t*>(d_hidden));
     }
-    enqueue_bwd(p, ws, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, d_weight,
-                static_cast<uint16_t*>(exp_cache), cache, s);
+    enqueue_bwd(p, ws, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, d_weight, s);
     return oi_launch_status();
 }
 
 extern "C" size_t oi_lmhead_grpo_workspace_bytes(int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab,
-                                                 int64_t cache_chunks) {
+                                                 int want_d_weight, int64_t slab_tokens) {
     if (rows <= 0 || cols <= 0 || hidden_dim <= 0 || vocab <= 0) return 0;
-    if (cache_chunks < 0) return plan_slabs(rows, cols, hidden_dim, vocab, true, -cache_chunks).total;
-    return plan_step(rows, cols, hidden_dim, vocab, cache_chunks).total;
+    if (slab_tokens > 0) return plan_slabs(rows * cols, rows, cols, hidden_dim, vocab, want_d_weight != 0, slab_tokens).total;
+    return plan_step(rows, cols, hidden_dim, vocab).total;
 }
 
 namespace {
-// oi_lmhead_grpo_fwd_bwd in slabs of tokens (cache_chunks < 0); arguments as checked by the entry point
+// oi_lmhead_grpo_fwd_bwd in slabs of tokens (slab_tokens > 0); arguments as checked by the entry point
 int grpo_step_in_slabs(const void* hidden, const void* weight, const int64_t* labels, const uint8_t* mask,
                        const float* old_logprobs, const float* ref_logprobs, const float* advantages,
                        const float* rho_weights, int64_t rows, int64_t cols, int64_t hidden_dim, int64_t vocab,
                        float inv_temperature, int loss_fn, float ratio_lo, float ratio_hi, int kl_estimator, float beta,
                        int axis_mode, float denominator, float scale, float* logprob, float* entropy, float* out_stats,
-                       void* d_hidden, void* d_weight, int64_t slab_units, void* workspace, size_t workspace_bytes,
+                       void* d_hidden, void* d_weight, int64_t slab_tokens, void* workspace, size_t workspace_bytes,
                        void* stream) {
     const int64_t n_tokens = rows * cols;
-    const SlabPlan p = plan_slabs(rows, cols, hidden_dim, vocab, d_weight != nullptr, slab_units);
+    const SlabPlan p = plan_slabs(n_tokens, rows, cols, hidden_dim, vocab, d_weight != nullptr, slab_tokens);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     hipStream_t s = static_cast<hipStream_t>(stream);
     char* ws = static_cast<char*>(workspace);
-    char* ws_fwd = ws + p.off_fwd;
-    char* ws_bwd = ws + p.off_bwd;
-    float* lse = reinterpret_cast<float*>(ws + p.off_lse);
     float* grad = reinterpret_cast<float*>(ws + p.off_grad);
     float* row_denoms = reinterpret_cast<float*>(ws + p.off_denoms);
-    int32_t* counts = reinterpret_cast<int32_t*>(ws + p.off_counts);
-    uint16_t* ecache = reinterpret_cast<uint16_t*>(ws + p.off_cache);
-    float* dw32 = d_weight && p.n_slabs > 1 ? reinterpret_cast<float*>(ws + p.off_dw32) : nullptr;
-    uint32_t* fwd_queue = reinterpret_cast<uint32_t*>(ws_fwd + p.fwd.off_queue);
-    uint32_t* bwd_queues = reinterpret_cast<uint32_t*>(ws_bwd + p.bwd.off_queues);
-    const int n_bwd_words = (int)(3 * p.bwd.n_chunks * QUEUE_WORDS);
-
-    // one selection for every slab (the plan's offsets are relative to the workspace)
-    const RowInputs all = launch_selection(p.sel, ws, hidden, labels, nullptr, nullptr, mask, false, n_tokens, hidden_dim,
-                                           static_cast<uint32_t*>(nullptr), 0, s);
-    hipLaunchKernelGGL(slab_counts_kernel, dim3((unsigned)((p.n_slabs + 63) / 64)), dim3(64), 0, s, all.n_dev, (int)p.slab,
-                       (int)p.n_slabs, counts);
-    hipLaunchKernelGGL(zero_unselected_f32_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, mask,
-                       n_tokens, logprob, entropy, lse);
-    hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, mask,
-                       static_cast<const float*>(nullptr), hidden_dim, static_cast<uint16_t*>(d_hidden));
     // the denominators come from the mask alone: a first pass of the statistics over logprobs that are
     // not there yet leaves them in row_denoms (its other results are overwritten at the end)
     int rc = oi_grpo_fused_fwd(logprob, old_logprobs, ref_logprobs, advantages, mask, rho_weights, entropy, nullptr, nullptr,
@@ -1754,35 +1991,25 @@ int grpo_step_in_slabs(const void* hidden, const void* weight, const int64_t* la
                                denominator, scale, out_stats, row_denoms, ws + p.off_stats,
                                oi_grpo_fused_workspace_bytes(rows, cols), stream);
     if (rc != OI_OK) return rc;
-    float* lse_c = reinterpret_cast<float*>(ws + p.sel.off_lse);
-    float* grad_c = reinterpret_cast<float*>(ws + p.sel.off_grad);
-    float* logprob_c = reinterpret_cast<float*>(ws + p.sel.off_logprob);
-    for (int64_t i = 0; i < p.n_slabs; ++i) {
-        const int64_t r0 = i * p.slab;
-        RowInputs in = {all.hidden + r0 * hidden_dim, all.labels + r0, nullptr, nullptr, all.rows + r0, counts + i, nullptr};
-        hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, s, fwd_queue, FWD_QUEUE_WORDS);
-        hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_bwd_words + 255) / 256)), dim3(256), 0, s, bwd_queues,
-                           n_bwd_words);
-        enqueue_fwd(p.fwd, ws_fwd, in, nullptr, weight, p.slab, hidden_dim, vocab, inv_temperature, logprob, entropy, lse,
-                    ecache, p.cache, s);
-        // every token's d loss / d logprob; only this slab's tokens are read below (later slabs' are not there yet)
-        rc = oi_grpo_fused_bwd(logprob, old_logprobs, ref_logprobs, advantages, mask, rho_weights, rows, cols, loss_fn,
-                               ratio_lo, ratio_hi, kl_estimator, beta, scale, row_denoms, nullptr, grad, stream);
-        if (rc != OI_OK) return rc;
-        hipLaunchKernelGGL(gather_f32_kernel, dim3((unsigned)((p.slab + 255) / 256)), dim3(256), 0, s, lse, grad, logprob,
-                           in.rows, in.n_dev, lse_c + r0, grad_c + r0, logprob_c + r0);
-        in.lse = lse_c + r0;
-        in.grad = grad_c + r0;
-        in.logprob = logprob_c + r0;
-        const int dw_mode = p.n_slabs == 1 ? 2 : (i == 0 ? 0 : 1);
-        enqueue_bwd(p.bwd, ws_bwd, in, weight, p.slab, hidden_dim, vocab, inv_temperature, d_hidden, d_weight, ecache,
-                    p.cache, s, dw_mode, dw32);
-    }
-    if (dw32) {
-        const int64_t n8 = vocab * hidden_dim / 8;  // hidden_dim is a multiple of 64
-        hipLaunchKernelGGL(f32_to_bf16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, s, dw32, n8,
-                           static_cast<uint16_t*>(d_weight));
-    }
+    const SlabStep st = {hidden, weight, labels, mask, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy,
+                         d_hidden, d_weight};
+    rc = run_slab_passes(
+        p, ws, st, s,
+        [&](int32_t* order, int32_t* count, SlabMeta* meta) {
+            hipLaunchKernelGGL(select_rows_kernel, dim3(1), dim3(SELECT_THREADS), 0, s, mask,
+                               static_cast<const float*>(nullptr), n_tokens, order, count,
+                               static_cast<uint32_t*>(nullptr), 0);
+            hipLaunchKernelGGL(plan_equal_slabs_kernel, dim3((unsigned)((p.n_passes + 63) / 64)), dim3(64), 0, s, count,
+                               (int)p.cap, (int)p.n_passes, meta);
+        },
+        [&](bool) {
+            // every token's d loss / d logprob from its own logprob; tokens of later slabs hold numbers
+            // that nobody reads before their own slab has overwritten them
+            return oi_grpo_fused_bwd(logprob, old_logprobs, ref_logprobs, advantages, mask, rho_weights, rows, cols,
+                                     loss_fn, ratio_lo, ratio_hi, kl_estimator, beta, scale, row_denoms, nullptr, grad,
+                                     stream);
+        });
+    if (rc != OI_OK) return rc;
     // loss and statistics from all logprobs
     return oi_grpo_fused_fwd(logprob, old_logprobs, ref_logprobs, advantages, mask, rho_weights, entropy, nullptr, nullptr,
                              nullptr, nullptr, rows, cols, loss_fn, ratio_lo, ratio_hi, kl_estimator, beta, axis_mode,
@@ -1797,23 +2024,20 @@ extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, co
                                       int64_t hidden_dim, int64_t vocab, float inv_temperature, int loss_fn,
                                       float ratio_lo, float ratio_hi, int kl_estimator, float beta, int axis_mode,
                                       float denominator, float scale, float* logprob, float* entropy, float* out_stats,
-                                      void* d_hidden, void* d_weight, void* exp_cache, int64_t cache_chunks,
-                                      void* workspace, size_t workspace_bytes, void* stream) {
-    OI_RETURN_IF(rows <= 0 || cols <= 0 || rows > MAX_LD || cols > MAX_LD, OI_EINVAL);
+                                      void* d_hidden, void* d_weight, int64_t slab_tokens, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+    OI_RETURN_IF(rows <= 0 || cols <= 0 || rows > MAX_LD || cols > MAX_LD || slab_tokens < 0, OI_EINVAL);
     const int64_t n_tokens = rows * cols;
     int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
     if (rc != OI_OK) return rc;
     OI_RETURN_IF(!mask || !advantages || !logprob || !out_stats || !d_hidden || !workspace, OI_ENULL);
     OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 4) || !oi_aligned(d_weight, 4), OI_EALIGN);
-    if (cache_chunks < 0)
+    if (slab_tokens > 0)
         return grpo_step_in_slabs(hidden, weight, labels, mask, old_logprobs, ref_logprobs, advantages, rho_weights, rows,
                                   cols, hidden_dim, vocab, inv_temperature, loss_fn, ratio_lo, ratio_hi, kl_estimator,
                                   beta, axis_mode, denominator, scale, logprob, entropy, out_stats, d_hidden, d_weight,
-                                  -cache_chunks, workspace, workspace_bytes, stream);
-    rc = check_cache(exp_cache, cache_chunks);
-    if (rc != OI_OK) return rc;
-    const CachePlan cache = plan_cache(n_tokens, vocab, cache_chunks);
-    const StepPlan p = plan_step(rows, cols, hidden_dim, vocab, cache.chunks);
+                                  slab_tokens, workspace, workspace_bytes, stream);
+    const StepPlan p = plan_step(rows, cols, hidden_dim, vocab);
     OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
     hipStream_t s = static_cast<hipStream_t>(stream);
     char* ws = static_cast<char*>(workspace);
@@ -1822,7 +2046,6 @@ extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, co
     float* lse = reinterpret_cast<float*>(ws + p.off_lse);
     float* grad = reinterpret_cast<float*>(ws + p.off_grad);
     float* row_denoms = reinterpret_cast<float*>(ws + p.off_denoms);
-    uint16_t* ecache = static_cast<uint16_t*>(exp_cache);
 
     // one selection for both passes: it lives in the backward region; the select kernel also clears
     // the backward queues, the forward queue gets the small fill kernel
@@ -1837,7 +2060,7 @@ extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, co
     RowInputs in = launch_selection(p.bwd.sel, ws_bwd, hidden, labels, nullptr, nullptr, mask, false, n_tokens,
                                     hidden_dim, bwd_queues, select_clears_queues ? n_queue_words : 0, s);
     enqueue_fwd(p.fwd, ws_fwd, in, mask, weight, n_tokens, hidden_dim, vocab, inv_temperature, logprob, entropy, lse,
-                ecache, cache, s);
+                KeepPlan{nullptr, 0, 0, nullptr, nullptr}, s);
 
     // loss and statistics from the logprobs, then every token's d loss / d logprob (upstream gradient 1)
     rc = oi_grpo_fused_fwd(logprob, old_logprobs, ref_logprobs, advantages, mask, rho_weights, entropy, nullptr, nullptr,
@@ -1859,9 +2082,39 @@ extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, co
     in.logprob = logprob_c;
     hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n_tokens), dim3(256), 0, s, mask,
                        static_cast<const float*>(nullptr), hidden_dim, static_cast<uint16_t*>(d_hidden));
-    enqueue_bwd(p.bwd, ws_bwd, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, d_weight, ecache,
-                cache, s);
+    enqueue_bwd(p.bwd, ws_bwd, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, d_weight, s);
     return oi_launch_status();
+}
+
+extern "C" int oi_lmhead_probe_arm(int kernel) {
+    OI_RETURN_IF(kernel < 0 || kernel > 2 || g_probe.kernel >= 0, OI_EINVAL);
+    for (int i = 0; i < 2 * Probe::MAX_LAUNCHES; ++i) {
+        const hipError_t e = hipEventCreate(&g_probe.ev[i]);
+        if (e != hipSuccess) {
+            for (int j = 0; j < i; ++j) (void)hipEventDestroy(g_probe.ev[j]);
+            return (int)e;
+        }
+    }
+    g_probe.used = 0;
+    g_probe.kernel = kernel;
+    return OI_OK;
+}
+
+extern "C" int oi_lmhead_probe_read(float* ms, int capacity, int* n_launches) {
+    OI_RETURN_IF(g_probe.kernel < 0 || capacity < 0, OI_EINVAL);
+    OI_RETURN_IF(!n_launches || (capacity > 0 && !ms), OI_ENULL);
+    const int n = g_probe.used < capacity ? g_probe.used : capacity;
+    int rc = OI_OK;
+    for (int i = 0; i < n && rc == OI_OK; ++i) {
+        hipError_t e = hipEventSynchronize(g_probe.ev[2 * i + 1]);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms[i], g_probe.ev[2 * i], g_probe.ev[2 * i + 1]);
+        if (e != hipSuccess) rc = (int)e;
+    }
+    *n_launches = g_probe.used;
+    for (int i = 0; i < 2 * Probe::MAX_LAUNCHES; ++i) (void)hipEventDestroy(g_probe.ev[i]);
+    g_probe.kernel = -1;
+    g_probe.used = 0;
+    return rc;
 }
 
 extern "C" int oi_gemm_bf16_tn(const void* A, int64_t lda, int64_t M, const void* B, int64_t ldb, int64_t N, int64_t K,

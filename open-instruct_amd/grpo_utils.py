@@ -422,6 +422,19 @@ def _grpo_on_logits_launch(logits, labels, old, ref, adv, rho, coef, inv_tempera
     return logprob, entropy, dlogits
 
 
+def _hand_out_once(ctx) -> None:
+    """The stored gradients are scaled by the upstream gradient in place (the host never reads that
+    scalar, so it cannot tell whether it is 1), which can be done once: a second backward over a
+    retained graph would scale what the first one left.  It raises instead of returning that."""
+    if ctx.handed_out:
+        raise RuntimeError(
+            "the gradients of this fused loss were computed inside its forward call and have been handed out "
+            "(scaled in place by the upstream gradient) by an earlier backward(); call the loss function again "
+            "instead of backpropagating through it a second time"
+        )
+    ctx.handed_out = True
+
+
 class _AttachLogitsGrad(torch.autograd.Function):
     """Identity on the loss value whose backward hands out the gradient computed in the forward."""
 
@@ -434,9 +447,7 @@ class _AttachLogitsGrad(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_loss):
         (dlogits,) = ctx.saved_tensors
-        if ctx.handed_out:  # a second backward over a retained graph must not scale the same memory twice
-            dlogits = dlogits.clone()
-        ctx.handed_out = True
+        _hand_out_once(ctx)
         # The usual upstream gradient of a loss is exactly 1 and the stored tensor is the answer as it
         # is.  The kernel reads the device scalar and returns at once in that case; anything else is
         # applied in place.  The host never looks at the value.
@@ -530,10 +541,7 @@ class _AttachHeadGrads(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_loss):
         d_hidden, d_weight = ctx.saved_tensors
-        if ctx.handed_out:  # a second backward over a retained graph must not scale the same memory twice
-            d_hidden = d_hidden.clone()
-            d_weight = None if d_weight is None else d_weight.clone()
-        ctx.handed_out = True
+        _hand_out_once(ctx)
         g = _lib.f32c(grad_loss.detach()).reshape(1)
         for t in (d_hidden, d_weight):  # nothing is touched when the device scalar is exactly 1
             if t is not None:
@@ -543,6 +551,10 @@ class _AttachHeadGrads(torch.autograd.Function):
                 )  # fmt: skip
         need_h, need_w = ctx.needs_input_grad[1], ctx.needs_input_grad[2]
         return None, (d_hidden if need_h else None), (d_weight if need_w else None), None, None
+
+
+# slab size of the no-recompute step when the caller names none (selected tokens per slab)
+DEFAULT_SLAB_TOKENS = 8192
 
 
 def grpo_loss_on_hidden(
@@ -559,8 +571,7 @@ def grpo_loss_on_hidden(
     loss_denominator: float | None = None,
     axis: int | None = None,
     dp_scale: float = 1.0,
-    logit_cache_chunks: int | str = 0,
-    token_slabs: bool | int = False,
+    token_slabs: bool | int = True,
 ) -> tuple[torch.Tensor, dict[str, torch.Tensor], torch.Tensor, torch.Tensor]:
     """GRPO loss straight from final hidden states; returns ``(loss, stats, logprobs, entropy)``.
 
@@ -574,17 +585,23 @@ def grpo_loss_on_hidden(
     broadcasts).  ``logprobs`` and ``entropy`` are returned detached, 0 off the mask.  Without a
     gradient to compute (``torch.no_grad()``, inputs without ``requires_grad``) only the forward runs.
 
-    ``token_slabs=True`` (or a slab size in tokens, a multiple of 4096; ``True`` = 8192) runs the step in
-    slabs of that many selected tokens without recomputing anything: a
-    slab's forward leaves its exponentials (all vocabulary columns, bf16) in a slab-sized scratch
+    ``token_slabs`` (default ``True`` = slabs of at most ``DEFAULT_SLAB_TOKENS`` selected tokens; or a
+    number of tokens) runs the step slab by slab without recomputing anything: the selected rows are
+    split on the device into the fewest equal slabs, a slab's forward leaves its exponentials (all
+    vocabulary columns, bf16, relative to each token's own label logit) in a slab-sized scratch
     buffer, the slab's tokens get their upstream gradient at once, and both backward products read
     that buffer before the next slab overwrites it (``d_weight`` accumulates in fp32 over the
     slabs).  6·N·H·V of matrix work instead of 8·N·H·V; the scratch is ``[slab, vocab]`` bf16 plus an
     fp32 ``[vocab, hidden]``, never ``[tokens, vocab]``.  Larger slabs are faster (fewer passes over the
-    fp32 ``d_weight``, fewer launch ends).  Not together with ``logit_cache_chunks``.
+    fp32 ``d_weight``, fewer launch ends).  The route has no limit on the size of the logits or on the
+    temperature: a token whose label is extremely unlikely (largest logit more than 44 nats above the
+    label's) or whose logits hold a NaN is flagged on the device and served by a recomputing backward
+    over the flagged rows inside the same call.  ``token_slabs=False`` is the recomputing step: one
+    forward over all selected rows, then a backward that recomputes the logits one vocabulary chunk at
+    a time (8·N·H·V, scratch ``[tokens, 32768]`` bf16).
+
+    ``loss.backward()`` may be called once per call of this function.
     """
-    if token_slabs and logit_cache_chunks not in (0, None):
-        raise ValueError("token_slabs keeps its own scratch; it cannot be combined with logit_cache_chunks")
     if axis not in (None, 1, -1):
         raise ValueError("axis must be None or the token axis (1)")
     if loss_denominator is not None and float(loss_denominator) <= 0.0:
@@ -629,30 +646,20 @@ def grpo_loss_on_hidden(
     d_hidden = torch.empty_like(hid)
     d_weight = torch.empty_like(w) if weight.requires_grad else None
     lib = _lib.load()
-    from . import lm_head
-
-    cache_chunks = lm_head.resolve_cache_chunks(logit_cache_chunks, rows * cols, v, dev) if rows * cols > 0 else 0
-    cache = None
+    slab_tokens = 0
     if token_slabs:
-        # the C entry's tag for the slab-wise step (minus the slab size in units of 4096 rows); its scratch is
-        # part of the workspace
-        slab_tokens = 8192 if token_slabs is True else int(token_slabs)
-        if slab_tokens < 4096 or slab_tokens % 4096:
-            raise ValueError("token_slabs must be True or a multiple of 4096 tokens")
-        cache_chunks = -(slab_tokens // 4096)
-    elif cache_chunks:
-        cache = torch.empty(lib.oi_lmhead_cache_bytes(rows * cols, v, cache_chunks), dtype=torch.uint8, device=dev)
-    if cache is None and cache_chunks > 0:
-        cache_chunks = 0
-    ws_bytes = lib.oi_lmhead_grpo_workspace_bytes(rows, cols, h, v, cache_chunks)
+        slab_tokens = DEFAULT_SLAB_TOKENS if token_slabs is True else int(token_slabs)
+        if slab_tokens < 256:
+            raise ValueError("token_slabs must be True, False or a number of tokens (at least 256)")
+    ws_bytes = lib.oi_lmhead_grpo_workspace_bytes(rows, cols, h, v, int(d_weight is not None), slab_tokens)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     _lib.call(
         "oi_lmhead_grpo_fwd_bwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), m.data_ptr(), _lib.ptr(old_c),
         _lib.ptr(ref_c), adv_c.data_ptr(), _lib.ptr(rho_c), rows, cols, h, v, inv_t, _loss_fn_tag(config), lo, hi,
         int(config.kl_estimator), float(config.beta), 0 if axis is None else 1,
         0.0 if loss_denominator is None else float(loss_denominator), float(dp_scale), logprob.data_ptr(),
-        entropy.data_ptr(), stats.data_ptr(), d_hidden.data_ptr(), _lib.ptr(d_weight), _lib.ptr(cache), cache_chunks,
-        ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
+        entropy.data_ptr(), stats.data_ptr(), d_hidden.data_ptr(), _lib.ptr(d_weight), slab_tokens, ws.data_ptr(),
+        ws_bytes, _lib.stream_of(hid),
     )  # fmt: skip
     loss = _AttachHeadGrads.apply(stats[0], hidden, weight, d_hidden.reshape(hidden.shape), d_weight)
     return loss, _StatsView(stats), logprob, entropy

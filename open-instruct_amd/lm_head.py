@@ -17,30 +17,10 @@ import torch
 from . import _lib
 
 
-# share of the free device memory that ``logit_cache_chunks="auto"`` may take for the cache of exponentials
-AUTO_CACHE_MEMORY_SHARE = 0.25
-
-
-def resolve_cache_chunks(logit_cache_chunks, n_tokens: int, vocab: int, device) -> int:
-    """Number of vocabulary chunks to cache.  An integer is taken as it is; ``"auto"`` takes as many
-    chunks as fit into a quarter of the device memory that is free right now (2 bytes per cached
-    logit), which on a 288 GB part is all of them for any batch the path is used with."""
-    if logit_cache_chunks != "auto":
-        return max(0, int(logit_cache_chunks))
-    lib = _lib.load()
-    n_chunks = -(-int(vocab) // 32768)
-    free, _total = torch.cuda.mem_get_info(device)
-    budget = int(free * AUTO_CACHE_MEMORY_SHARE)
-    chunks = n_chunks
-    while chunks > 0 and lib.oi_lmhead_cache_bytes(n_tokens, vocab, chunks) > budget:
-        chunks -= 1
-    return chunks
-
-
 class _FusedLMHead(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, weight, labels, mask, inv_temperature, want_entropy, compact_backward=False,
-                cache_chunks=0, dhidden_in_forward="auto"):
+                dhidden_in_forward="auto"):
         dev = _lib.require_gpu(hidden, weight, labels, mask)
         if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
             raise ValueError("fused lm_head expects bf16 hidden states and weight")
@@ -62,82 +42,73 @@ class _FusedLMHead(torch.autograd.Function):
         logprob = torch.empty(n, dtype=torch.float32, device=dev)
         entropy = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
         lse = torch.empty(n, dtype=torch.float32, device=dev)
-        # the cache of exponentials only pays for itself when a backward pass follows
-        wants_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
-        cache_chunks = resolve_cache_chunks(cache_chunks, n, v, dev) if wants_grad and n > 0 else 0
-        if cache_chunks and compact_backward:
-            raise ValueError("compact_backward re-selects rows in the backward pass; it cannot be combined with a cache")
         # a backward pass that only needs d_hidden is prepared while the logits exist (no recomputation)
         if dhidden_in_forward == "auto":
-            dhidden_in_forward = not cache_chunks and not compact_backward
+            dhidden_in_forward = not compact_backward
         wsum_mode = bool(dhidden_in_forward) and ctx.needs_input_grad[0] and not ctx.needs_input_grad[1] and n > 0
-        if wsum_mode and (cache_chunks or compact_backward):
-            raise ValueError("dhidden_in_forward cannot be combined with a cache of exponentials or compact_backward")
-        cache = wsum = None
+        if wsum_mode and compact_backward:
+            raise ValueError("dhidden_in_forward cannot be combined with compact_backward")
+        wsum = xref = unsafe = None
         if wsum_mode:
             lib = _lib.load()
             wsum = torch.empty(n, h, dtype=torch.float32, device=dev)
+            xref = torch.empty(n, dtype=torch.float32, device=dev)
+            unsafe = torch.empty(n, dtype=torch.uint8, device=dev)
             ws_bytes = lib.oi_lmhead_fwd_wsum_workspace_bytes(n, h, v, int(m is not None))
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
             _lib.call(
                 "oi_lmhead_logp_fwd_wsum", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), _lib.ptr(m), n, h, v,
-                inv_temperature, logprob.data_ptr(), _lib.ptr(entropy), lse.data_ptr(), wsum.data_ptr(), ws.data_ptr(),
-                ws_bytes, _lib.stream_of(hid),
+                inv_temperature, logprob.data_ptr(), _lib.ptr(entropy), lse.data_ptr(), wsum.data_ptr(),
+                xref.data_ptr(), unsafe.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
             )  # fmt: skip
         elif n > 0:
             lib = _lib.load()
-            if cache_chunks > 0:
-                cache = torch.empty(lib.oi_lmhead_cache_bytes(n, v, cache_chunks), dtype=torch.uint8, device=dev)
             ws_bytes = lib.oi_lmhead_fwd_workspace_bytes(n, h, v, int(m is not None))
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
             _lib.call(
                 "oi_lmhead_logp_fwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), _lib.ptr(m), n, h, v,
-                inv_temperature, logprob.data_ptr(), _lib.ptr(entropy), lse.data_ptr(), _lib.ptr(cache),
-                cache_chunks if cache is not None else 0, ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
+                inv_temperature, logprob.data_ptr(), _lib.ptr(entropy), lse.data_ptr(), ws.data_ptr(), ws_bytes,
+                _lib.stream_of(hid),
             )  # fmt: skip
-        ctx.save_for_backward(hid, w, lab, lse, m, cache, logprob, wsum)
+        ctx.save_for_backward(hid, w, lab, lse, m, logprob, wsum, xref, unsafe)
         ctx.inv_temperature = inv_temperature
         ctx.compact_backward = bool(compact_backward)
-        ctx.cache_chunks = cache_chunks if cache is not None else 0
         if want_entropy:
             ctx.mark_non_differentiable(entropy)
         return logprob, entropy
 
     @staticmethod
     def backward(ctx, grad_logprob, _grad_entropy):
-        hid, w, lab, lse, m, cache, logprob, wsum = ctx.saved_tensors
+        hid, w, lab, lse, m, logprob, wsum, xref, unsafe = ctx.saved_tensors
         n, h = hid.shape
         v = w.shape[0]
         need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if grad_logprob is None or not (need_h or need_w):
-            return (None,) * 9
+            return (None,) * 8
         g = _lib.f32c(grad_logprob)
         d_hidden = torch.empty_like(hid)
         if wsum is not None:
-            ws_bytes = _lib.load().oi_lmhead_dh_workspace_bytes(n) if m is not None else 0
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=hid.device) if ws_bytes else None
+            ws_bytes = _lib.load().oi_lmhead_dh_workspace_bytes(n, h, v)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=hid.device)
             _lib.call(
-                "oi_lmhead_dh_from_wsum", w.data_ptr(), lab.data_ptr(), lse.data_ptr(), logprob.data_ptr(), g.data_ptr(),
-                _lib.ptr(m), wsum.data_ptr(), n, h, v, ctx.inv_temperature, d_hidden.data_ptr(), _lib.ptr(ws), ws_bytes,
-                _lib.stream_of(hid),
+                "oi_lmhead_dh_from_wsum", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), lse.data_ptr(),
+                logprob.data_ptr(), g.data_ptr(), _lib.ptr(m), wsum.data_ptr(), xref.data_ptr(), unsafe.data_ptr(), n, h,
+                v, ctx.inv_temperature, d_hidden.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
             )  # fmt: skip
-            return (d_hidden,) + (None,) * 8
+            return (d_hidden,) + (None,) * 7
         d_weight = torch.empty_like(w) if need_w else None
         if n > 0:
             selecting = m is not None or ctx.compact_backward
-            ws_bytes = _lib.load().oi_lmhead_bwd_workspace_bytes(
-                n, h, v, int(need_w), int(selecting), ctx.cache_chunks
-            )
+            ws_bytes = _lib.load().oi_lmhead_bwd_workspace_bytes(n, h, v, int(need_w), int(selecting))
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=hid.device)
             _lib.call(
                 "oi_lmhead_logp_bwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), lse.data_ptr(), g.data_ptr(),
                 _lib.ptr(m), int(ctx.compact_backward), n, h, v, ctx.inv_temperature, _lib.ptr(logprob),
-                _lib.ptr(cache), ctx.cache_chunks, d_hidden.data_ptr(), _lib.ptr(d_weight), ws.data_ptr(), ws_bytes,
-                _lib.stream_of(hid),
+                d_hidden.data_ptr(), _lib.ptr(d_weight), ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
             )  # fmt: skip
         elif d_weight is not None:
             d_weight.zero_()
-        return (d_hidden if need_h else None), d_weight, None, None, None, None, None, None, None
+        return (d_hidden if need_h else None), d_weight, None, None, None, None, None, None
 
 
 def fused_lm_head_logprobs(
@@ -148,7 +119,6 @@ def fused_lm_head_logprobs(
     mask: torch.Tensor | None = None,
     return_entropy: bool = False,
     compact_backward: bool = False,
-    logit_cache_chunks: int | str = 0,
     dhidden_in_forward: bool | str = "auto",
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """``log_softmax(hidden @ weight.T / temperature)[labels]`` (+ entropy) per token, fp32.
@@ -164,19 +134,22 @@ def fused_lm_head_logprobs(
     upstream gradient is exactly zero (zero-advantage completions, clipped ratios without a KL
     term) out of the backward products; it changes no result.
 
-    ``logit_cache_chunks`` (default 0: nothing of size ``[tokens, vocab]`` ever exists and the
-    backward recomputes every vocabulary chunk) trades memory for that recomputation: the forward
-    keeps ``2^(logit / temperature * log2 e)`` in bf16 for the first so many chunks of 32768 vocabulary
-    columns (2 bytes per cached logit, held until the backward pass) and the backward multiplies
-    the cache directly.  With every chunk cached a quarter of the step's matrix work goes away.
-    ``"auto"`` caches as many chunks as fit into a quarter of the free device memory.
+    Nothing of size ``[tokens, vocab]`` ever exists.  When ``weight`` takes a gradient the backward
+    recomputes the logits one vocabulary chunk at a time (for a step without that recomputation see
+    :func:`open_instruct_amd.grpo_utils.grpo_loss_on_hidden` and
+    :func:`open_instruct_amd.dpo_utils.dpo_loss_on_hidden`, which know the loss and can therefore
+    finish a slab of tokens before they start the next).
 
     ``dhidden_in_forward`` (default ``"auto"``: on whenever ``hidden`` takes a gradient and ``weight``
     does not, e.g. a frozen lm_head) lets the forward also accumulate, per token, the
     softmax-weighted sum of the weight rows, which is all the backward to ``hidden`` needs besides
     the upstream gradient: the backward is then one pass over ``[tokens, hidden]`` and the logits
     are never recomputed (4·N·H·V matrix work for both passes instead of 6·N·H·V).  It holds an
-    fp32 ``[tokens, hidden]`` tensor between the passes.
+    fp32 ``[tokens, hidden]`` tensor between the passes.  The exponentials behind that sum are kept
+    relative to each token's own label logit, so the route has no limit on the size of the logits or
+    on the temperature; a token whose label is extremely unlikely (its largest logit more than 44
+    nats above the label's) or whose logits hold a NaN is flagged on the device and recomputed in the
+    backward pass like a row of the recomputing route, with the same results.
     """
     lead = hidden.shape[:-1]
     hid2 = hidden.reshape(-1, hidden.shape[-1])
@@ -186,9 +159,7 @@ def fused_lm_head_logprobs(
         raise ValueError(f"temperature must be positive, got {temperature}")
     if mask is not None and tuple(mask.shape) != tuple(lead):
         raise ValueError(f"mask {tuple(mask.shape)} does not match the rows of hidden {tuple(lead)}")
-    lp, ent = _FusedLMHead.apply(
-        hid2, weight, lab1, mask, inv_t, return_entropy, compact_backward, logit_cache_chunks, dhidden_in_forward
-    )
+    lp, ent = _FusedLMHead.apply(hid2, weight, lab1, mask, inv_t, return_entropy, compact_backward, dhidden_in_forward)
     return lp.reshape(lead), (ent.reshape(lead) if ent is not None else None)
 
 
@@ -200,7 +171,6 @@ def fused_linear_cross_entropy(
     shift_labels: torch.Tensor | None = None,
     num_items_in_batch: torch.Tensor | int | float | None = None,
     ignore_index: int = -100,
-    logit_cache_chunks: int = 0,
     token_slabs: bool | int = False,
 ) -> torch.Tensor:
     """Causal-LM cross-entropy of ``hidden @ weight.T`` against next-token labels, scalar fp32.
@@ -211,9 +181,8 @@ def fused_linear_cross_entropy(
     label equals ``ignore_index`` are never multiplied.  The result is the mean over kept tokens,
     or ``sum / num_items_in_batch`` when that count is given (gradient accumulation over several
     micro-batches).  Differentiable with respect to ``hidden`` and ``weight``.
-    ``logit_cache_chunks`` as for :func:`fused_lm_head_logprobs`.
 
-    ``token_slabs`` (``True`` = slabs of 8192 kept tokens, or a multiple of 4096) computes the loss and
+    ``token_slabs`` (``True`` = the default slab size, or a number of tokens) computes the loss and
     both gradients in one call with nothing recomputed: every token's upstream gradient is the known
     constant ``-1 / count``, so the step can run slab by slab like
     :func:`open_instruct_amd.grpo_utils.grpo_loss_on_hidden` (whose ``loss_fn="cispo"`` term with
@@ -245,7 +214,7 @@ def fused_linear_cross_entropy(
             loss_denominator=denominator, token_slabs=token_slabs,
         )  # fmt: skip
         return loss
-    logps, _ = fused_lm_head_logprobs(hidden, weight, shift_labels, mask=keep, logit_cache_chunks=logit_cache_chunks)
+    logps, _ = fused_lm_head_logprobs(hidden, weight, shift_labels, mask=keep)
     total = -logps.sum()
     if num_items_in_batch is None:
         return total / keep.sum().clamp(min=1)

@@ -42,9 +42,6 @@ class DPOLMHead(torch.nn.Module):
     """
 
     score_ignored_positions = False
-    # > 0: keep 2^logit of that many vocabulary chunks in bf16 for the backward pass instead of
-    # recomputing them (see lm_head.fused_lm_head_logprobs); 0 stores nothing of size [tokens, vocab]
-    logit_cache_chunks = 0
 
     def __init__(self, d_model: int, vocab_size: int, bias: bool = False, norm: torch.nn.Module | None = None,
                  dtype: torch.dtype = torch.bfloat16, device=None):  # fmt: skip
@@ -73,9 +70,7 @@ class DPOLMHead(torch.nn.Module):
             return self.w_out(h)
         shifted = padding_free_collator.shift_labels(labels)
         keep = None if self.score_ignored_positions else shifted != ignore_index
-        per_token_logps, _ = lm_head.fused_lm_head_logprobs(
-            h, self.w_out.weight, shifted, mask=keep, logit_cache_chunks=self.logit_cache_chunks
-        )
+        per_token_logps, _ = lm_head.fused_lm_head_logprobs(h, self.w_out.weight, shifted, mask=keep)
         return LMOutputWithLoss(
             logits=None, loss=per_token_logps, ce_loss=per_token_logps.detach().clone(), z_loss=None
         )

@@ -62,7 +62,7 @@ def test_rejected_arguments_return_codes_without_launching():
     # empty problem is fine
     assert lib.oi_lsg_entropy_fwd(None, 0, 0, 4, 0, 8, 8, None, 1.0, None, None, None, None) == 0
     # hidden size not a multiple of 64
-    assert lib.oi_lmhead_logp_fwd(None, None, None, None, 4, 100, 32, 1.0, None, None, None, None, 0, None, 0, None) == -1
+    assert lib.oi_lmhead_logp_fwd(None, None, None, None, 4, 100, 32, 1.0, None, None, None, None, 0, None) == -1
     # unknown loss function / estimator
     assert lib.oi_grpo_terms_fwd(None, None, None, None, None, 4, 7, 0.8, 1.2, 2, None, None, None, None) == -1
     assert lib.oi_grpo_terms_fwd(None, None, None, None, None, 4, 0, 0.8, 1.2, 9, None, None, None, None) == -1
@@ -71,8 +71,8 @@ def test_rejected_arguments_return_codes_without_launching():
     assert lib.oi_seq_logp_fwd(None, None, None, 2, 0, 0, None, None, None) == -1
     # row strides beyond 2^22 elements do not fit the tile engine's 32-bit lane offsets
     big = (1 << 22) + 64
-    assert lib.oi_lmhead_logp_fwd(None, None, None, None, 4, big, 32, 1.0, None, None, None, None, 0, None, 0, None) == -1
-    assert lib.oi_lmhead_logp_fwd(None, None, None, None, big, 64, 32, 1.0, None, None, None, None, 0, None, 0, None) == -1
+    assert lib.oi_lmhead_logp_fwd(None, None, None, None, 4, big, 32, 1.0, None, None, None, None, 0, None) == -1
+    assert lib.oi_lmhead_logp_fwd(None, None, None, None, big, 64, 32, 1.0, None, None, None, None, 0, None) == -1
     assert lib.oi_gemm_bf16_tn(None, big, 4, None, 64, 4, 64, None, None, 4, 0, None) == -1
     assert lib.oi_gemm_bf16_tn(None, 72, 4, None, 72, 4, 72, None, None, 4, 0, None) == -1  # K % 64
     assert lib.oi_gemm_bf16_layouts(None, 72, 1, None, 72, 0, 4, 8, 64, None, None, 8, 0, None) == -1  # M % 8, A k-major
@@ -94,18 +94,11 @@ def test_rejected_arguments_return_codes_without_launching():
     assert lib.oi_lmhead_fwd_workspace_bytes(0, 64, 10, 0) == 0
     # one dZ chunk (bf16), the fp32 d_hidden accumulator, three queues of 8 words; no transposed copies
     plain = 256 * 256 * 2 + 256 * 64 * 4 + 256
-    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1, 0, 0) == plain
-    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 0, 0, 0) == plain
-    # a row selection adds the row index, the count, the gathered hidden rows / labels / lse / gradient
-    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1, 1, 0) == plain + 256 * 4 + 256 + 256 * 64 * 2 + 256 * 8 + 3 * 256 * 4
-    # a cache of exponentials adds the two per-token factors and the scaled hidden rows
-    # (every chunk cached: no dZ chunk, no fp32 accumulator)
-    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1, 0, 1) == 256 + 2 * 256 * 4 + 256 * 64 * 2
-    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 70000, 1, 0, 1) == 256 * 32768 * 2 + 256 * 64 * 4 + 512 + 2 * 256 * 4 + 256 * 64 * 2
-    # 2 bytes per cached logit, whole chunks of 32768 columns (or the padded vocabulary)
-    assert lib.oi_lmhead_cache_bytes(300, 1000, 1) == 512 * 1024 * 2
-    assert lib.oi_lmhead_cache_bytes(256, 70000, 1) == 256 * 32768 * 2 and lib.oi_lmhead_cache_bytes(256, 70000, 9) == 256 * 70144 * 2
-    assert lib.oi_lmhead_cache_bytes(256, 70000, 0) == 0
+    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1, 0) == plain
+    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 0, 0) == plain
+    # a row selection adds the row index, the count, the gathered hidden rows / labels / lse / gradient / logprob
+    selection = 256 * 4 + 256 + 256 * 64 * 2 + 256 * 8 + 3 * 256 * 4
+    assert lib.oi_lmhead_bwd_workspace_bytes(256, 64, 256, 1, 1) == plain + selection
     assert lib.oi_lmhead_fwd_workspace_bytes(256, 64, 256, 1) == lib.oi_lmhead_fwd_workspace_bytes(256, 64, 256, 0) + 256 * 4 + 256 + 256 * 64 * 2 + 256 * 8
     # the forward that also accumulates the weighted sum of weight rows: the plain forward's buffers (one split per
     # vocabulary tile at this size), one pair of queue sets per vocabulary chunk of 65536 columns and the chunk of
@@ -113,16 +106,24 @@ def test_rejected_arguments_return_codes_without_launching():
     assert lib.oi_lmhead_fwd_wsum_workspace_bytes(0, 64, 10, 0) == 0
     assert lib.oi_lmhead_fwd_wsum_workspace_bytes(256, 64, 256, 0) == 256 * 16 + 256 * 4 + 256 + 256 * 256 * 2
     assert lib.oi_lmhead_fwd_wsum_workspace_bytes(256, 64, 70000, 0) >= 256 * 65536 * 2
-    assert lib.oi_lmhead_dh_workspace_bytes(0) == 0 and lib.oi_lmhead_dh_workspace_bytes(300) == 512 * 4 + 256
-    assert lib.oi_lmhead_logp_fwd_wsum(None, None, None, None, 4, 100, 32, 1.0, None, None, None, None, None, 0, None) == -1
-    assert lib.oi_lmhead_logp_fwd_wsum(16, 32, 8, None, 4, 64, 32, 1.0, None, None, None, None, None, 0, None) == -2
-    assert lib.oi_lmhead_dh_from_wsum(None, None, None, None, None, None, None, 4, 100, 32, 1.0, None, None, 0, None) == -1
-    assert lib.oi_lmhead_dh_from_wsum(None, None, None, None, None, None, None, 4, 64, 32, 1.0, None, None, 0, None) == -2
-    assert lib.oi_lmhead_dh_from_wsum(None, None, None, None, None, None, None, 0, 64, 32, 1.0, None, None, 0, None) == 0
-    # the whole step in token slabs (cache_chunks < 0) sizes its own scratch: a slab of exponentials and an fp32 d_weight
-    slabs = lib.oi_lmhead_grpo_workspace_bytes(4, 4096, 64, 1000, -1)
+    # its backward: the mask's row index and count, and the recomputing backward (with a row selection) for flagged rows
+    assert lib.oi_lmhead_dh_workspace_bytes(0, 64, 256) == 0
+    assert lib.oi_lmhead_dh_workspace_bytes(256, 64, 256) == 256 * 4 + 256 + plain + selection
+    assert lib.oi_lmhead_logp_fwd_wsum(None, None, None, None, 4, 100, 32, 1.0, *([None] * 7), 0, None) == -1
+    assert lib.oi_lmhead_logp_fwd_wsum(16, 32, 8, None, 4, 64, 32, 1.0, *([None] * 7), 0, None) == -2
+    assert lib.oi_lmhead_dh_from_wsum(*([None] * 10), 4, 100, 32, 1.0, None, None, 0, None) == -1
+    assert lib.oi_lmhead_dh_from_wsum(*([None] * 10), 4, 64, 32, 1.0, None, None, 0, None) == -2
+    assert lib.oi_lmhead_dh_from_wsum(*([None] * 10), 0, 64, 32, 1.0, None, None, 0, None) == 0
+    # the whole step: recomputing (slab size 0: forward and backward regions side by side), or in slabs of tokens
+    # (a slab of exponentials or the recomputing backward for flagged rows, whichever is larger; with d_weight and
+    # more than one slab an fp32 d_weight)
+    whole = lib.oi_lmhead_grpo_workspace_bytes(4, 4096, 64, 1000, 1, 0)
+    assert whole >= lib.oi_lmhead_bwd_workspace_bytes(4 * 4096, 64, 1000, 1, 1)
+    slabs = lib.oi_lmhead_grpo_workspace_bytes(4, 4096, 64, 1000, 1, 4096)
     assert slabs >= 4096 * 1024 * 2 + 1000 * 64 * 4
-    assert lib.oi_lmhead_grpo_workspace_bytes(4, 4096, 64, 1000, -2) >= slabs + 4096 * 1024 * 2
+    assert lib.oi_lmhead_grpo_workspace_bytes(4, 4096, 64, 1000, 0, 4096) <= slabs - 1000 * 64 * 4
+    assert lib.oi_lmhead_grpo_workspace_bytes(4, 4096, 64, 1000, 1, 16384) < slabs + 12288 * 1024 * 2  # one slab: no fp32 d_weight
+    assert lib.oi_lmhead_grpo_fwd_bwd(*([8] * 8), 4, 4096, 64, 1000, 1.0, 0, 0.8, 1.2, 2, 0.05, 0, 0.0, 1.0, *([8] * 5), -1, 8, 0, None) == -1
 
 
 def test_cpu_tensors_are_refused_loudly():

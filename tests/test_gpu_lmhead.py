@@ -179,7 +179,7 @@ def test_d_hidden_in_forward_is_the_default_without_d_weight():
     with pytest.raises(ValueError):
         lm_head.fused_lm_head_logprobs(
             hidden.to(DEV).requires_grad_(True), weight.to(DEV), labels.to(DEV), dhidden_in_forward=True,
-            logit_cache_chunks=1,
+            compact_backward=True,
         )
 
 
@@ -365,119 +365,94 @@ def test_row_selection_with_compact_backward_and_mask():
     assert (dw.grad.float().cpu() - rw.grad).abs().max().item() <= TOL + rw.grad.abs().max().item() * 2**-7
 
 
-@pytest.mark.parametrize(
-    "n,h,v,chunks",
-    [
-        (300, 128, 1000, 1),  # one chunk, all of it cached; ragged tokens and vocabulary
-        (700, 256, 5000, 1),
-        (260, 64, 70000, 1),  # three chunks: the first from the cache, the others recomputed
-        (260, 64, 70000, 2),
-        (260, 64, 70000, 3),  # everything from the cache: no recomputation at all
-        (130, 128, 100000, 9),  # more chunks asked for than there are
-        (2, 64, 7, 1),
-    ],
-)
-@pytest.mark.parametrize("want_dw", [True, False])
-@pytest.mark.parametrize("masked", [False, True])
-def test_backward_from_cache_of_exponentials(n, h, v, chunks, want_dw, masked):
-    """The optional cache of 2^(logit) written by the forward replaces the recomputation of the cached
-    vocabulary chunks in the backward: same gradients as the oracle (and as the recomputing path, up to
-    bf16 rounding), forward results bit-identical with and without the cache."""
-    print(f"case N={n} H={h} V={v} cached chunks={chunks} dW={want_dw} masked={masked}", flush=True)
-    hidden, weight, labels = _case(n, h, v, seed=31, w_scale=3.0 / math.sqrt(h))
-    g = torch.Generator().manual_seed(32)
-    upstream = torch.randn(n, generator=g)
-    upstream[::5] = 0.0
-    mask = (torch.rand(n, generator=g) < 0.7) if masked else torch.ones(n, dtype=torch.bool)
-    labels[0], labels[n - 1] = v - 1, 0
-    rh = hidden.float().requires_grad_(True)
-    rw = weight.float().requires_grad_(True)
-    lp_o, _ = o_lm.lm_head_logprobs(rh, rw, labels, 0.9)
-    (lp_o * mask).backward(upstream)
+def _rows_of_any_logit_size(n, h, v, seed):
+    """Token rows whose logits cover what a float can hold: the largest logit / temperature of a row near
+    0, 60, 85, 100 and 300 nats (the kept exponentials of such rows would overflow bf16 were they not taken
+    relative to the label's own logit), rows whose logits are all near -120 nats, labels that are the row's
+    most likely token, ordinary labels, and labels more than 44 nats below the row's maximum (which the
+    kernels flag and recompute).  Returns ``(hidden, weight, labels, flagged)``; `flagged` marks the rows
+    whose label is that unlikely, computed here in fp64."""
+    g = torch.Generator().manual_seed(seed)
+    u = torch.nn.functional.normalize(torch.randn(h, generator=g), dim=0)
+    weight = (torch.randn(v, h, generator=g) / math.sqrt(h) + 2.0 * u).bfloat16()
+    hidden = torch.randn(n, h, generator=g)
+    hidden -= (hidden @ u)[:, None] * u  # no component along the common direction of the weight rows ...
+    z = hidden.double() @ weight.double().T
+    targets = torch.tensor([0.0, 60.0, 85.0, 100.0, 300.0, -120.0])
+    group = torch.arange(n) % len(targets)
+    top = z.max(dim=1).values
+    scale = torch.where(targets[group] > 0, targets[group] / top, torch.ones(n, dtype=torch.float64))
+    hidden = hidden * scale.float()[:, None]
+    hidden += torch.where(targets[group] < 0, targets[group] / 2.0, torch.zeros(n))[:, None] * u  # ... except here
+    hidden = hidden.bfloat16()
+    z = hidden.double() @ weight.double().T
+    labels = torch.randint(0, v, (n,), generator=g)
+    likely = (torch.arange(n) // len(targets)) % 3 == 0
+    labels[likely] = z.argmax(dim=1)[likely]
+    return hidden, weight, labels, z
 
-    def run(cache_chunks):
+
+@pytest.mark.parametrize("temperature", [1.0, 0.5])
+@pytest.mark.parametrize("masked", [False, True])
+def test_d_hidden_in_forward_for_logits_of_any_size(temperature, masked):
+    """The forward that prepares d_hidden keeps its exponentials relative to each token's own label logit:
+    logprob, entropy and d_hidden against the oracle for rows whose largest logit / temperature runs from 0
+    to 600 nats and for rows whose logits are all very negative; rows whose label is too unlikely for that
+    are flagged on the device (checked through the C-ABI below) and recomputed, with the same results."""
+    n, h, v = 600, 128, 3000
+    hidden, weight, labels, z = _rows_of_any_logit_size(n, h, v, seed=61)
+    g = torch.Generator().manual_seed(62)
+    mask = (torch.rand(n, generator=g) < 0.7) if masked else torch.ones(n, dtype=torch.bool)
+    upstream = torch.randn(n, generator=g)
+    rh = hidden.double().requires_grad_(True)
+    # the oracle in fp64: at logits of several hundred the fp32 form of the reference's entropy,
+    # lse - sum p z, cancels two numbers of that size and is itself off by more than the tolerance
+    lp_o, ent_o = o_lm.lm_head_logprobs(rh, weight.double(), labels, temperature, True, compute_dtype=torch.float64)
+    (lp_o * mask).backward(upstream.double())
+    zt = z / temperature
+    gap = zt.max(dim=1).values - zt.gather(1, labels[:, None])[:, 0]
+    assert zt.max().item() >= 299.0 and zt.max(dim=1).values.min().item() <= -90.0
+    assert (gap > 60.0).sum() >= 20 and (gap < 1e-9).sum() >= 50  # both kinds of label are there
+    grads = {}
+    for route in (True, False):
         dh = hidden.to(DEV).requires_grad_(True)
-        dw = weight.to(DEV).requires_grad_(want_dw)
         lp, ent = lm_head.fused_lm_head_logprobs(
-            dh, dw, labels.to(DEV), 0.9, mask=mask.to(DEV) if masked else None, return_entropy=True,
-            logit_cache_chunks=cache_chunks,
+            dh, weight.to(DEV), labels.to(DEV), temperature, mask=mask.to(DEV) if masked else None,
+            return_entropy=True, dhidden_in_forward=route,
         )  # fmt: skip
         lp.backward(upstream.to(DEV))
-        return lp.detach(), ent, dh.grad, (dw.grad if want_dw else None)
+        # logprobs of several hundred nats: fp32 results, so the bound is relative to their size
+        assert ((lp.detach().cpu().double() - lp_o.detach()) * mask).abs().max().item() <= TOL + 1e-6 * lp_o.abs().max().item()
+        assert ((ent.cpu().double() - ent_o.detach()) * mask).abs().max().item() <= TOL
+        got = dh.grad.double().cpu()
+        assert torch.isfinite(got).all() and (got[~mask] == 0).all()
+        # per row: 3 % of the row's own gradient; the absolute part covers rows whose label holds nearly all
+        # of the probability (a gradient of 1e-30 is met to the rounding of the fp32 logprob, not relatively)
+        err, size = (got - rh.grad).norm(dim=1), rh.grad.norm(dim=1)
+        worst = (err - 3e-2 * size)[mask].max().item()
+        assert worst <= 1e-4, (route, worst)
+        assert (err[mask & (size > 1e-2)] / size[mask & (size > 1e-2)]).max().item() <= 3e-2
+        grads[route] = got
+    assert not torch.equal(grads[True], grads[False])  # the two routes are different code
 
-    lp_c, ent_c, dh_c, dw_c = run(chunks)
-    lp_r, ent_r, dh_r, dw_r = run(0)
-    assert torch.equal(lp_c, lp_r) and torch.equal(ent_c, ent_r)
-    assert ((lp_c.cpu() - lp_o.detach()) * mask).abs().max().item() <= TOL
-    tol_h = TOL + rh.grad.abs().max().item() * 2**-7
-    assert (dh_c.float().cpu() - rh.grad).abs().max().item() <= tol_h
-    assert ((dh_c.float().cpu() - rh.grad).norm() / rh.grad.norm()).item() <= 2e-2
-    assert (dh_c.cpu()[~mask] == 0).all() and (dh_c.cpu()[::5] == 0).all()
-    assert (dh_c.float() - dh_r.float()).abs().max().item() <= 2**-6 * dh_r.float().abs().max().item()
-    if n >= 130:  # another order of roundings: the two routes are not the same code
-        assert not torch.equal(dh_c, dh_r)
-    if want_dw:
-        tol_w = TOL + rw.grad.abs().max().item() * 2**-7
-        assert (dw_c.float().cpu() - rw.grad).abs().max().item() <= tol_w
-        assert ((dw_c.float().cpu() - rw.grad).norm() / rw.grad.norm()).item() <= 2e-2
-
-
-def test_cache_of_exponentials_confident_tokens_and_no_grad():
-    """Tokens whose label carries almost all of the probability (1 - p around 1e-2): the label's entry
-    of the cache is rebuilt from the fp32 logprob, so the gradient stays accurate where the bf16 entry
-    (relative error 2^-9 of p, i.e. tens of percent of 1 - p) would have cancelled.  Under no_grad no
-    cache is made at all."""
-    torch.manual_seed(41)
-    n, h, v = 256, 64, 2000
-    hidden = torch.randn(n, h).bfloat16()
-    weight = (torch.randn(v, h) * 0.05).bfloat16()
-    labels = torch.randint(0, v, (n,))
-    labels[:64] = torch.arange(64)  # distinct rows of W for the confident tokens
-    weight[:64] = (hidden[:64].float() * 0.19).bfloat16()  # logit of the label ~ 0.19 |h|^2 ~ 12
-    rh = hidden.float().requires_grad_(True)
-    lp_o, _ = o_lm.lm_head_logprobs(rh, weight.float(), labels, 1.0)
-    assert lp_o[:64].median().item() > -0.05  # p(label) > 0.95 on most of these rows
-    up = torch.randn(n)
-    lp_o.backward(up)
-    dh = hidden.to(DEV).requires_grad_(True)
-    lp, _ = lm_head.fused_lm_head_logprobs(dh, weight.to(DEV), labels.to(DEV), logit_cache_chunks=1)
-    lp.backward(up.to(DEV))
-    assert (lp.detach().cpu() - lp_o.detach()).abs().max().item() <= TOL
-    rel_rows = (dh.grad.float().cpu() - rh.grad).norm(dim=1) / rh.grad.norm(dim=1).clamp(min=1e-12)
-    assert rel_rows.max().item() <= 3e-2, rel_rows.max().item()
-    with torch.no_grad():
-        lp2, _ = lm_head.fused_lm_head_logprobs(dh, weight.to(DEV), labels.to(DEV), logit_cache_chunks=1)
-    assert torch.equal(lp2, lp.detach())
-    with pytest.raises(ValueError, match="compact_backward"):
-        lm_head.fused_lm_head_logprobs(dh, weight.to(DEV), labels.to(DEV), compact_backward=True, logit_cache_chunks=1)
-
-
-def test_cache_chunks_auto_takes_what_fits(monkeypatch):
-    """``logit_cache_chunks="auto"``: as many chunks as fit into the allowed share of the free device
-    memory - all of them on an empty GPU (bitwise the same gradients as an explicit count), none when the
-    share is made tiny (bitwise the recomputing path)."""
-    n, h, v = 130, 64, 70000  # three vocabulary chunks
-    hidden, weight, labels = _case(n, h, v, seed=41, w_scale=3.0 / math.sqrt(h))
-    upstream = torch.randn(n, generator=torch.Generator().manual_seed(42))
-
-    def run(cache_chunks):
-        dh = hidden.to(DEV).requires_grad_(True)
-        dw = weight.to(DEV).requires_grad_(True)
-        lp, _ = lm_head.fused_lm_head_logprobs(dh, dw, labels.to(DEV), logit_cache_chunks=cache_chunks)
-        lp.backward(upstream.to(DEV))
-        return dh.grad, dw.grad
-
-    assert lm_head.resolve_cache_chunks("auto", n, v, torch.device(DEV)) == 3
-    assert lm_head.resolve_cache_chunks(2, n, v, torch.device(DEV)) == 2
-    auto, full, none = run("auto"), run(3), run(0)
-    assert torch.equal(auto[0], full[0]) and torch.equal(auto[1], full[1])
-    assert not torch.equal(auto[0], none[0])
-    monkeypatch.setattr(lm_head, "AUTO_CACHE_MEMORY_SHARE", 1e-9)
-    assert lm_head.resolve_cache_chunks("auto", n, v, torch.device(DEV)) == 0
-    tiny = run("auto")
-    assert torch.equal(tiny[0], none[0]) and torch.equal(tiny[1], none[1])
-    # a share that holds one chunk of this shape but not two
-    one_chunk = _lib.load().oi_lmhead_cache_bytes(n, v, 1)
-    free, _ = torch.cuda.mem_get_info(torch.device(DEV))
-    monkeypatch.setattr(lm_head, "AUTO_CACHE_MEMORY_SHARE", 1.5 * one_chunk / free)
-    assert lm_head.resolve_cache_chunks("auto", n, v, torch.device(DEV)) == 1
+    # the flags, read through the C-ABI: exactly the rows whose label is more than 64 binary orders down
+    lib = _lib.load()
+    hid, w, lab = hidden.to(DEV), weight.to(DEV), labels.to(DEV)
+    m = mask.to(DEV).view(torch.uint8) if masked else None
+    out = {k: torch.empty(n, dtype=torch.float32, device=DEV) for k in ("lp", "lse", "xref")}
+    wsum = torch.empty(n, h, dtype=torch.float32, device=DEV)
+    unsafe = torch.full((n,), 7, dtype=torch.uint8, device=DEV)
+    ws_bytes = lib.oi_lmhead_fwd_wsum_workspace_bytes(n, h, v, int(masked))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=DEV)
+    _lib.call(
+        "oi_lmhead_logp_fwd_wsum", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), _lib.ptr(m), n, h, v, 1.0 / temperature,
+        out["lp"].data_ptr(), None, out["lse"].data_ptr(), wsum.data_ptr(), out["xref"].data_ptr(), unsafe.data_ptr(),
+        ws.data_ptr(), ws_bytes, _lib.stream_of(hid),
+    )  # fmt: skip
+    torch.cuda.synchronize()
+    gap2 = gap * math.log2(math.e)
+    flagged = unsafe.cpu().bool()
+    assert set(unsafe.cpu().unique().tolist()) <= {0, 1}
+    clear = (gap2 - 64.0).abs() > 0.5  # away from the threshold the flag is determined
+    assert torch.equal(flagged[clear & mask], (gap2 > 64.0)[clear & mask]) and not flagged[~mask].any()
+    assert flagged.sum() >= 20
