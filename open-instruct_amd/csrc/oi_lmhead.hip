@@ -949,6 +949,8 @@ struct DynRows {
     // optional factors of row r of the product, applied as (acc * scale_a[r]) * scale_b[r] before it
     // is stored or accumulated (two factors so that neither has to leave the fp32 range)
     const float *scale_a, *scale_b;
+    // optional: the store mode comes from device memory (a negative value: the launch does nothing)
+    const int32_t* mode_dev;
 };
 
 // `queue` null: one workgroup per tile id (blockIdx); otherwise a launch of resident workgroups
@@ -958,6 +960,10 @@ __global__ void __launch_bounds__(NTHREADS)
     gemm_store_kernel(Operand A, int64_t M, Operand B, int64_t N, int64_t K, int mode, float* out_f32,
                       uint16_t* out_bf16, int64_t ldo, int64_t m_valid, DynRows dyn, uint32_t* __restrict__ queue) {
     __shared__ __align__(16) uint16_t lds[LDS_ELEMS];
+    if (dyn.mode_dev) {
+        mode = *dyn.mode_dev;
+        if (mode < 0) return;
+    }
     if (dyn.n_dev) {
         const int64_t n = *dyn.n_dev;
         if (dyn.role == 1) {
@@ -1095,6 +1101,10 @@ __global__ void __launch_bounds__(256)
 // on the device.  Written by a planning kernel, read by every kernel of the pass.
 struct SlabMeta {
     int32_t offset, count;
+    // how the slab's d_weight product is stored (the modes of gemm_store_tile): the only slab writes
+    // bf16 rows (2); of several, the first stores fp32 (0), the middle ones add to it (1) and the last
+    // one adds the fp32 sum to its own product and writes bf16 rows (3); a pass without rows: -1
+    int32_t dw_mode, reserved;
 };
 
 // Workgroup j copies row order[meta->offset + j] into the slab's own buffers: the hidden-state row
@@ -1445,7 +1455,7 @@ void enqueue_fwd_wsum(const FwdPlan& p, char* ws, const RowInputs& in, const uin
                            in.hidden, in.labels, n_tokens, in.n_dev, hidden_dim, vocab, c, fl, p.n_pad, partial, zy, q);
         const Operand a = {chunk_buf, cols, 0, p.n_pad, cols};
         const Operand b = {Wp + v_begin * hidden_dim, hidden_dim, 0, hidden_dim, valid};
-        const DynRows dyn = {in.n_dev, 1, nullptr, nullptr, nullptr};
+        const DynRows dyn = {in.n_dev, 1, nullptr, nullptr, nullptr, nullptr};
         hipLaunchKernelGGL((gemm_store_kernel<false, true>), dim3(resident_grid(p.n_pad / BM, h_tiles)), dim3(NTHREADS), 0,
                            s, a, p.n_pad, b, hidden_dim, round_up(valid, BK), ci == 0 ? 0 : 1, wsum,
                            static_cast<uint16_t*>(nullptr), hidden_dim, n_tokens, dyn, q + FWD_QUEUE_WORDS);
@@ -1500,9 +1510,17 @@ __global__ void __launch_bounds__(256)
 // first call's product (0) and adds the following ones (1; a call without tokens adds nothing and
 // costs nothing); the caller rounds dw32 to bf16 when the last call is through.  4: the product is
 // added to bf16 rows that an earlier call wrote.
+// max_grid > 0 caps the number of resident workgroups of every launch (the queues work with any
+// number): the launches that serve flagged rows normally find none, and a launch over a few CUs that
+// finds nothing costs a fraction of one over all of them.
+constexpr unsigned REPAIR_GRID = 32;
 void enqueue_bwd(const BwdPlan& p, char* ws, const RowInputs& in, const void* weight, int64_t n_tokens,
                  int64_t hidden_dim, int64_t vocab, float inv_temperature, void* d_hidden, void* d_weight,
-                 hipStream_t s, int dw_mode = 2, float* dw32 = nullptr) {
+                 hipStream_t s, int dw_mode = 2, float* dw32 = nullptr, unsigned max_grid = 0) {
+    auto grid_of = [&](int64_t tiles_m, int64_t tiles_n) {
+        const unsigned g = resident_grid(tiles_m, tiles_n);
+        return dim3(max_grid > 0 && g > max_grid ? max_grid : g);
+    };
     uint16_t* dz = reinterpret_cast<uint16_t*>(ws + p.off_dz);
     float* dh32 = reinterpret_cast<float*>(ws + p.off_dh32);
     uint32_t* queues = reinterpret_cast<uint32_t*>(ws + p.off_queues);
@@ -1515,7 +1533,7 @@ void enqueue_bwd(const BwdPlan& p, char* ws, const RowInputs& in, const void* we
         const int64_t cols = v_end - v_begin;                                   // multiple of 256
         const int64_t valid = vocab - v_begin < cols ? vocab - v_begin : cols;  // real rows of W
         uint32_t* q = queues + ci * 3 * QUEUE_WORDS;
-        hipLaunchKernelGGL(lmhead_dz_kernel, dim3(resident_grid(cols / BM, p.n_pad / BN)), dim3(NTHREADS), 0, s, Wp,
+        hipLaunchKernelGGL(lmhead_dz_kernel, grid_of(cols / BM, p.n_pad / BN), dim3(NTHREADS), 0, s, Wp,
                            in.hidden, in.labels, in.lse, in.grad, in.logprob, n_tokens, in.n_dev, hidden_dim, vocab, c,
                            inv_temperature, v_begin, cols, p.n_pad, dz, q);
         const bool first = ci == 0, last = ci == p.n_chunks - 1;
@@ -1523,16 +1541,16 @@ void enqueue_bwd(const BwdPlan& p, char* ws, const RowInputs& in, const void* we
         {
             const Operand a = {dz, cols, 0, p.n_pad, cols};
             const Operand b = {Wp + v_begin * hidden_dim, hidden_dim, 0, hidden_dim, valid};
-            const DynRows dyn = {in.n_dev, 1, in.rows, nullptr, nullptr};
-            hipLaunchKernelGGL((gemm_store_kernel<false, true>), dim3(resident_grid(p.n_pad / BM, h_tiles)),
+            const DynRows dyn = {in.n_dev, 1, in.rows, nullptr, nullptr, nullptr};
+            hipLaunchKernelGGL((gemm_store_kernel<false, true>), grid_of(p.n_pad / BM, h_tiles),
                                dim3(NTHREADS), 0, s, a, p.n_pad, b, hidden_dim, round_up(valid, BK), mode, dh32,
                                static_cast<uint16_t*>(d_hidden), hidden_dim, n_tokens, dyn, q + QUEUE_WORDS);
         }
         if (d_weight) {
             const Operand a = {dz, cols, 0, cols, p.n_pad};
             const Operand b = {in.hidden, hidden_dim, 0, hidden_dim, n_tokens};
-            const DynRows dyn = {in.n_dev, 2, nullptr, nullptr, nullptr};
-            hipLaunchKernelGGL((gemm_store_kernel<true, true>), dim3(resident_grid(cols / BM, h_tiles)),
+            const DynRows dyn = {in.n_dev, 2, nullptr, nullptr, nullptr, nullptr};
+            hipLaunchKernelGGL((gemm_store_kernel<true, true>), grid_of(cols / BM, h_tiles),
                                dim3(NTHREADS), 0, s, a, cols, b, hidden_dim, round_up(n_tokens, BK), dw_mode,
                                dw32 ? dw32 + v_begin * hidden_dim : static_cast<float*>(nullptr),
                                static_cast<uint16_t*>(d_weight) + v_begin * hidden_dim, hidden_dim, valid, dyn,
@@ -1543,19 +1561,21 @@ void enqueue_bwd(const BwdPlan& p, char* ws, const RowInputs& in, const void* we
 
 // Both backward products of a slab from its kept exponentials (see slab_prepare_kernel): the whole
 // vocabulary as one chunk, d_hidden rows stored once through the slab's row numbers, d_weight
-// stored / accumulated as dw_mode says (see enqueue_bwd).  `queues`: 2 * QUEUE_WORDS zeroed words.
+// stored / accumulated as *dw_mode_dev says (the slab's place among the slabs of the call is known
+// on the device only: the first one stores, the last one rounds to bf16, see SlabMeta).
+// `queues`: 2 * QUEUE_WORDS zeroed words.
 void enqueue_products_from_exponentials(const uint16_t* ecache, int64_t cache_ld, int64_t slab_pad,
                                         const int32_t* count, const int32_t* rows_s, const float* scale_a,
                                         const float* scale_b, const uint16_t* scaled_hidden, const void* weight,
                                         int64_t hidden_dim, int64_t vocab, void* d_hidden, void* d_weight,
-                                        int dw_mode, float* dw32, uint32_t* queues, hipStream_t s) {
+                                        const int32_t* dw_mode_dev, float* dw32, uint32_t* queues, hipStream_t s) {
     const uint16_t* Wp = static_cast<const uint16_t*>(weight);
     const int64_t h_tiles = (hidden_dim + BN - 1) / BN;
     {
         const ProbeScope probe(1, s);
         const Operand a = {ecache, cache_ld, 0, slab_pad, cache_ld};
         const Operand b = {Wp, hidden_dim, 0, hidden_dim, vocab};
-        const DynRows dyn = {count, 1, rows_s, scale_a, scale_b};
+        const DynRows dyn = {count, 1, rows_s, scale_a, scale_b, nullptr};
         hipLaunchKernelGGL((gemm_store_kernel<false, true>), dim3(resident_grid(slab_pad / BM, h_tiles)),
                            dim3(NTHREADS), 0, s, a, slab_pad, b, hidden_dim, round_up(vocab, BK), 2,
                            static_cast<float*>(nullptr), static_cast<uint16_t*>(d_hidden), hidden_dim, slab_pad, dyn,
@@ -1565,9 +1585,9 @@ void enqueue_products_from_exponentials(const uint16_t* ecache, int64_t cache_ld
         const ProbeScope probe(2, s);
         const Operand a = {ecache, cache_ld, 0, cache_ld, slab_pad};
         const Operand b = {scaled_hidden, hidden_dim, 0, hidden_dim, slab_pad};
-        const DynRows dyn = {count, 2, nullptr, nullptr, nullptr};
+        const DynRows dyn = {count, 2, nullptr, nullptr, nullptr, dw_mode_dev};
         hipLaunchKernelGGL((gemm_store_kernel<true, true>), dim3(resident_grid(cache_ld / BM, h_tiles)),
-                           dim3(NTHREADS), 0, s, a, cache_ld, b, hidden_dim, round_up(slab_pad, BK), dw_mode, dw32,
+                           dim3(NTHREADS), 0, s, a, cache_ld, b, hidden_dim, round_up(slab_pad, BK), 2, dw32,
                            static_cast<uint16_t*>(d_weight), hidden_dim, vocab, dyn, queues + QUEUE_WORDS);
     }
 }
@@ -1669,15 +1689,9 @@ __global__ void plan_equal_slabs_kernel(const int32_t* __restrict__ count, int c
     const int left = n - i * size;
     meta[i].offset = i * size;
     meta[i].count = left < 0 ? 0 : (left > size ? size : left);
-}
-
-// out[8 i .. 8 i + 8) = bf16(in[8 i .. 8 i + 8))
-__global__ void __launch_bounds__(256) f32_to_bf16_kernel(const float* __restrict__ in, int64_t n8, uint16_t* __restrict__ out) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n8) return;
-    const float4 a = reinterpret_cast<const float4*>(in)[2 * i], b = reinterpret_cast<const float4*>(in)[2 * i + 1];
-    reinterpret_cast<oi_u32x4*>(out)[i] =
-        oi_u32x4{oi_pack_bf16x2(a.x, a.y), oi_pack_bf16x2(a.z, a.w), oi_pack_bf16x2(b.x, b.y), oi_pack_bf16x2(b.z, b.w)};
+    const bool first = i == 0, last = i == k - 1;
+    meta[i].dw_mode = i >= k ? -1 : (last ? (first ? 2 : 3) : (first ? 0 : 1));
+    meta[i].reserved = 0;
 }
 
 // the per-token outputs of rows that take no part are zero
@@ -1755,9 +1769,8 @@ int run_slab_passes(const SlabPlan& p, char* ws, const SlabStep& st, hipStream_t
         hipLaunchKernelGGL(slab_prepare_kernel, dim3((unsigned)p.cap), dim3(256), 0, s, lse, grad, st.logprob, unsafe,
                            rows_s, labels_s, xref_s, meta + i, st.inv_temperature, vocab, hdim, keep_buf, p.v_pad,
                            hidden_s, scale_a, scale_b, scaled_hidden);
-        const int dw_mode = p.n_passes == 1 ? 2 : (i == 0 ? 0 : 1);
         enqueue_products_from_exponentials(keep_buf, p.v_pad, p.cap, cnt, rows_s, scale_a, scale_b, scaled_hidden,
-                                           st.weight, hdim, vocab, st.d_hidden, st.d_weight, dw_mode, dw32,
+                                           st.weight, hdim, vocab, st.d_hidden, st.d_weight, &meta[i].dw_mode, dw32,
                                            queues + FWD_QUEUE_WORDS, s);
     }
     // the flagged rows, if any: one recomputing backward over them (its workspace takes the place of
@@ -1773,13 +1786,8 @@ int run_slab_passes(const SlabPlan& p, char* ws, const SlabStep& st, hipStream_t
             hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_words + 255) / 256)), dim3(256), 0, s, rq, n_words);
         const RowInputs in = launch_selection(p.repair.sel, ws_rep, st.hidden, st.labels, lse, grad, unsafe, false, n,
                                               hdim, rq, select_clears ? n_words : 0, s, st.logprob);
-        enqueue_bwd(p.repair, ws_rep, in, st.weight, n, hdim, vocab, st.inv_temperature, st.d_hidden, st.d_weight, s,
-                    dw32 ? 1 : 4, dw32);
-    }
-    if (dw32) {
-        const int64_t n8 = vocab * hdim / 8;  // hidden_dim is a multiple of 64
-        hipLaunchKernelGGL(f32_to_bf16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, s, dw32, n8,
-                           static_cast<uint16_t*>(st.d_weight));
+        enqueue_bwd(p.repair, ws_rep, in, st.weight, n, hdim, vocab, st.inv_temperature, st.d_hidden, st.d_weight, s, 4,
+                    nullptr, REPAIR_GRID);
     }
     return oi_launch_status();
 }
@@ -1915,7 +1923,8 @@ extern "C" int oi_lmhead_dh_from_wsum(const void* hidden, const void* weight, co
         hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n_words + 255) / 256)), dim3(256), 0, s, rq, n_words);
     const RowInputs in = launch_selection(p.repair.sel, ws_rep, hidden, labels, lse, grad_logprob, unsafe, false,
                                           n_tokens, hidden_dim, rq, select_clears ? n_words : 0, s, logprob);
-    enqueue_bwd(p.repair, ws_rep, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, nullptr, s);
+    enqueue_bwd(p.repair, ws_rep, in, weight, n_tokens, hidden_dim, vocab, inv_temperature, d_hidden, nullptr, s, 2, nullptr,
+                REPAIR_GRID);
     return oi_launch_status();
 }
 
@@ -2133,7 +2142,7 @@ extern "C" int oi_gemm_bf16_tn(const void* A, int64_t lda, int64_t M, const void
     const Operand b = {static_cast<const uint16_t*>(B), ldb, 0, N, K};
     hipLaunchKernelGGL((gemm_store_kernel<false, false>), dim3(grid_for_tiles((M + BM - 1) / BM, (N + BN - 1) / BN)),
                        dim3(NTHREADS), 0, static_cast<hipStream_t>(stream), a, M, b, N, K, mode, out_f32,
-                       static_cast<uint16_t*>(out_bf16), ldo, M, DynRows{nullptr, 0, nullptr, nullptr, nullptr}, static_cast<uint32_t*>(nullptr));
+                       static_cast<uint16_t*>(out_bf16), ldo, M, DynRows{nullptr, 0, nullptr, nullptr, nullptr, nullptr}, static_cast<uint32_t*>(nullptr));
     return oi_launch_status();
 }
 
@@ -2157,7 +2166,7 @@ extern "C" int oi_gemm_bf16_layouts(const void* A, int64_t lda, int a_k_major, c
     hipStream_t s = static_cast<hipStream_t>(stream);
     uint16_t* o16 = static_cast<uint16_t*>(out_bf16);
     uint32_t* no_queue = nullptr;
-    const DynRows fixed = {nullptr, 0, nullptr, nullptr, nullptr};
+    const DynRows fixed = {nullptr, 0, nullptr, nullptr, nullptr, nullptr};
     if (a_k_major && b_k_major)
         hipLaunchKernelGGL((gemm_store_kernel<true, true>), grid, dim3(NTHREADS), 0, s, a, M, b, N, K, mode, out_f32, o16,
                            ldo, M, fixed, no_queue);
