@@ -465,6 +465,48 @@ int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, const int64_t
                            size_t workspace_bytes, void* stream);
 
 /*
+ * The whole DPO step on hidden states in one call, with nothing recomputed and with a d_weight: the
+ * fused lm_head forward (per-token logps), the per-sequence sums, the sigmoid preference loss per pair
+ * and the backward to d_hidden / d_weight.  It replaces, for a model that hands its final hidden
+ * states to the head, the sequence open_instruct/olmo_core_train_modules.py:71-76 (DPOLMHead: w_out,
+ * calculate_per_token_logps) -> open_instruct/padding_free_collator.py:202-229 or
+ * open_instruct/dpo_utils.py:689-712 (per-sequence logps) -> open_instruct/dpo_utils.py:523-563 /
+ * :617-642 (dpo_loss / simpo_loss) -> losses.mean().backward()
+ * (open_instruct/olmo_core_train_modules.py:190-207); no single reference function computes it.
+ *
+ * hidden: bf16 [n, hidden_dim]; labels: the batch's own (unshifted) int64 labels; position t is scored
+ * against labels[t + 1] when that is not -100.  cu_seq_lens NULL: n_seqs padded rows of `total`
+ * positions (n = n_seqs * total); otherwise one packed row of `total` positions with boundaries
+ * cu_seq_lens int32 [n_seqs + 1] (n = total), segments as for oi_seq_logp_fwd.  The first n_seqs / 2
+ * sequences are the chosen answers, the others the rejected ones, pair i = (i, n_seqs / 2 + i)
+ * (open_instruct/dpo_utils.py:876-877).  ref_chosen / ref_rejected (fp32 [n_seqs / 2], both or
+ * neither), beta, label_smoothing, margin as for oi_dpo_sigmoid_fwd; average_log_prob != 0 divides
+ * every sequence sum by its count (dpo_norm, simpo).  grad_scale is d (caller's scalar) / d losses[i],
+ * e.g. 1 / (n_seqs / 2) for losses.mean().
+ * Outputs: per_token_logps fp32 [n] (0 where nothing is scored), seq_logps fp32 [n_seqs], losses and
+ * (optional) rewards fp32 [n_seqs / 2], d_hidden bf16 [n, hidden_dim] (zero rows where nothing is
+ * scored), d_weight bf16 [vocab, hidden_dim] (NULL skips it).
+ *
+ * The step runs like the slab-wise oi_lmhead_grpo_fwd_bwd, with the slabs (at most slab_tokens
+ * scored rows, > 0) filled with whole pairs: a token's upstream gradient depends on the sums of both
+ * sequences of its pair, so a pair's rows are gathered next to each other (the row index is built on
+ * the device in pair order) and a slab ends where the next pair would not fit.  A pair with more
+ * scored rows than a slab holds is cut across slabs and its tokens take the recomputing backward
+ * after the last slab, like flagged tokens; pass a slab_tokens of at least the largest pair to avoid
+ * that.  6 N H V of matrix work; the workspace holds [slab, vocab] bf16 and, with d_weight, an fp32
+ * [vocab, hidden_dim].
+ */
+size_t oi_lmhead_dpo_workspace_bytes(int64_t n_seqs, int64_t total, int packed, int64_t hidden_dim, int64_t vocab,
+                                     int want_d_weight, int64_t slab_tokens);
+int oi_lmhead_dpo_fwd_bwd(const void* hidden, const void* weight, const int64_t* labels, const int32_t* cu_seq_lens,
+                          int64_t n_seqs, int64_t total, int64_t hidden_dim, int64_t vocab, float inv_temperature,
+                          const float* ref_chosen, const float* ref_rejected, float beta, float label_smoothing,
+                          float margin, int average_log_prob, float grad_scale, float* per_token_logps,
+                          float* seq_logps, float* losses, float* chosen_rewards, float* rejected_rewards,
+                          void* d_hidden, void* d_weight, int64_t slab_tokens, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
+/*
  * Timing probe of the slab-wise entry points (no reference counterpart; it exists for the
  * measurement harness, which has to time one kernel inside a call that launches several).  Between
  * oi_lmhead_probe_arm(kernel) and oi_lmhead_probe_read the slab-wise calls of this process record a

@@ -72,6 +72,11 @@ SIGNATURES: dict[str, tuple] = {
         _I,
         [_P] * 8 + [_I64, _I64, _I64, _I64, _F, _I, _F, _F, _I, _F, _I, _F, _F] + [_P] * 5 + [_I64, _P, _SZ, _P],
     ),
+    "oi_lmhead_dpo_workspace_bytes": (_SZ, [_I64, _I64, _I, _I64, _I64, _I, _I64]),
+    "oi_lmhead_dpo_fwd_bwd": (
+        _I,
+        [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _F, _P, _P, _F, _F, _F, _I, _F] + [_P] * 7 + [_I64, _P, _SZ, _P],
+    ),
     "oi_lmhead_probe_arm": (_I, [_I]),
     "oi_lmhead_probe_read": (_I, [_P, _I, _P]),
     "oi_gemm_bf16_tn": (_I, [_P, _I64, _I64, _P, _I64, _I64, _I64, _P, _P, _I64, _I, _P]),

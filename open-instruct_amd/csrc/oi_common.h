@@ -100,3 +100,25 @@ __device__ __forceinline__ float oi_block_sum(float v, float* scratch) {
     for (int w = 0; w < nw; ++w) t += scratch[w];
     return t;
 }
+
+// ---- per-sequence ranges of a batch of token positions ---------------------------------------------
+// cu != null: one packed row of `total` positions with sequence boundaries cu[0 .. n_seqs]
+// (open_instruct/padding_free_collator.py:202-229); cu == null: n_seqs padded rows of `total`
+// positions each (open_instruct/dpo_utils.py:689-712).
+// Segment [start, end) of scored positions for sequence s; position t is scored against labels[t+1].
+__device__ __forceinline__ void oi_seq_range(const int32_t* cu, int64_t s, int64_t n_seqs, int64_t total, int64_t* start,
+                                          int64_t* end) {
+    if (cu) {
+        // boundaries shifted left by one, leading 0 kept, everything past the last start stays in the
+        // last segment; the packed row has total-1 scored positions
+        int64_t a = s == 0 ? 0 : (int64_t)cu[s] - 1;
+        int64_t b = s == n_seqs - 1 ? total - 1 : (int64_t)cu[s + 1] - 1;
+        a = a < 0 ? 0 : (a > total - 1 ? total - 1 : a);
+        b = b < a ? a : (b > total - 1 ? total - 1 : b);
+        *start = a;
+        *end = b;
+    } else {
+        *start = s * total;
+        *end = s * total + total - 1;
+    }
+}

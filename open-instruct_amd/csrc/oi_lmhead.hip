@@ -2095,6 +2095,241 @@ extern "C" int oi_lmhead_grpo_fwd_bwd(const void* hidden, const void* weight, co
     return oi_launch_status();
 }
 
+// ---------------------------------------------------------------------------------------------
+// The whole DPO step on hidden states, in slabs of whole chosen / rejected pairs
+// ---------------------------------------------------------------------------------------------
+namespace {
+// Workgroup s handles sequence s: every position t of its range gets the label it is scored against
+// (labels[t + 1]) and a mask byte (that label is not -100); the number of scored positions goes to
+// cnt[s].  The positions that belong to no range (the last one of a padded row, of the packed row)
+// are masked out.
+__global__ void __launch_bounds__(256)
+    dpo_rows_kernel(const int64_t* __restrict__ labels, const int32_t* __restrict__ cu, int64_t n_seqs, int64_t total,
+                    int64_t* __restrict__ labels_eff, uint8_t* __restrict__ mask, int32_t* __restrict__ cnt) {
+    const int64_t s = blockIdx.x;
+    int64_t a, b;
+    oi_seq_range(cu, s, n_seqs, total, &a, &b);
+    float c = 0.f;
+    for (int64_t t = a + threadIdx.x; t < b; t += blockDim.x) {
+        const int64_t y = labels[t + 1];
+        labels_eff[t] = y;
+        const bool keep = y != -100;
+        mask[t] = keep ? 1 : 0;
+        c += keep ? 1.f : 0.f;
+    }
+    __shared__ float scratch[16];
+    c = oi_block_sum(c, scratch);  // exact: at most 2^22 positions per sequence
+    if (threadIdx.x == 0) {
+        cnt[s] = (int32_t)c;
+        const int64_t last = cu ? (s == n_seqs - 1 ? total - 1 : -1) : s * total + total - 1;
+        if (last >= 0) {
+            labels_eff[last] = -100;
+            mask[last] = 0;
+        }
+    }
+}
+
+// One thread.  The scored rows are taken pair by pair (pair p = sequences p and n_seqs / 2 + p, the
+// chosen and the rejected answer to one prompt: open_instruct/dpo_utils.py:734-763, 876-877): off[s]
+// is where sequence s starts in the row index, and the slabs are filled with whole pairs in that order
+// (a pair that does not fit the current slab starts the next one), because the upstream gradient of a
+// token depends on the logprob sums of both sequences of its pair and must be known when the slab's
+// exponentials are multiplied.  A pair with more rows than a slab holds is cut across slabs and its
+// sequences are marked (seq_unsafe): their tokens take the recomputing backward after the last slab.
+// Two consecutive slabs always hold more than `cap` rows together, so 2 ceil(rows / cap) + 1 passes
+// are enough.
+__global__ void dpo_plan_kernel(const int32_t* __restrict__ cnt, int n_seqs, int cap, int n_passes,
+                                int32_t* __restrict__ off, uint8_t* __restrict__ seq_unsafe, int32_t* __restrict__ count,
+                                SlabMeta* __restrict__ meta) {
+    if (blockIdx.x != 0 || threadIdx.x != 0) return;
+    const int bs = n_seqs / 2;
+    int run = 0;
+    for (int p = 0; p < bs; ++p) {
+        off[p] = run;
+        run += cnt[p];
+        off[bs + p] = run;
+        run += cnt[bs + p];
+    }
+    *count = run;
+    int i = 0, start = 0, fill = 0;
+    auto close = [&]() {
+        if (i < n_passes) {
+            meta[i].offset = start;
+            meta[i].count = fill;
+        }
+        ++i;
+        start += fill;
+        fill = 0;
+    };
+    for (int p = 0; p < bs; ++p) {
+        int rows = cnt[p] + cnt[bs + p];
+        const bool oversize = rows > cap;
+        seq_unsafe[p] = seq_unsafe[bs + p] = oversize ? 1 : 0;
+        if (oversize) {
+            while (rows > 0) {
+                const int take = rows < cap - fill ? rows : cap - fill;
+                fill += take;
+                rows -= take;
+                if (fill == cap) close();
+            }
+        } else {
+            if (fill + rows > cap) close();
+            fill += rows;
+        }
+    }
+    if (fill > 0) close();
+    const int k = i < n_passes ? i : n_passes;  // slabs with rows (at least the one that stores zeros)
+    for (int j = k; j < n_passes; ++j) {
+        meta[j].offset = start;
+        meta[j].count = 0;
+    }
+    const int kk = k > 0 ? k : 1;
+    for (int j = 0; j < n_passes; ++j) {
+        const bool first = j == 0, last = j == kk - 1;
+        meta[j].dw_mode = j >= kk ? -1 : (last ? (first ? 2 : 3) : (first ? 0 : 1));
+        meta[j].reserved = 0;
+    }
+}
+
+// Workgroup s writes the scored positions of sequence s, in ascending order, to
+// order[off[s] .. off[s] + cnt[s]) and marks them in `unsafe` when the sequence is marked.
+__global__ void __launch_bounds__(256)
+    dpo_order_kernel(const uint8_t* __restrict__ mask, const int32_t* __restrict__ cu, int64_t n_seqs, int64_t total,
+                     const int32_t* __restrict__ off, const uint8_t* __restrict__ seq_unsafe,
+                     int32_t* __restrict__ order, uint8_t* __restrict__ unsafe) {
+    const int64_t s = blockIdx.x;
+    int64_t a, b;
+    oi_seq_range(cu, s, n_seqs, total, &a, &b);
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int64_t per = (b - a + 255) / 256;
+    const int64_t lo = a + t * per, hi = lo + per < b ? lo + per : b;
+    int c = 0;
+    for (int64_t i = lo; i < hi; ++i) c += mask[i] ? 1 : 0;
+    int incl = c;
+#pragma unroll
+    for (int o = 1; o < OI_WAVE; o <<= 1) {
+        const int up = __shfl_up(incl, o, OI_WAVE);
+        if (lane >= o) incl += up;
+    }
+    __shared__ int wave_total[4];
+    if (lane == OI_WAVE - 1) wave_total[wave] = incl;
+    __syncthreads();
+    int base = 0;
+    for (int w = 0; w < wave; ++w) base += wave_total[w];
+    int pos = off[s] + base + incl - c;
+    const bool flag = seq_unsafe[s] != 0;
+    for (int64_t i = lo; i < hi; ++i)
+        if (mask[i]) {
+            order[pos++] = (int32_t)i;
+            if (flag) unsafe[i] = 1;
+        }
+}
+
+__global__ void fill_f32_kernel(float* __restrict__ p, int64_t n, float v) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+struct DpoPlan {
+    SlabPlan slabs;
+    int64_t n, bs;
+    size_t off_slabs, off_labels_eff, off_mask, off_cnt, off_off, off_seq_unsafe, off_counts, off_dseq, off_gl, total;
+};
+DpoPlan plan_dpo(int64_t n_seqs, int64_t total, bool packed, int64_t hdim, int64_t vocab, bool want_dw,
+                 int64_t slab_tokens) {
+    DpoPlan p;
+    p.n = packed ? total : n_seqs * total;
+    p.bs = n_seqs / 2;
+    const int64_t n_pad = round_up(p.n, 256);
+    const int64_t cap = round_up(slab_tokens < SLAB_UNIT ? SLAB_UNIT : slab_tokens, SLAB_UNIT);
+    const int64_t cap_eff = n_pad < cap ? n_pad : cap;
+    p.slabs = plan_slabs(p.n, 1, 1, hdim, vocab, want_dw, slab_tokens, 2 * ((n_pad + cap_eff - 1) / cap_eff) + 1);
+    Carver cv;
+    p.off_slabs = cv.take(p.slabs.total);
+    p.off_labels_eff = cv.take((size_t)p.n * sizeof(int64_t));
+    p.off_mask = cv.take((size_t)p.n);
+    p.off_cnt = cv.take((size_t)n_seqs * sizeof(int32_t));
+    p.off_off = cv.take((size_t)n_seqs * sizeof(int32_t));
+    p.off_seq_unsafe = cv.take((size_t)n_seqs);
+    p.off_counts = cv.take((size_t)n_seqs * sizeof(float));
+    p.off_dseq = cv.take((size_t)n_seqs * sizeof(float));
+    p.off_gl = cv.take((size_t)p.bs * sizeof(float));
+    p.total = cv.off;
+    return p;
+}
+}  // namespace
+
+extern "C" size_t oi_lmhead_dpo_workspace_bytes(int64_t n_seqs, int64_t total, int packed, int64_t hidden_dim,
+                                                int64_t vocab, int want_d_weight, int64_t slab_tokens) {
+    if (n_seqs <= 0 || total <= 0 || hidden_dim <= 0 || vocab <= 0 || slab_tokens <= 0) return 0;
+    return plan_dpo(n_seqs, total, packed != 0, hidden_dim, vocab, want_d_weight != 0, slab_tokens).total;
+}
+
+extern "C" int oi_lmhead_dpo_fwd_bwd(const void* hidden, const void* weight, const int64_t* labels,
+                                     const int32_t* cu_seq_lens, int64_t n_seqs, int64_t total, int64_t hidden_dim,
+                                     int64_t vocab, float inv_temperature, const float* ref_chosen,
+                                     const float* ref_rejected, float beta, float label_smoothing, float margin,
+                                     int average_log_prob, float grad_scale, float* per_token_logps, float* seq_logps,
+                                     float* losses, float* chosen_rewards, float* rejected_rewards, void* d_hidden,
+                                     void* d_weight, int64_t slab_tokens, void* workspace, size_t workspace_bytes,
+                                     void* stream) {
+    OI_RETURN_IF(n_seqs < 2 || n_seqs % 2 != 0 || total < 1 || slab_tokens <= 0, OI_EINVAL);
+    OI_RETURN_IF(n_seqs > MAX_LD || total > MAX_LD, OI_EINVAL);
+    const bool packed = cu_seq_lens != nullptr;
+    const int64_t n_tokens = packed ? total : n_seqs * total;
+    int rc = check_lmhead(hidden, weight, labels, n_tokens, hidden_dim, vocab, inv_temperature);
+    if (rc != OI_OK) return rc;
+    OI_RETURN_IF((ref_chosen == nullptr) != (ref_rejected == nullptr), OI_EINVAL);
+    OI_RETURN_IF(!per_token_logps || !seq_logps || !losses || !d_hidden || !workspace, OI_ENULL);
+    OI_RETURN_IF(!oi_aligned(workspace, 256) || !oi_aligned(d_hidden, 4) || !oi_aligned(d_weight, 4), OI_EALIGN);
+    const DpoPlan p = plan_dpo(n_seqs, total, packed, hidden_dim, vocab, d_weight != nullptr, slab_tokens);
+    OI_RETURN_IF(workspace_bytes < p.total, OI_EWORKSPACE);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    char* ws = static_cast<char*>(workspace);
+    char* ws_slabs = ws + p.off_slabs;
+    int64_t* labels_eff = reinterpret_cast<int64_t*>(ws + p.off_labels_eff);
+    uint8_t* mask = reinterpret_cast<uint8_t*>(ws + p.off_mask);
+    int32_t* cnt = reinterpret_cast<int32_t*>(ws + p.off_cnt);
+    int32_t* off = reinterpret_cast<int32_t*>(ws + p.off_off);
+    uint8_t* seq_unsafe = reinterpret_cast<uint8_t*>(ws + p.off_seq_unsafe);
+    float* counts = reinterpret_cast<float*>(ws + p.off_counts);
+    float* d_seq = reinterpret_cast<float*>(ws + p.off_dseq);
+    float* grad_losses = reinterpret_cast<float*>(ws + p.off_gl);
+    float* grad = reinterpret_cast<float*>(ws_slabs + p.slabs.off_grad);
+    uint8_t* unsafe = reinterpret_cast<uint8_t*>(ws_slabs + p.slabs.off_unsafe);
+    const int64_t bs = p.bs;
+
+    hipLaunchKernelGGL(dpo_rows_kernel, dim3((unsigned)n_seqs), dim3(256), 0, s, labels, cu_seq_lens, n_seqs, total,
+                       labels_eff, mask, cnt);
+    hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)((bs + 63) / 64)), dim3(64), 0, s, grad_losses, bs, grad_scale);
+    const SlabStep st = {hidden, weight, labels_eff, mask, n_tokens, hidden_dim, vocab, inv_temperature, per_token_logps,
+                         nullptr, d_hidden, d_weight};
+    // per-sequence sums of the logprobs computed so far, the loss derivative of every pair, and from it
+    // every token's d loss / d logprob (right for the pairs whose tokens are all there)
+    auto upstream = [&](bool) {
+        int r = oi_seq_logp_fwd(per_token_logps, labels, cu_seq_lens, n_seqs, total, average_log_prob, seq_logps, counts,
+                                stream);
+        if (r != OI_OK) return r;
+        r = oi_dpo_sigmoid_bwd(seq_logps, seq_logps + bs, ref_chosen, ref_rejected, nullptr, grad_losses, bs, beta,
+                               label_smoothing, margin, d_seq, d_seq + bs, stream);
+        if (r != OI_OK) return r;
+        return oi_seq_logp_bwd(d_seq, labels, cu_seq_lens, counts, n_seqs, total, average_log_prob, grad, stream);
+    };
+    rc = run_slab_passes(
+        p.slabs, ws_slabs, st, s,
+        [&](int32_t* order, int32_t* count, SlabMeta* meta) {
+            hipLaunchKernelGGL(dpo_plan_kernel, dim3(1), dim3(1), 0, s, cnt, (int)n_seqs, (int)p.slabs.cap,
+                               (int)p.slabs.n_passes, off, seq_unsafe, count, meta);
+            hipLaunchKernelGGL(dpo_order_kernel, dim3((unsigned)n_seqs), dim3(256), 0, s, mask, cu_seq_lens, n_seqs, total,
+                               off, seq_unsafe, order, unsafe);
+        },
+        upstream);
+    if (rc != OI_OK) return rc;
+    // the sums are those of the last upstream pass (every logprob was there); losses and rewards from them
+    return oi_dpo_sigmoid_fwd(seq_logps, seq_logps + bs, ref_chosen, ref_rejected, nullptr, bs, beta, label_smoothing,
+                              margin, losses, chosen_rewards, rejected_rewards, stream);
+}
+
 extern "C" int oi_lmhead_probe_arm(int kernel) {
     OI_RETURN_IF(kernel < 0 || kernel > 2 || g_probe.kernel >= 0, OI_EINVAL);
     for (int i = 0; i < 2 * Probe::MAX_LAUNCHES; ++i) {

@@ -300,31 +300,13 @@ __global__ void masked_bwd_kernel(const float* __restrict__ grad_out, const void
 }
 
 // ---- per-sequence logprob sums ------------------------------------------------------------------
-// Segment [start, end) of scored positions for sequence s; position t is scored against labels[t+1].
-__device__ __forceinline__ void seq_range(const int32_t* cu, int64_t s, int64_t n_seqs, int64_t total, int64_t* start,
-                                          int64_t* end) {
-    if (cu) {
-        // boundaries shifted left by one, leading 0 kept, everything past the last start stays in the
-        // last segment; the packed row has total-1 scored positions
-        int64_t a = s == 0 ? 0 : (int64_t)cu[s] - 1;
-        int64_t b = s == n_seqs - 1 ? total - 1 : (int64_t)cu[s + 1] - 1;
-        a = a < 0 ? 0 : (a > total - 1 ? total - 1 : a);
-        b = b < a ? a : (b > total - 1 ? total - 1 : b);
-        *start = a;
-        *end = b;
-    } else {
-        *start = s * total;
-        *end = s * total + total - 1;
-    }
-}
-
 __global__ void __launch_bounds__(256)
     seq_logp_fwd_kernel(const float* __restrict__ lp, const int64_t* __restrict__ labels,
                         const int32_t* __restrict__ cu, int64_t n_seqs, int64_t total, int average,
                         float* __restrict__ out, float* __restrict__ counts) {
     const int64_t s = blockIdx.x;
     int64_t a, b;
-    seq_range(cu, s, n_seqs, total, &a, &b);
+    oi_seq_range(cu, s, n_seqs, total, &a, &b);
     float sum = 0.f, cnt = 0.f;
     for (int64_t t = a + threadIdx.x; t < b; t += blockDim.x) {
         const float keep = labels[t + 1] != -100 ? 1.f : 0.f;
@@ -346,7 +328,7 @@ __global__ void __launch_bounds__(256)
                         int64_t total, int average, float* __restrict__ d_lp) {
     const int64_t s = blockIdx.x;
     int64_t a, b;
-    seq_range(cu, s, n_seqs, total, &a, &b);
+    oi_seq_range(cu, s, n_seqs, total, &a, &b);
     const float g = average ? grad_out[s] / fmaxf(counts[s], 1.f) : grad_out[s];
     for (int64_t t = a + threadIdx.x; t < b; t += blockDim.x) d_lp[t] = labels[t + 1] != -100 ? g : 0.f;
     // the unscored last position of a padded row, or of the packed row

@@ -10,6 +10,7 @@ Names and signatures follow open_instruct/dpo_utils.py in the reference (``dpo_l
 from __future__ import annotations
 
 import contextlib
+import dataclasses
 import pathlib
 from collections.abc import Callable, Iterable
 
@@ -312,6 +313,201 @@ def concatenated_forward_olmo(
         output = model(input_ids, labels=labels)
     chosen, rejected = _split_pairs(_sequence_logps(output.loss, labels, concat, packing, average_log_prob), bs)
     return chosen, rejected, None
+
+
+@dataclasses.dataclass
+class FusedDPOResult:
+    """What :func:`dpo_loss_on_hidden` returns.  ``loss`` (``losses.mean()``) carries the graph: its
+    ``backward()`` hands the gradients computed inside the call to ``hidden`` and ``weight``; every
+    other field is detached."""
+
+    loss: torch.Tensor
+    losses: torch.Tensor
+    chosen_logps: torch.Tensor
+    rejected_logps: torch.Tensor
+    chosen_rewards: torch.Tensor
+    rejected_rewards: torch.Tensor
+    per_token_logps: torch.Tensor
+
+
+# slab size of the no-recompute DPO step when the caller names none (scored tokens per slab); a slab holds
+# whole chosen / rejected pairs, so it should not be smaller than the largest pair of the batch
+DEFAULT_DPO_SLAB_TOKENS = 8192
+
+
+def dpo_loss_on_hidden(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    reference_chosen_logps: torch.Tensor | None,
+    reference_rejected_logps: torch.Tensor | None,
+    beta: float,
+    *,
+    cu_seq_lens: torch.Tensor | None = None,
+    average_log_prob: bool = False,
+    reference_free: bool = False,
+    label_smoothing: float = 0.0,
+    gamma_beta_ratio: float = 0.0,
+    token_slabs: bool | int = True,
+) -> FusedDPOResult:
+    """Sigmoid preference loss straight from the final hidden states of a concatenated chosen + rejected
+    batch, with both gradients and nothing recomputed.
+
+    One call for the reference's sequence "``DPOLMHead`` (``w_out``, ``calculate_per_token_logps``:
+    open_instruct/olmo_core_train_modules.py:71-76) -> per-sequence logps
+    (open_instruct/padding_free_collator.py:202-229 / open_instruct/dpo_utils.py:689-712) -> ``dpo_loss`` /
+    ``simpo_loss`` (open_instruct/dpo_utils.py:523-563, :617-642) -> ``losses.mean().backward()``
+    (open_instruct/olmo_core_train_modules.py:190-207)".  Because the loss is known inside the call, a
+    slab of token rows can be finished (forward, upstream gradient, ``d_hidden``, its share of ``d_weight``)
+    before the next one starts, so a trainable lm_head costs 6·N·H·V of matrix work instead of the 8·N·H·V of
+    the differentiable route through :class:`~open_instruct_amd.olmo_core_train_modules.DPOLMHead`, whose
+    backward has to recompute the logits.  The ``[tokens, vocab]`` logits never exist; the scratch is a
+    ``[slab, vocab]`` bf16 buffer and an fp32 ``[vocab, hidden]``.
+
+    ``hidden`` is ``[2 * bs, T, H]`` bf16 with ``labels`` ``[2 * bs, T]`` (padded; chosen rows first:
+    open_instruct/dpo_utils.py:734-763), or ``[1, T_total, H]`` with ``labels`` ``[1, T_total]`` and
+    ``cu_seq_lens`` int32 ``[2 * bs + 1]`` (packed: open_instruct/padding_free_collator.py:166-199).  The
+    labels are the batch's own, unshifted; position ``t`` is scored against ``labels[t + 1]`` where that
+    is not -100, other positions are not multiplied.  ``average_log_prob`` as in ``dpo_norm`` / ``simpo``;
+    ``reference_free`` drops the reference term from the loss (the rewards keep it, as in the reference);
+    ``gamma_beta_ratio`` is simpo's margin (pass no reference logps for simpo).
+
+    ``token_slabs``: ``True`` = slabs of ``DEFAULT_DPO_SLAB_TOKENS`` scored tokens, or a number.  A slab
+    is filled with whole pairs (a token's upstream gradient needs the logprob sums of both sequences of
+    its pair); a pair that is larger than a slab still gives the right result but its tokens go through a
+    recomputing backward, so pass at least the largest pair's scored tokens.  ``result.loss.backward()``
+    may be called once.
+    """
+    from . import grpo_utils
+
+    if hidden.ndim != 3 or labels.ndim != 2 or tuple(hidden.shape[:2]) != tuple(labels.shape):
+        raise ValueError(f"hidden {tuple(hidden.shape)} and labels {tuple(labels.shape)} must be [B, T, H] and [B, T]")
+    packed = cu_seq_lens is not None
+    if packed and labels.shape[0] != 1:
+        raise ValueError("a packed batch is one row: hidden [1, T, H], labels [1, T]")
+    n_seqs = int(cu_seq_lens.numel()) - 1 if packed else int(labels.shape[0])
+    if n_seqs < 2 or n_seqs % 2:
+        raise ValueError(f"{n_seqs} sequences: a concatenated batch holds the chosen and the rejected half")
+    if (reference_chosen_logps is None) != (reference_rejected_logps is None):
+        raise ValueError("pass both reference logps or neither")
+    bs, total = n_seqs // 2, int(labels.shape[1])
+    dev = _lib.require_gpu(hidden, weight, labels, cu_seq_lens, reference_chosen_logps, reference_rejected_logps)
+    if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise ValueError("the fused lm_head expects bf16 hidden states and weight")
+    h, v = int(hidden.shape[-1]), int(weight.shape[0])
+    if weight.ndim != 2 or weight.shape[1] != h or h % 64:
+        raise ValueError(f"weight {tuple(weight.shape)} does not fit hidden size {h} (a multiple of 64)")
+    ref_c = None if reference_chosen_logps is None else _lib.f32c(reference_chosen_logps.detach()).reshape(-1)
+    ref_r = None if reference_rejected_logps is None else _lib.f32c(reference_rejected_logps.detach()).reshape(-1)
+    if ref_c is not None and (ref_c.numel() != bs or ref_r.numel() != bs):
+        raise ValueError(f"reference logps must hold {bs} entries each")
+    loss_ref_c, loss_ref_r = (None, None) if reference_free else (ref_c, ref_r)
+    slab_tokens = DEFAULT_DPO_SLAB_TOKENS if token_slabs is True else int(token_slabs)
+    if slab_tokens < 256:
+        raise ValueError("token_slabs must be True or a number of tokens (at least 256)")
+    n = labels.numel()
+    hid = hidden.detach().reshape(n, h).contiguous()
+    w = weight.detach().contiguous()
+    lab = labels.to(torch.int64).contiguous()
+    cu = None if not packed else cu_seq_lens.to(torch.int32).contiguous()
+    per_token = torch.empty(labels.shape, dtype=torch.float32, device=dev)
+    seq_logps = torch.empty(n_seqs, dtype=torch.float32, device=dev)
+    out = torch.empty((3, bs), dtype=torch.float32, device=dev)
+    wants_grad = torch.is_grad_enabled() and (hidden.requires_grad or weight.requires_grad)
+    if not wants_grad:
+        shifted = padding_free_collator.shift_labels(lab)
+        with torch.no_grad():
+            lp, _ = lm_head.fused_lm_head_logprobs(hidden, weight, shifted, mask=shifted != -100)
+            logps = _sequence_logps(lp, lab, {"concatenated_cu_seq_lens_k": cu}, packed, average_log_prob)
+            losses, _, _ = _SigmoidPairLoss.apply(
+                logps[:bs], logps[bs:], loss_ref_c, loss_ref_r, None, float(beta), float(label_smoothing),
+                float(gamma_beta_ratio),
+            )  # fmt: skip
+            _, cr, rj = _SigmoidPairLoss.apply(logps[:bs], logps[bs:], ref_c, ref_r, None, float(beta), 0.0, 0.0)
+        return FusedDPOResult(losses.mean(), losses, logps[:bs], logps[bs:], cr, rj, lp)
+    d_hidden = torch.empty_like(hid)
+    d_weight = torch.empty_like(w) if weight.requires_grad else None
+    lib = _lib.load()
+    ws_bytes = lib.oi_lmhead_dpo_workspace_bytes(n_seqs, total, int(packed), h, v, int(d_weight is not None), slab_tokens)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    _lib.call(
+        "oi_lmhead_dpo_fwd_bwd", hid.data_ptr(), w.data_ptr(), lab.data_ptr(), _lib.ptr(cu), n_seqs, total, h, v, 1.0,
+        _lib.ptr(loss_ref_c), _lib.ptr(loss_ref_r), float(beta), float(label_smoothing), float(gamma_beta_ratio),
+        int(bool(average_log_prob)), 1.0 / bs, per_token.data_ptr(), seq_logps.data_ptr(), out[0].data_ptr(),
+        out[1].data_ptr(), out[2].data_ptr(), d_hidden.data_ptr(), _lib.ptr(d_weight), slab_tokens, ws.data_ptr(),
+        ws_bytes, _lib.stream_of(hid),
+    )  # fmt: skip
+    losses, cr, rj = out.unbind(0)
+    if reference_free and ref_c is not None:  # the rewards keep the reference term
+        cr, rj = float(beta) * (seq_logps[:bs] - ref_c), float(beta) * (seq_logps[bs:] - ref_r)
+    loss = grpo_utils._AttachHeadGrads.apply(losses.mean(), hidden, weight, d_hidden.reshape(hidden.shape), d_weight)
+    return FusedDPOResult(loss, losses, seq_logps[:bs], seq_logps[bs:], cr, rj, per_token)
+
+
+def fused_loss_olmo(
+    model,
+    batch: dict,
+    args,
+    reference_cache=None,
+    average_log_prob: bool | None = None,
+    packing: bool = False,
+    token_slabs: bool | int = True,
+) -> FusedDPOResult:
+    """``concatenated_forward_olmo`` -> ``compute_loss`` -> ``losses.mean()`` (the body of
+    open_instruct/olmo_core_train_modules.py:190-207) with the lm_head, the per-sequence sums and the
+    pair loss in one no-recompute call.
+
+    The model must follow the olmo-core interface with a
+    :class:`~open_instruct_amd.olmo_core_train_modules.DPOLMHead` as ``model.lm_head``: the labels go into
+    the model, the head receives the final hidden states and, because a loss specification is set on it for
+    the duration of this call, computes the loss and both gradients right there (see
+    :func:`dpo_loss_on_hidden`).  ``args`` is duck-typed like the reference's (``loss_type``, ``beta``,
+    ``label_smoothing``, ``gamma_beta_ratio``); ``loss_type`` ``dpo``, ``dpo_norm`` and ``simpo`` are
+    served, ``wpo`` (whose weight needs the finished sequence means inside the gradient) is not.
+    ``result.loss.backward()`` continues into the trunk through the hidden states.
+    """
+    loss_type = str(getattr(args.loss_type, "value", args.loss_type))
+    if loss_type not in ("dpo", "dpo_norm", "simpo"):
+        raise ValueError(f"loss type {loss_type!r} has no fused form; use concatenated_forward_olmo and compute_loss")
+    if average_log_prob is None:
+        average_log_prob = loss_type in ("dpo_norm", "simpo")
+    if packing:
+        concat, _ = padding_free_collator.concatenated_inputs(batch)
+    else:
+        concat = concatenated_inputs(batch)
+    labels = concat["concatenated_labels"]
+    input_ids = concat["concatenated_input_ids"]
+    ref_c = ref_r = None
+    if loss_type != "simpo":
+        assert reference_cache is not None
+        ref = reference_cache[batch["index"]]
+        ref_c, ref_r = ref["chosen_logps"], ref["rejected_logps"]
+    head = model.lm_head
+    head.fused_loss = dict(
+        reference_chosen_logps=ref_c, reference_rejected_logps=ref_r, beta=args.beta,
+        cu_seq_lens=concat["concatenated_cu_seq_lens_k"] if packing else None, average_log_prob=average_log_prob,
+        label_smoothing=getattr(args, "label_smoothing", 0.0),
+        gamma_beta_ratio=getattr(args, "gamma_beta_ratio", 0.0) if loss_type == "simpo" else 0.0,
+        token_slabs=token_slabs,
+    )  # fmt: skip
+    try:
+        if packing:
+            doc_lens, max_doc_lens = olmo_core_utils.doc_lens_from_cu_seq_lens(
+                concat["concatenated_cu_seq_lens_k"], seq_len=input_ids.shape[-1]
+            )
+            model(
+                input_ids, labels=labels, position_ids=concat.get("concatenated_position_ids"), doc_lens=doc_lens,
+                max_doc_lens=max_doc_lens,
+            )  # fmt: skip
+        else:
+            model(input_ids, labels=labels)
+        result = head.fused_result
+    finally:
+        head.fused_loss = None
+        head.fused_result = None
+    if result is None:
+        raise RuntimeError("the model's lm_head did not run the fused loss (is it a DPOLMHead?)")
+    return result
 
 
 def build_reference_logprobs_cache(

@@ -42,6 +42,11 @@ class DPOLMHead(torch.nn.Module):
     """
 
     score_ignored_positions = False
+    # Set for the duration of one model call by open_instruct_amd.dpo_utils.fused_loss_olmo: the keyword
+    # arguments of dpo_loss_on_hidden.  The head then computes the preference loss and both gradients in the
+    # same call as the logps (nothing recomputed) and leaves the result in `fused_result`.
+    fused_loss: dict | None = None
+    fused_result = None
 
     def __init__(self, d_model: int, vocab_size: int, bias: bool = False, norm: torch.nn.Module | None = None,
                  dtype: torch.dtype = torch.bfloat16, device=None):  # fmt: skip
@@ -68,6 +73,14 @@ class DPOLMHead(torch.nn.Module):
         if labels is None:
             # no labels: the parent class returns plain logits (library GEMM; not the fused path)
             return self.w_out(h)
+        if self.fused_loss is not None:
+            from . import dpo_utils
+
+            if ignore_index != -100:
+                raise ValueError("the fused preference loss scores against -100 as the ignored label")
+            self.fused_result = dpo_utils.dpo_loss_on_hidden(h, self.w_out.weight, labels, **self.fused_loss)
+            logps = self.fused_result.per_token_logps
+            return LMOutputWithLoss(logits=None, loss=logps, ce_loss=logps.clone(), z_loss=None)
         shifted = padding_free_collator.shift_labels(labels)
         keep = None if self.score_ignored_positions else shifted != ignore_index
         per_token_logps, _ = lm_head.fused_lm_head_logprobs(h, self.w_out.weight, shifted, mask=keep)

@@ -138,6 +138,182 @@ def test_dpo_chain_matches_oracle(packed):
     assert ((dh.grad.float().cpu() - rh.grad).norm() / rh.grad.norm()).item() <= 2e-2
 
 
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("loss_type,slabs,want_dw,w_scale", [
+    ("dpo", True, True, 2.0),  # every pair in one slab
+    ("dpo_norm", 1024, True, 2.0),  # slabs of whole pairs (two or three pairs each), d_weight accumulates over them
+    ("simpo", 512, False, 2.0),  # one pair per slab; no reference model, a margin, averages
+    ("dpo", 256, True, 2.0),  # every pair is larger than a slab: cut across slabs, recomputing backward
+    ("dpo", 1024, True, 40.0),  # logits of +-100: most labels too unlikely for kept exponentials, flagged and recomputed
+    ("dpo_reference_free", True, True, 2.0),
+])  # fmt: skip
+def test_dpo_loss_on_hidden_whole_step(packed, loss_type, slabs, want_dw, w_scale):
+    """One C call for DPOLMHead -> per-sequence logps -> preference loss -> losses.mean().backward()
+    (open_instruct/olmo_core_train_modules.py:71-76, :190-207, open_instruct/padding_free_collator.py:202-229,
+    open_instruct/dpo_utils.py:523-563, :617-642, :689-712) with a trainable head and nothing recomputed,
+    against the oracle chain: padded and packed batches, sums and averages, pair-aligned slabs."""
+    torch.manual_seed(16)
+    h, v, pairs = 128, 3000, 5
+    n_seqs = 2 * pairs
+    beta, ls = 0.1, 0.05
+    if packed:
+        lens = torch.randint(40, 260, (n_seqs,)).tolist()
+        cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+        total = int(cu[-1])
+        labels = torch.randint(0, v, (1, total))
+        for i in range(n_seqs):
+            labels[0, cu[i] : cu[i] + min(lens[i] - 1, 5 + 3 * i)] = -100  # prompts
+        hidden = torch.randn(1, total, h).bfloat16()
+    else:
+        cu, total = None, 220
+        labels = torch.randint(0, v, (n_seqs, total))
+        for i in range(n_seqs):
+            labels[i, : 5 + 3 * i] = -100  # prompts
+            labels[i, total - 7 * i :] = -100 if i else labels[i, total:]  # padding tails of different lengths
+        hidden = torch.randn(n_seqs, total, h).bfloat16()
+    weight = (torch.randn(v, h) * w_scale / math.sqrt(h)).bfloat16()
+    ref_c, ref_r = -torch.rand(pairs) * 300, -torch.rand(pairs) * 300
+    average = loss_type in ("dpo_norm", "simpo")
+
+    rh = hidden.double().requires_grad_(True)
+    rw = weight.double().requires_grad_(True)
+    z = o_lm.lm_head_logits(rh, rw, torch.float64)
+    lp_o = o_logprob.calculate_per_token_logps(z, labels)
+    seq_o = o_red.get_batch_logps_packed(lp_o, labels, cu, average) if packed else o_red.get_batch_logps_padded(lp_o, labels, average)
+    if loss_type == "simpo":
+        losses_o, cr_o, rr_o = o_dpo.simpo_loss(seq_o[:pairs], seq_o[pairs:], beta, 0.3, ls)
+    else:
+        losses_o, cr_o, rr_o = o_dpo.dpo_loss(
+            seq_o[:pairs], seq_o[pairs:], ref_c.double(), ref_r.double(), beta, loss_type == "dpo_reference_free", ls
+        )
+    losses_o.mean().backward()
+
+    d = lambda x: None if x is None else x.to(DEV)  # noqa: E731
+    dh = d(hidden).requires_grad_(True)
+    dw = d(weight).requires_grad_(want_dw)
+    res = dpo_utils.dpo_loss_on_hidden(
+        dh, dw, d(labels), None if loss_type == "simpo" else d(ref_c), None if loss_type == "simpo" else d(ref_r), beta,
+        cu_seq_lens=d(cu), average_log_prob=average, reference_free=loss_type == "dpo_reference_free",
+        label_smoothing=ls, gamma_beta_ratio=0.3 if loss_type == "simpo" else 0.0, token_slabs=slabs,
+    )  # fmt: skip
+    (2.0 * res.loss).backward()  # an upstream gradient other than 1 is applied on the device
+    keep = o_logprob.shift_labels(labels) != -100
+    size = lp_o.detach().abs().max().item()
+    assert ((res.per_token_logps.cpu().double() - lp_o.detach()) * keep).abs().max().item() <= TOL + 1e-6 * size
+    assert (res.per_token_logps.cpu()[~keep] == 0).all()
+    n_kept = keep.sum().item() / n_seqs
+    got_seq = torch.cat([res.chosen_logps, res.rejected_logps]).cpu().double()
+    seq_tol = TOL * (1.0 if average else 2.0 * n_kept) + 1e-6 * seq_o.detach().abs().max().item()
+    assert (got_seq - seq_o.detach()).abs().max().item() <= seq_tol
+    assert (res.losses.cpu().double() - losses_o.detach()).abs().max().item() <= beta * 2 * seq_tol + 1e-5
+    assert abs(res.loss.item() - losses_o.detach().mean().item()) <= beta * 2 * seq_tol + 1e-5
+    assert (res.chosen_rewards.cpu().double() - cr_o).abs().max().item() <= beta * seq_tol + 1e-4
+    assert (res.rejected_rewards.cpu().double() - rr_o).abs().max().item() <= beta * seq_tol + 1e-4
+    got = dh.grad.double().cpu()
+    exp_dh, exp_dw = 2.0 * rh.grad, 2.0 * rw.grad
+    assert torch.isfinite(got).all() and (got[~keep] == 0).all()
+    assert ((got - exp_dh).norm() / exp_dh.norm()).item() <= 2e-2
+    err, norm = (got - exp_dh).flatten(0, 1).norm(dim=1), exp_dh.flatten(0, 1).norm(dim=1)
+    assert (err - 3e-2 * norm).max().item() <= 1e-4 * norm.max().item()
+    if want_dw:
+        gw = dw.grad.double().cpu()
+        assert torch.isfinite(gw).all()
+        assert ((gw - exp_dw).norm() / exp_dw.norm()).item() <= 2e-2
+    else:
+        assert dw.grad is None
+    # the differentiable route through the head's per-token logps gives the same numbers
+    dh2 = d(hidden).requires_grad_(True)
+    shifted = padding_free_collator.shift_labels(d(labels))
+    lp2, _ = lm_head.fused_lm_head_logprobs(dh2, d(weight), shifted, mask=shifted != -100)
+    assert (lp2.detach() - res.per_token_logps).abs().max().item() <= 1e-5 + 1e-6 * size
+    # no gradient wanted: forward only, same values
+    with torch.no_grad():
+        res0 = dpo_utils.dpo_loss_on_hidden(
+            dh, dw, d(labels), None if loss_type == "simpo" else d(ref_c), None if loss_type == "simpo" else d(ref_r),
+            beta, cu_seq_lens=d(cu), average_log_prob=average, reference_free=loss_type == "dpo_reference_free",
+            label_smoothing=ls, gamma_beta_ratio=0.3 if loss_type == "simpo" else 0.0,
+        )  # fmt: skip
+    assert not res0.loss.requires_grad and abs(res0.loss.item() - res.loss.item()) <= 1e-5 + 1e-6 * abs(res.loss.item())
+
+
+class _OlmoStyleModel(torch.nn.Module):
+    """Stand-in with the olmo-core interface: the labels go into the model, ``lm_head`` is a DPOLMHead."""
+
+    def __init__(self, vocab, hidden):
+        super().__init__()
+        from open_instruct_amd.olmo_core_train_modules import DPOLMHead
+
+        self.embed = torch.nn.Embedding(vocab, hidden, dtype=torch.bfloat16)
+        self.mix = torch.nn.Linear(hidden, hidden, bias=False, dtype=torch.bfloat16)
+        self.lm_head = DPOLMHead(hidden, vocab)
+
+    def forward(self, input_ids, labels=None, position_ids=None, doc_lens=None, max_doc_lens=None):
+        x = self.embed(input_ids)
+        x = x + torch.tanh(self.mix(x))
+        return self.lm_head(x, labels=labels)
+
+
+@pytest.mark.parametrize("packing", [False, True])
+@pytest.mark.parametrize("loss_type", ["dpo_norm", "simpo"])
+def test_fused_loss_olmo_matches_the_reference_sequence(packing, loss_type):
+    """fused_loss_olmo against concatenated_forward_olmo -> compute_loss -> losses.mean().backward()
+    (open_instruct/olmo_core_train_modules.py:190-207) of this package on the same model: loss, logps and
+    the gradient of every parameter (trunk and head)."""
+    import types
+
+    from open_instruct_amd import model_utils as mu
+
+    torch.manual_seed(26)
+    vocab, hid, bs = 400, 64, 3
+    model = _OlmoStyleModel(vocab, hid).to(DEV)
+    args = types.SimpleNamespace(loss_type=loss_type, beta=5.0, label_smoothing=0.0, gamma_beta_ratio=0.3)
+    cache = mu.TensorCache(tensors={"chosen_logps": -torch.rand(8, device=DEV) * 3, "rejected_logps": -torch.rand(8, device=DEV) * 3})
+    if packing:
+        def side(lens):
+            ids = torch.randint(1, vocab, (1, sum(lens)), device=DEV)
+            cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=DEV)
+            lab = ids.clone()
+            for i in range(len(lens)):
+                lab[0, cu[i] : cu[i] + 4] = -100
+            return ids, lab, cu
+        c_ids, c_lab, c_cu = side([20, 33, 17])
+        r_ids, r_lab, r_cu = side([25, 19, 30])
+        batch = {
+            "chosen_input_ids": c_ids, "chosen_labels": c_lab, "chosen_cu_seq_lens_k": c_cu, "chosen_cu_seq_lens_q": c_cu,
+            "chosen_max_length_q": 33, "chosen_max_length_k": 33,
+            "rejected_input_ids": r_ids, "rejected_labels": r_lab, "rejected_cu_seq_lens_k": r_cu,
+            "rejected_cu_seq_lens_q": r_cu, "rejected_max_length_q": 30, "rejected_max_length_k": 30,
+            "index": torch.tensor([5, 1, 6], device=DEV),
+        }  # fmt: skip
+    else:
+        batch = {
+            "chosen_input_ids": torch.randint(1, vocab, (bs, 30), device=DEV),
+            "rejected_input_ids": torch.randint(1, vocab, (bs, 24), device=DEV),
+            "index": torch.tensor([5, 1, 6], device=DEV),
+        }
+        batch["chosen_labels"] = batch["chosen_input_ids"].clone()
+        batch["rejected_labels"] = batch["rejected_input_ids"].clone()
+        batch["chosen_labels"][:, :6] = -100
+        batch["rejected_labels"][:, :4] = -100
+    average = loss_type in ("dpo_norm", "simpo")
+    c0, r0, _ = dpo_utils.concatenated_forward_olmo(model, batch, average_log_prob=average, packing=packing)
+    losses0, cr0, rr0 = dpo_utils.compute_loss(args, batch, c0, r0, cache)
+    losses0.mean().backward()
+    g0 = [p.grad.float().clone() for p in model.parameters()]
+    model.zero_grad()
+    res = dpo_utils.fused_loss_olmo(model, batch, args, cache, packing=packing)
+    res.loss.backward()
+    g1 = [p.grad.float().clone() for p in model.parameters()]
+    assert model.lm_head.fused_loss is None and model.lm_head.fused_result is None
+    assert (res.chosen_logps - c0.detach()).abs().max().item() <= 1e-4 and (res.rejected_logps - r0.detach()).abs().max().item() <= 1e-4
+    assert (res.losses - losses0.detach()).abs().max().item() <= 1e-3
+    assert (res.chosen_rewards - cr0).abs().max().item() <= 1e-3 and (res.rejected_rewards - rr0).abs().max().item() <= 1e-3
+    for x, y in zip(g0, g1):
+        assert (x - y).abs().max().item() <= 2e-2 * max(1e-4, x.abs().max().item()), (x - y).abs().max().item()
+    with pytest.raises(ValueError):
+        dpo_utils.fused_loss_olmo(model, batch, types.SimpleNamespace(loss_type="wpo", beta=0.1), cache, packing=packing)
+
+
 @pytest.mark.parametrize("m,n,k", [(256, 256, 64), (300, 515, 192), (1, 70, 128), (1030, 257, 4096)])
 def test_gemm_bf16_tn_entry_point(m, n, k):
     """out[m, n] = sum_k A[m, k] * B[n, k] through the raw C-ABI, bf16 and fp32 outputs, accumulate."""
