@@ -16,6 +16,9 @@ synthetic inputs that already live in HBM.  Workloads are the BASELINE configs:
   c4: packed batch at OLMo-2-7B shape (16 sequences, cu_seqlens, V=100352), per-sequence sums + GRPO loss
       (c4-recompute: through the three differentiable calls).
   c5: DPO at Llama-3.1-70B head shape: hidden [32768, 8192], W [128256, 8192], bwd to dHidden only.
+      c5-train-head: the same batch with a trainable head (what the reference's DPO trains), loss and
+      both gradients from one no-recompute call (dpo_loss_on_hidden); c5-train-head-recompute: the same
+      through the differentiable calls.
 
 `roofline` describes the dominant kernel of the workload, timed with HIP events on the stream it
 runs on inside the timed region; `cpu_baseline` is the oracle's restatement of the reference's
@@ -110,19 +113,25 @@ class KernelProbe:
     def reset(self):
         self.samples = []
 
-    def mean_ms(self, skip_below_ms=0.05):
-        """Average over the launches that had rows to work on (a pass past the last slab takes microseconds)."""
-        real = [x for x in self.samples if x >= skip_below_ms]
+    def threshold(self):
+        """A launch without rows (a pass past the last slab) takes microseconds, one with rows milliseconds."""
+        return 0.1 * max(self.samples, default=0.0)
+
+    def mean_ms(self):
+        """Average over the launches that had rows to work on."""
+        real = [x for x in self.samples if x >= self.threshold()]
         return sum(real) / max(1, len(real))
 
 
-def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, route="slabs"):
+def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, route="slabs", train_head=False):
     """route: "slabs" = grpo_loss_on_hidden as it runs by default, "one-call-recompute" = the same entry with
-    token_slabs=False, "recompute" = fused_lm_head_logprobs -> grpo_loss_fused -> backward."""
+    token_slabs=False, "recompute" = fused_lm_head_logprobs -> grpo_loss_fused -> backward.  dpo: the frozen
+    head of the DPO config unless train_head (then route "slabs" = dpo_loss_on_hidden, else the differentiable
+    calls with a recomputing backward)."""
     dev = "cuda:0"
     torch.manual_seed(0)
     hidden = torch.randn(n_tokens, hdim, device=dev).bfloat16().requires_grad_(True)
-    weight = (torch.randn(vocab, hdim, device=dev) * w_std).bfloat16().requires_grad_(not dpo)
+    weight = (torch.randn(vocab, hdim, device=dev) * w_std).bfloat16().requires_grad_(not dpo or train_head)
     labels = torch.randint(0, vocab, (n_tokens,), device=dev)
     cfg = _cfg()
     if not dpo:
@@ -149,11 +158,18 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, route="slabs"
         n_eff = int(mask.sum().item())
     fwd_timer = EventTimer(torch)
     probe = KernelProbe(oi, 2)  # the d_weight product: the largest share of the slab-wise step
+    dpo_slab = oi.dpo_utils.DEFAULT_DPO_SLAB_TOKENS
 
     def step():
         hidden.grad = None
         weight.grad = None
-        if dpo:
+        if dpo and train_head and route == "slabs":
+            with probe:
+                res = oi.dpo_utils.dpo_loss_on_hidden(
+                    hidden[None], weight, labels, ref_c, ref_r, 0.1, cu_seq_lens=cu, token_slabs=dpo_slab
+                )
+            loss = res.loss
+        elif dpo:
             with fwd_timer:
                 lp, _ = oi.fused_lm_head_logprobs(hidden, weight, shifted.view(-1), mask=mask)
             logps = oi.padding_free_collator.get_batch_logps(lp.view(1, -1), labels, cu)
@@ -190,7 +206,16 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, route="slabs"
         "bound": "mfma",
         "timer": fwd_timer,
     }
-    if dpo:
+    if dpo and train_head:
+        info["flops_step"] = 3.0 * flops_fwd
+        if route == "slabs":
+            info["kernel"] = (
+                f"gemm_store_kernel<true, true> (d_weight product of a slab of whole chosen/rejected pairs, at most {dpo_slab} "
+                "scored tokens, added to the fp32 d_weight; timed launch by launch through the library's event probe)"
+            )
+            info["alg_per_launch"] = None  # filled in from the number of launches that had rows
+            info["timer"] = probe
+    elif dpo:
         # the weight takes no gradient: the forward call also accumulates the weighted sum of weight rows that
         # the backward to hidden needs (per vocabulary chunk: statistics + exponentials, then E_chunk @ W_chunk)
         info["kernel"] = (
@@ -443,7 +468,10 @@ def cpu_baseline(torch, workload):
     threads = torch.get_num_threads()
     cfg = _cfg()
     torch.manual_seed(0)
-    workload = {"c3-recompute": "c3", "c3-one-call-recompute": "c3", "c4-recompute": "c4"}.get(workload, workload)
+    workload = {"c3-recompute": "c3", "c3-one-call-recompute": "c3", "c4-recompute": "c4", "c5-train-head": "c5t",
+                "c5-train-head-recompute": "c5t"}.get(workload, workload)
+    train_head = workload == "c5t"
+    workload = "c5" if train_head else workload
     if workload == "c5":
         # one chosen / rejected pair of 2 x 1024 tokens (of the 8 pairs of 2 x 2048), prompts masked out
         from oracle import dpo as o_dpo
@@ -451,7 +479,7 @@ def cpu_baseline(torch, workload):
         hdim, vocab, per = 8192, 128256, 1024
         n = 2 * per
         hidden = torch.randn(n, hdim).bfloat16().requires_grad_(True)
-        weight = (torch.randn(vocab, hdim) * 0.01).bfloat16()
+        weight = (torch.randn(vocab, hdim) * 0.01).bfloat16().requires_grad_(train_head)
         labels = torch.randint(0, vocab, (2, per))
         prompt = torch.randint(64, 513, (2,))
         labels[torch.arange(per).unsqueeze(0) < prompt.unsqueeze(1)] = -100
@@ -459,6 +487,7 @@ def cpu_baseline(torch, workload):
 
         def run():
             hidden.grad = None
+            weight.grad = None
             # reference order: bf16 lm_head GEMM, fp32 log_softmax + gather of the shifted labels, per-sequence
             # sums, sigmoid DPO loss, backward to the hidden states
             z = torch.nn.functional.linear(hidden, weight).view(2, per, vocab)
@@ -468,7 +497,8 @@ def cpu_baseline(torch, workload):
             losses.mean().backward()
 
         sample = (f"one pair of 2 x {per} tokens (of 8 pairs of 2 x 2048) at full H={hdim}, V={vocab}, W ~ N(0, 0.01); "
-                  "fwd + bwd to the hidden states; bf16 GEMM + fp32 log_softmax + sigmoid DPO loss")
+                  f"fwd + bwd to the hidden states{' and the head' if train_head else ''}; bf16 GEMM + fp32 log_softmax + "
+                  "sigmoid DPO loss")
     elif workload in ("c3", "c4"):
         hdim = 4096
         vocab, n = (100352 if workload == "c4" else 128256), 2048
@@ -589,9 +619,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="c3",
                     choices=["c1", "c2", "c2-two-pass", "c3", "c3-recompute", "c3-one-call-recompute", "c4",
-                             "c4-recompute", "c5", "pack"])
+                             "c4-recompute", "c5", "c5-train-head", "c5-train-head-recompute", "pack"])
     ap.add_argument("--slab-tokens", type=int, default=0,
-                    help="c3 / c4 only: slab size of the no-recompute step (0 = the package's default)")
+                    help="c3 / c4 / c5-train-head only: slab size of the no-recompute step (0 = the package's default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-library-gemm", action="store_true",
                     help="skip the reference points beside the measurement: the vendor bf16 GEMM of the same shape and, "
@@ -614,6 +644,7 @@ def main():
 
     if args.slab_tokens:
         oi.grpo_utils.DEFAULT_SLAB_TOKENS = args.slab_tokens
+        oi.dpo_utils.DEFAULT_DPO_SLAB_TOKENS = args.slab_tokens
     slab_note = f"slabs of at most {oi.grpo_utils.DEFAULT_SLAB_TOKENS} selected tokens, nothing recomputed, no [tokens, vocab] tensor"
     if args.workload == "c3":
         step, info = make_fused(torch, oi, 32768, 4096, 128256, 0.02)
@@ -643,6 +674,17 @@ def main():
     elif args.workload == "c5":
         step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True)
         name = "c5: fused lm_head+per-sequence logprob sums+sigmoid DPO loss, hidden bf16 [32768,8192], W bf16 [128256,8192], bwd to dHidden only"
+        dtype = "bf16"
+    elif args.workload == "c5-train-head":
+        step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True, train_head=True)
+        name = ("c5 with a trainable head: sigmoid DPO loss, d_hidden and d_weight from one call of dpo_loss_on_hidden, "
+                "hidden bf16 [32768,8192], W bf16 [128256,8192]; slabs of whole chosen/rejected pairs (at most "
+                f"{oi.dpo_utils.DEFAULT_DPO_SLAB_TOKENS} scored tokens), nothing recomputed")
+        dtype = "bf16"
+    elif args.workload == "c5-train-head-recompute":
+        step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True, train_head=True, route="recompute")
+        name = ("c5 with a trainable head through the differentiable calls (DPOLMHead's route): the backward recomputes "
+                "the logits (8 N H V executed for 6 N H V credited)")
         dtype = "bf16"
     elif args.workload == "c2":
         step, info = make_c2(torch, oi)
@@ -680,6 +722,10 @@ def main():
     value = info["tokens"] / (elapsed / args.steps)
 
     kernel_ms = info["timer"].mean_ms()
+    if info["alg_per_launch"] is None:  # launches of a probed kernel that had rows, per step
+        probe = info["timer"]
+        real = [x for x in probe.samples if x >= probe.threshold()]
+        info["alg_per_launch"] = info["flops_step"] / 3.0 / max(1.0, len(real) / args.steps)
     if info["bound"] == "mfma":
         achieved = info["alg_per_launch"] / (kernel_ms * 1e-3) / 1e12
         peak, unit = PEAK_BF16_TFLOPS, "TFLOP/s"
@@ -702,7 +748,7 @@ def main():
         roofline["whole_step_tflops"] = info["flops_step"] / (ms_per_step * 1e-3) / 1e12
         roofline["whole_step_frac"] = roofline["whole_step_tflops"] / PEAK_BF16_TFLOPS
         if not args.no_library_gemm:
-            hdim = 8192 if args.workload == "c5" else 4096
+            hdim = 8192 if args.workload.startswith("c5") else 4096
             vocab = 100352 if args.workload in ("c4", "c4-recompute") else 128256
             roofline["library_bf16_gemm_tflops"] = library_gemm_tflops(torch, 32768, hdim, vocab)
     if "bytes_step" in info:

@@ -374,6 +374,50 @@ def test_c5_llama70b_head_dpo_full_shape(dhidden_in_forward):
     _check_fused_head(hidden, weight, shifted.view(-1), mask, lp_leaf.grad, lp, None, hidden.grad, None, seed=5)
 
 
+@pytest.mark.parametrize("average_log_prob", [False, True])
+def test_c5_llama70b_head_dpo_with_trainable_head_full_shape(average_log_prob):
+    """The c5 batch with a trainable head, as the reference's DPO trains it
+    (open_instruct/olmo_core_train_modules.py:190-207): loss, d_hidden and d_weight from one call of
+    dpo_loss_on_hidden (slabs of whole pairs, nothing recomputed), sums (`dpo`) and averages (`dpo_norm`)."""
+    print(f"case c5 trainable head N=32768 H=8192 V=128256 average={average_log_prob}", flush=True)
+    torch.manual_seed(0)
+    n, h, v, per = 32768, 8192, 128256, 2048
+    seqs = n // per
+    hidden = torch.randn(n, h, device=DEV).bfloat16().requires_grad_(True)
+    weight = (torch.randn(v, h, device=DEV) * 0.01).bfloat16().requires_grad_(True)
+    labels = torch.randint(0, v, (seqs, per), device=DEV)
+    prompt = torch.randint(128, 1025, (seqs,), device=DEV)
+    pos = torch.arange(per, device=DEV).unsqueeze(0).expand(seqs, per)
+    labels[pos < prompt.unsqueeze(1)] = -100
+    labels = labels.view(1, -1)
+    cu = torch.arange(0, n + 1, per, device=DEV, dtype=torch.int32)
+    shifted = padding_free_collator.shift_labels(labels)
+    mask = (shifted != -100).view(-1)
+    bs = seqs // 2
+    scale = 1.0 / 1500 if average_log_prob else 1.0
+    ref_c = (torch.randn(bs, device=DEV) * 50 - 400) * scale
+    ref_r = (torch.randn(bs, device=DEV) * 50 - 400) * scale
+    beta = 5.0 if average_log_prob else 0.1
+
+    res = dpo_utils.dpo_loss_on_hidden(
+        hidden[None], weight, labels, ref_c, ref_r, beta, cu_seq_lens=cu, average_log_prob=average_log_prob
+    )
+    res.loss.backward()
+    torch.cuda.synchronize()
+    lp = res.per_token_logps.view(-1)
+
+    lp_leaf = lp.detach().cpu().requires_grad_(True)
+    logps_o = o_red.get_batch_logps_packed(lp_leaf[None], labels.cpu(), cu.cpu(), average_log_prob)
+    losses_o, cr_o, rr_o = o_dpo.dpo_loss(logps_o[:bs], logps_o[bs:], ref_c.cpu(), ref_r.cpu(), beta)
+    losses_o.mean().backward()
+    got_logps = torch.cat([res.chosen_logps, res.rejected_logps]).cpu()
+    assert (got_logps - logps_o.detach()).abs().max().item() <= 1e-5 * logps_o.detach().abs().max().item()
+    assert (res.losses.cpu() - losses_o.detach()).abs().max().item() <= 1e-2
+    assert abs(res.loss.item() - losses_o.detach().mean().item()) <= 1e-2
+    assert (res.chosen_rewards.cpu() - cr_o).abs().max().item() <= 1e-2
+    _check_fused_head(hidden, weight, shifted.view(-1), mask, lp_leaf.grad, lp, None, hidden.grad, weight.grad, seed=7)
+
+
 def _oracle_rows(logits, labels, rows_b, rows_t, temperature=1.0):
     """fp32 oracle logprob / entropy / softmax of single rows of a device logits tensor."""
     out = []
