@@ -48,11 +48,16 @@ PEAK_BF16_TFLOPS = 2500.0
 # be read from inside the process, so the figures are carried here from the committed summaries in
 # profiles/; workloads without a counter run report null.
 MEASURED_TRAFFIC_BYTES = {
+    # gemm_store_kernel<true, true>, the d_weight product of one slab (average of the launches with rows: two of them
+    # write fp32, the last one bf16): L2 misses of the tiled operand re-reads + the result
+    "c3": 14.45e9 + 1.75e9,
+    "c4": 11.31e9 + 1.44e9,
+    "c5-train-head": 31.41e9 + 3.50e9,
     # lmhead_fwd_kernel: L2 misses of the tiled operand re-reads (1.24 GB of unique operands at c3) + the partials
-    "c3-recompute": 42.01e9 + 0.20e9,
-    "c4-recompute": 40.21e9 + 0.20e9,
-    # oi_lmhead_logp_fwd_wsum: four launches of lmhead_fwd_kernel<true> and four of gemm_store_kernel<false, true>
-    "c5": 2 * (42.62e9 + 3.06e9) + 2 * (43.14e9 + 0.75e9),
+    "c3-recompute": 42.04e9 + 0.20e9,
+    "c4-recompute": 40.03e9 + 0.20e9,
+    # oi_lmhead_logp_fwd_wsum: two launches of lmhead_fwd_kernel<true> and two of gemm_store_kernel<false, true>
+    "c5": 2 * (44.55e9 + 3.09e9) + 2 * (49.66e9 + 0.75e9),
     # lsg_grpo_fused_kernel: one read of the logits (the row waits on the CU for the gradient pass) + one write of
     # dlogits
     "c2": 16.88e9 + 16.94e9,
