@@ -828,6 +828,26 @@ __global__ void __launch_bounds__(NTHREADS)
 // ---------------------------------------------------------------------------------------------
 // backward steps 2 and 3: plain tile products with a store epilogue
 // ---------------------------------------------------------------------------------------------
+// Transposes the 4 x 4 block that a quad of lanes holds: on entry lane k of the quad has v[e] = M[e][k]
+// (one column, four consecutive rows, which is how the MFMA leaves its results), on return
+// v[f] = M[k][f] (one row, four consecutive columns, which is what a 16-byte store wants).  Two
+// exchange steps inside the quad (DPP), every lane of the wave must take part.
+__device__ __forceinline__ float quad_swap(float x, bool far) {
+    const int i = __float_as_int(x);
+    return __int_as_float(far ? __builtin_amdgcn_mov_dpp(i, 0x4E /* quad_perm 2,3,0,1 */, 0xF, 0xF, true)
+                              : __builtin_amdgcn_mov_dpp(i, 0xB1 /* quad_perm 1,0,3,2 */, 0xF, 0xF, true));
+}
+__device__ __forceinline__ void quad_transpose(float (&v)[4], int lane) {
+    const bool b0 = lane & 1, b1 = lane & 2;
+    const float r01 = quad_swap(b0 ? v[0] : v[1], false), r23 = quad_swap(b0 ? v[2] : v[3], false);
+    const float t0 = b0 ? r01 : v[0], t1 = b0 ? v[1] : r01, t2 = b0 ? r23 : v[2], t3 = b0 ? v[3] : r23;
+    const float ra = quad_swap(b1 ? t0 : t2, true), rb = quad_swap(b1 ? t1 : t3, true);
+    v[0] = b1 ? ra : t0;
+    v[1] = b1 ? rb : t1;
+    v[2] = b1 ? t2 : ra;
+    v[3] = b1 ? t3 : rb;
+}
+
 // mode 0: out_f32  = acc          mode 1: out_f32 += acc
 // mode 2: out_bf16 = acc          mode 3: out_bf16 = out_f32 + acc   (last chunk of d_hidden)
 // mode 4: out_bf16 += acc         (rows added to a d_weight that was already rounded)
@@ -855,6 +875,92 @@ __device__ __forceinline__ void gemm_store_tile(Operand A, int64_t M, Operand B,
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    }
+    if (((N | ldo) & 3) == 0 && (reinterpret_cast<uintptr_t>(out_f32) & 15) == 0 &&
+        (reinterpret_cast<uintptr_t>(out_bf16) & 7) == 0) {
+        // Every store and load of the epilogue as a 16-byte piece (8 bytes of bf16): after a 4 x 4
+        // transpose inside each quad of lanes a lane holds four consecutive columns of one row.  A
+        // quarter of the memory instructions of the one-value-per-lane form, whose address
+        // processing is what an epilogue of 128 values per lane waits for.  The fp32 sum of the
+        // accumulating modes is requested before the transposes of the half tile it belongs to and
+        // added with plain loads and stores: every element has one writer per launch and the
+        // launches follow each other on the stream, so no atomic is needed.
+        const int kq = lane & 3, g = (lane & 31) >> 2, hl = lane >> 5;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            int64_t row[4], dst[4];
+            bool ok[4];
+            float sa[4], sb[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                row[q] = m0 + wm * 64 + i * 32 + q * 8 + hl * 4 + kq;
+                ok[q] = row[q] < m_valid;
+                dst[q] = (ok[q] && out_rows) ? (int64_t)out_rows[row[q]] : row[q];
+                sa[q] = (ok[q] && scale_a) ? scale_a[row[q]] : 1.f;
+                sb[q] = (ok[q] && scale_a) ? scale_b[row[q]] : 1.f;
+            }
+            // two of the four 32-column blocks at a time: 32 registers of sums in flight
+#pragma unroll
+            for (int jh = 0; jh < 2; ++jh) {
+                oi_f32x4 part[2][4];
+                uint2 part16[2][4];
+                if (mode == 1 || mode == 3) {
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const int64_t col = n0 + wn * 128 + (2 * jh + jj) * 32 + 4 * g;
+                            part[jj][q] = (ok[q] && col < N)
+                                              ? *reinterpret_cast<const oi_f32x4*>(out_f32 + row[q] * ldo + col)
+                                              : oi_f32x4{0.f, 0.f, 0.f, 0.f};
+                        }
+                } else if (mode == 4) {
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const int64_t col = n0 + wn * 128 + (2 * jh + jj) * 32 + 4 * g;
+                            part16[jj][q] = (ok[q] && col < N)
+                                                ? *reinterpret_cast<const uint2*>(out_bf16 + dst[q] * ldo + col)
+                                                : make_uint2(0u, 0u);
+                        }
+                }
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+                    const int j = 2 * jh + jj;
+                    const int64_t col = n0 + wn * 128 + j * 32 + 4 * g;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float v[4] = {acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+                        quad_transpose(v, lane);
+                        if (!ok[q] || col >= N) continue;
+                        if (scale_a) {
+                            // a row whose factor is exactly 0 is 0 whatever its sum holds (the sums of
+                            // rows that were taken out may have left the fp32 range)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] = sb[q] == 0.f ? 0.f : v[e] * sa[q] * sb[q];
+                        }
+                        if (mode == 1 || mode == 3) {
+                            v[0] += part[jj][q].x;
+                            v[1] += part[jj][q].y;
+                            v[2] += part[jj][q].z;
+                            v[3] += part[jj][q].w;
+                        } else if (mode == 4) {
+                            v[0] += oi_bf16lo_to_f32(part16[jj][q].x);
+                            v[1] += oi_bf16hi_to_f32(part16[jj][q].x);
+                            v[2] += oi_bf16lo_to_f32(part16[jj][q].y);
+                            v[3] += oi_bf16hi_to_f32(part16[jj][q].y);
+                        }
+                        if (mode <= 1)
+                            *reinterpret_cast<oi_f32x4*>(out_f32 + row[q] * ldo + col) = oi_f32x4{v[0], v[1], v[2], v[3]};
+                        else
+                            *reinterpret_cast<uint2*>(out_bf16 + dst[q] * ldo + col) =
+                                make_uint2(oi_pack_bf16x2(v[0], v[1]), oi_pack_bf16x2(v[2], v[3]));
+                    }
+                }
+            }
+        }
+        return;
     }
     if (mode >= 2 && (ldo & 1) == 0) {
         // bf16 output: neighbouring lanes hold neighbouring columns of the same rows; after one DPP
@@ -976,6 +1082,8 @@ __global__ void __launch_bounds__(NTHREADS)
             B.k_valid = n;
         }
     }
+    // a product without terms that would only be added changes nothing: no tile is drawn at all
+    if (K <= 0 && (mode == 1 || mode == 4)) return;
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (queue) {
         for_each_tile(queue, tiles_m, tiles_n, lds, [&](int64_t tm, int64_t tn) {
