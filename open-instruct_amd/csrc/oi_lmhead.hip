@@ -696,26 +696,41 @@ constexpr float KEEP_MAX_LOG2 = 64.f;
 // `unsafe` (one byte per caller row, optional, cleared by the caller beforehand): set for a token
 // whose kept exponentials cannot be trusted (its maximum is too far above xref[n], or is not a
 // number); never cleared here, so marks that the caller has put there survive.
-__global__ void lmhead_fwd_combine_kernel(const float4* __restrict__ partial, const float* __restrict__ zy,
-                                          int64_t n_tokens, const int32_t* __restrict__ n_dev,
-                                          const int32_t* __restrict__ rows, const uint8_t* __restrict__ row_mask,
-                                          int64_t n_total, int64_t n_splits, int64_t n_pad, float inv_t, float c,
-                                          float* __restrict__ logprob, float* __restrict__ entropy,
-                                          float* __restrict__ lse_out, const float* __restrict__ xref,
-                                          uint8_t* __restrict__ unsafe) {
-    const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+// Launch: 256 threads = 4 waves; a workgroup handles 64 tokens (lane = token, so the 16-byte partials
+// of a split are read as one contiguous piece per wave), wave w merges the splits w, w + 4, ... and
+// the four results meet in the LDS.
+constexpr int COMBINE_TOKENS = 64;
+__global__ void __launch_bounds__(256)
+    lmhead_fwd_combine_kernel(const float4* __restrict__ partial, const float* __restrict__ zy, int64_t n_tokens,
+                              const int32_t* __restrict__ n_dev, const int32_t* __restrict__ rows,
+                              const uint8_t* __restrict__ row_mask, int64_t n_total, int64_t n_splits, int64_t n_pad,
+                              float inv_t, float c, float* __restrict__ logprob, float* __restrict__ entropy,
+                              float* __restrict__ lse_out, const float* __restrict__ xref,
+                              uint8_t* __restrict__ unsafe) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t n = (int64_t)blockIdx.x * COMBINE_TOKENS + lane;
     if (n_dev) n_tokens = *n_dev;
-    if (row_mask && n < n_total && !row_mask[n]) {
+    if (wave == 0 && row_mask && n < n_total && !row_mask[n]) {
         logprob[n] = 0.f;
         if (entropy) entropy[n] = 0.f;
         if (lse_out) lse_out[n] = 0.f;
     }
-    if (n >= n_tokens) return;
     float m = OI_NEG_BIG, s = 0.f, t = 0.f;
-    for (int64_t sp = 0; sp < n_splits; ++sp) {
-        const float4 p = partial[sp * n_pad + n];
-        merge_stats(m, s, t, p.x, p.y, p.z, &m, &s, &t);
+    if (n < n_tokens)
+        for (int64_t sp = wave; sp < n_splits; sp += 4) {
+            const float4 p = partial[sp * n_pad + n];
+            merge_stats(m, s, t, p.x, p.y, p.z, &m, &s, &t);
+        }
+    __shared__ float red[3][3][COMBINE_TOKENS];
+    if (wave > 0) {
+        red[wave - 1][0][lane] = m;
+        red[wave - 1][1][lane] = s;
+        red[wave - 1][2][lane] = t;
     }
+    __syncthreads();
+    if (wave != 0 || n >= n_tokens) return;
+#pragma unroll
+    for (int w = 0; w < 3; ++w) merge_stats(m, s, t, red[w][0][lane], red[w][1][lane], red[w][2][lane], &m, &s, &t);
     const double ln2 = 0.69314718055994530942;
     const double log2s = log2((double)s);
     // the statistics are in units of x = z * c with the fp32 constant c the tile kernel multiplied by:
@@ -1519,7 +1534,7 @@ void enqueue_fwd(const FwdPlan& p, char* ws, const RowInputs& in, const uint8_t*
     } else
         hipLaunchKernelGGL(lmhead_fwd_kernel<false>, grid, dim3(NTHREADS), 0, s, Wp, in.hidden, in.labels, n_tokens,
                            in.n_dev, hidden_dim, vocab, c, fl, p.n_pad, partial, zy, queue);
-    hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
+    hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + COMBINE_TOKENS - 1) / COMBINE_TOKENS)), dim3(256), 0, s, partial,
                        zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, c, logprob,
                        entropy, lse, keep.buf ? keep.xref : static_cast<const float*>(nullptr),
                        keep.buf ? keep.unsafe : static_cast<uint8_t*>(nullptr));
@@ -1568,7 +1583,7 @@ void enqueue_fwd_wsum(const FwdPlan& p, char* ws, const RowInputs& in, const uin
                            s, a, p.n_pad, b, hidden_dim, round_up(valid, BK), ci == 0 ? 0 : 1, wsum,
                            static_cast<uint16_t*>(nullptr), hidden_dim, n_tokens, dyn, q + FWD_QUEUE_WORDS);
     }
-    hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, partial,
+    hipLaunchKernelGGL(lmhead_fwd_combine_kernel, dim3((unsigned)((n_tokens + COMBINE_TOKENS - 1) / COMBINE_TOKENS)), dim3(256), 0, s, partial,
                        zy, n_tokens, in.n_dev, in.rows, row_mask, n_tokens, p.n_splits, p.n_pad, inv_temperature, c, logprob,
                        entropy, lse, static_cast<const float*>(xref), unsafe);
 }
@@ -1802,11 +1817,12 @@ __global__ void plan_equal_slabs_kernel(const int32_t* __restrict__ count, int c
     meta[i].reserved = 0;
 }
 
-// the per-token outputs of rows that take no part are zero
-__global__ void zero_unselected_f32_kernel(const uint8_t* __restrict__ mask, int64_t n, float* __restrict__ a,
-                                           float* __restrict__ b, float* __restrict__ c) {
+// The per-token outputs start at zero: rows that take no part stay there, and the passes that look
+// at every row before its own slab has run (the upstream gradient of a slab is computed for all rows)
+// read zeros rather than whatever the caller's buffers held.
+__global__ void zero_f32_kernel(int64_t n, float* __restrict__ a, float* __restrict__ b, float* __restrict__ c) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n || mask[i]) return;
+    if (i >= n) return;
     a[i] = 0.f;
     if (b) b[i] = 0.f;
     if (c) c[i] = 0.f;
@@ -1853,8 +1869,7 @@ int run_slab_passes(const SlabPlan& p, char* ws, const SlabStep& st, hipStream_t
     hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((p.n_pad / 4 + 255) / 256)), dim3(256), 0, s,
                        reinterpret_cast<uint32_t*>(unsafe), (int)(p.n_pad / 4));
     plan_rows(order, count, meta);
-    hipLaunchKernelGGL(zero_unselected_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, st.mask, n,
-                       st.logprob, st.entropy, lse);
+    hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, st.logprob, st.entropy, lse);
     hipLaunchKernelGGL(zero_unselected_rows_kernel, dim3((unsigned)n), dim3(256), 0, s, st.mask,
                        static_cast<const float*>(nullptr), hdim, static_cast<uint16_t*>(st.d_hidden));
     for (int64_t i = 0; i < p.n_passes; ++i) {
@@ -2102,7 +2117,9 @@ int grpo_step_in_slabs(const void* hidden, const void* weight, const int64_t* la
     float* grad = reinterpret_cast<float*>(ws + p.off_grad);
     float* row_denoms = reinterpret_cast<float*>(ws + p.off_denoms);
     // the denominators come from the mask alone: a first pass of the statistics over logprobs that are
-    // not there yet leaves them in row_denoms (its other results are overwritten at the end)
+    // not there yet (zeros) leaves them in row_denoms (its other results are overwritten at the end)
+    hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s, n_tokens, logprob, entropy,
+                       static_cast<float*>(nullptr));
     int rc = oi_grpo_fused_fwd(logprob, old_logprobs, ref_logprobs, advantages, mask, rho_weights, entropy, nullptr, nullptr,
                                nullptr, nullptr, rows, cols, loss_fn, ratio_lo, ratio_hi, kl_estimator, beta, axis_mode,
                                denominator, scale, out_stats, row_denoms, ws + p.off_stats,
