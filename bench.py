@@ -128,7 +128,7 @@ class KernelProbe:
         return sum(real) / max(1, len(real))
 
 
-def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, route="slabs", train_head=False):
+def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, route="slabs", train_head=False, one_call=False):
     """route: "slabs" = grpo_loss_on_hidden as it runs by default, "one-call-recompute" = the same entry with
     token_slabs=False, "recompute" = fused_lm_head_logprobs -> grpo_loss_fused -> backward.  dpo: the frozen
     head of the DPO config unless train_head (then route "slabs" = dpo_loss_on_hidden, else the differentiable
@@ -162,13 +162,14 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, route="slabs"
         ref_r = torch.randn(seqs // 2, device=dev) * 50 - 400
         n_eff = int(mask.sum().item())
     fwd_timer = EventTimer(torch)
-    probe = KernelProbe(oi, 2)  # the d_weight product: the largest share of the slab-wise step
+    # the d_weight product: the largest share of the slab-wise step (without d_weight: the d_hidden product)
+    probe = KernelProbe(oi, 1 if (dpo and one_call and not train_head) else 2)
     dpo_slab = oi.dpo_utils.DEFAULT_DPO_SLAB_TOKENS
 
     def step():
         hidden.grad = None
         weight.grad = None
-        if dpo and train_head and route == "slabs":
+        if dpo and route == "slabs" and (train_head or one_call):
             with probe:
                 res = oi.dpo_utils.dpo_loss_on_hidden(
                     hidden[None], weight, labels, ref_c, ref_r, 0.1, cu_seq_lens=cu, token_slabs=dpo_slab
@@ -205,15 +206,24 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, route="slabs"
     info = {
         "tokens": n_tokens,
         "rows_multiplied": n_eff,
+        "hdim": hdim,
+        "vocab": vocab,
         "flops_step": (2.0 if dpo else 3.0) * flops_fwd,
         "kernel": "lmhead_fwd_kernel (fused lm_head forward: MFMA tiles + online softmax statistics)",
         "alg_per_launch": flops_fwd,
         "bound": "mfma",
         "timer": fwd_timer,
     }
-    if dpo and train_head:
-        info["flops_step"] = 3.0 * flops_fwd
-        if route == "slabs":
+    if dpo and (train_head or one_call):
+        info["flops_step"] = (3.0 if train_head else 2.0) * flops_fwd
+        if route == "slabs" and one_call and not train_head:
+            info["kernel"] = (
+                f"gemm_store_kernel<false, true> (d_hidden product of a slab of whole chosen/rejected pairs, at most {dpo_slab} "
+                "scored tokens; timed launch by launch through the library's event probe)"
+            )
+            info["alg_per_launch"] = None
+            info["timer"] = probe
+        elif route == "slabs":
             info["kernel"] = (
                 f"gemm_store_kernel<true, true> (d_weight product of a slab of whole chosen/rejected pairs, at most {dpo_slab} "
                 "scored tokens, added to the fp32 d_weight; timed launch by launch through the library's event probe)"
@@ -398,6 +408,8 @@ def make_c4(torch, oi, hdim=4096, vocab=100352, n_seqs=16, budget=32768, route="
     info = {
         "tokens": n_tokens,
         "rows_multiplied": n_eff,
+        "hdim": hdim,
+        "vocab": vocab,
         "flops_step": 3.0 * flops_fwd,
         "kernel": "lmhead_fwd_kernel (fused lm_head forward: MFMA tiles + online softmax statistics)",
         "alg_per_launch": flops_fwd,
@@ -473,7 +485,7 @@ def cpu_baseline(torch, workload):
     threads = torch.get_num_threads()
     cfg = _cfg()
     torch.manual_seed(0)
-    workload = {"c3-recompute": "c3", "c3-one-call-recompute": "c3", "c4-recompute": "c4", "c5-train-head": "c5t",
+    workload = {"c3-recompute": "c3", "c3-one-call-recompute": "c3", "c4-recompute": "c4", "c5-one-call": "c5", "c5-train-head": "c5t",
                 "c5-train-head-recompute": "c5t"}.get(workload, workload)
     train_head = workload == "c5t"
     workload = "c5" if train_head else workload
@@ -624,7 +636,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="c3",
                     choices=["c1", "c2", "c2-two-pass", "c3", "c3-recompute", "c3-one-call-recompute", "c4",
-                             "c4-recompute", "c5", "c5-train-head", "c5-train-head-recompute", "pack"])
+                             "c4-recompute", "c5", "c5-one-call", "c5-train-head", "c5-train-head-recompute", "pack"])
     ap.add_argument("--slab-tokens", type=int, default=0,
                     help="c3 / c4 / c5-train-head only: slab size of the no-recompute step (0 = the package's default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -680,6 +692,12 @@ def main():
         step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True)
         name = "c5: fused lm_head+per-sequence logprob sums+sigmoid DPO loss, hidden bf16 [32768,8192], W bf16 [128256,8192], bwd to dHidden only"
         dtype = "bf16"
+    elif args.workload == "c5-one-call":
+        step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True, one_call=True)
+        name = ("c5 from one call of dpo_loss_on_hidden (frozen head): sigmoid DPO loss and d_hidden, hidden bf16 [32768,8192], "
+                f"W bf16 [128256,8192]; slabs of whole chosen/rejected pairs (at most {oi.dpo_utils.DEFAULT_DPO_SLAB_TOKENS} "
+                "scored tokens), nothing recomputed, no fp32 sums between the passes")
+        dtype = "bf16"
     elif args.workload == "c5-train-head":
         step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True, train_head=True)
         name = ("c5 with a trainable head: sigmoid DPO loss, d_hidden and d_weight from one call of dpo_loss_on_hidden, "
@@ -730,7 +748,7 @@ def main():
     if info["alg_per_launch"] is None:  # launches of a probed kernel that had rows, per step
         probe = info["timer"]
         real = [x for x in probe.samples if x >= probe.threshold()]
-        info["alg_per_launch"] = info["flops_step"] / 3.0 / max(1.0, len(real) / args.steps)
+        info["alg_per_launch"] = 2.0 * info["rows_multiplied"] * info["hdim"] * info["vocab"] / max(1.0, len(real) / args.steps)
     if info["bound"] == "mfma":
         achieved = info["alg_per_launch"] / (kernel_ms * 1e-3) / 1e12
         peak, unit = PEAK_BF16_TFLOPS, "TFLOP/s"
@@ -749,6 +767,27 @@ def main():
         "kernel_ms": kernel_ms,
         "algorithmic_per_launch": info["alg_per_launch"],
     }
+    if isinstance(info["timer"], KernelProbe):
+        # the other tile kernels of the slab-wise call, each timed over three more steps (outside the timed region)
+        probe, timed_kernel = info["timer"], info["timer"].kernel
+        names = {0: "lmhead_fwd_kernel<true> (forward that keeps its exponentials)", 1: "gemm_store_kernel<false, true> (d_hidden product)",
+                 2: "gemm_store_kernel<true, true> (d_weight product)"}
+        per_kernel = {names[timed_kernel]: {"ms_per_launch": kernel_ms, "frac": achieved / peak}}
+        for k in (0, 1, 2):
+            if k == timed_kernel or (k == 2 and info["flops_step"] < 2.5 * 2.0 * info["rows_multiplied"] * info["hdim"] * info["vocab"]):
+                continue
+            probe.kernel = k
+            probe.reset()
+            for _ in range(3):
+                step()
+            torch.cuda.synchronize()
+            real = [x for x in probe.samples if x >= probe.threshold()]
+            if real:
+                ms_k = sum(real) / len(real)
+                alg_k = 2.0 * info["rows_multiplied"] * info["hdim"] * info["vocab"] / (len(real) / 3.0)
+                per_kernel[names[k]] = {"ms_per_launch": ms_k, "frac": alg_k / (ms_k * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
+        probe.kernel = timed_kernel
+        roofline["tile_kernels_of_the_call"] = per_kernel
     if "flops_step" in info:
         roofline["whole_step_tflops"] = info["flops_step"] / (ms_per_step * 1e-3) / 1e12
         roofline["whole_step_frac"] = roofline["whole_step_tflops"] / PEAK_BF16_TFLOPS
