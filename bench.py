@@ -50,14 +50,14 @@ PEAK_BF16_TFLOPS = 2500.0
 MEASURED_TRAFFIC_BYTES = {
     # gemm_store_kernel<true, true>, the d_weight product of one slab (average of the launches with rows: two of them
     # write fp32, the last one bf16): L2 misses of the tiled operand re-reads + the result
-    "c3": 14.45e9 + 1.75e9,
-    "c4": 11.31e9 + 1.44e9,
-    "c5-train-head": 31.41e9 + 3.50e9,
+    "c3": 15.75e9 + 1.81e9,
+    "c4": 13.68e9 + 1.49e9,
+    "c5-train-head": 31.04e9 + 3.57e9,
     # lmhead_fwd_kernel: L2 misses of the tiled operand re-reads (1.24 GB of unique operands at c3) + the partials
-    "c3-recompute": 42.04e9 + 0.20e9,
-    "c4-recompute": 40.03e9 + 0.20e9,
+    "c3-recompute": 42.57e9 + 0.20e9,
+    "c4-recompute": 40.24e9 + 0.20e9,
     # oi_lmhead_logp_fwd_wsum: two launches of lmhead_fwd_kernel<true> and two of gemm_store_kernel<false, true>
-    "c5": 2 * (44.55e9 + 3.09e9) + 2 * (49.66e9 + 0.75e9),
+    "c5": 2 * (44.80e9 + 3.09e9) + 2 * (40.44e9 + 0.75e9),
     # lsg_grpo_fused_kernel: one read of the logits (the row waits on the CU for the gradient pass) + one write of
     # dlogits
     "c2": 16.88e9 + 16.94e9,
@@ -98,25 +98,48 @@ class EventTimer:
 # ------------------------------------------------------------------------------------------------
 class KernelProbe:
     """Times one tile kernel of the slab-wise entry points through the library's own event probe (the
-    call launches several kernels, so events around the call would time all of them)."""
+    call launches several kernels, so events around the call would time all of them).  The probe is armed
+    by reset() (or by the first step) and read only when the figures are asked for, after the caller has
+    synchronised: nothing inside the timed steps waits for the device.  The library records the first
+    1024 launches of the kernel; a run with more of them than that is refused."""
+
+    CAPACITY = 1024
 
     def __init__(self, oi, kernel):
-        self.oi, self.kernel, self.samples = oi, kernel, []
+        self.oi, self.kernel, self._samples, self._armed = oi, kernel, [], False
 
     def __enter__(self):
-        self.oi._lib.call("oi_lmhead_probe_arm", self.kernel)
+        if not self._armed:
+            self.oi._lib.call("oi_lmhead_probe_arm", self.kernel)
+            self._armed = True
         return self
 
     def __exit__(self, *exc):
+        pass
+
+    def _collect(self):
         import ctypes
 
-        ms = (ctypes.c_float * 256)()
-        n = ctypes.c_int(0)
-        self.oi._lib.call("oi_lmhead_probe_read", ms, 256, ctypes.byref(n))
-        self.samples += [ms[i] for i in range(min(n.value, 256))]
+        if self._armed:
+            ms = (ctypes.c_float * self.CAPACITY)()
+            n = ctypes.c_int(0)
+            self.oi._lib.call("oi_lmhead_probe_read", ms, self.CAPACITY, ctypes.byref(n))
+            if n.value >= self.CAPACITY:
+                raise SystemExit(f"bench.py: more than {self.CAPACITY} launches of the probed kernel between two readings; use fewer --steps")
+            self._samples += [ms[i] for i in range(n.value)]
+            self._armed = False
+
+    @property
+    def samples(self):
+        self._collect()
+        return self._samples
 
     def reset(self):
-        self.samples = []
+        """Drops what was recorded so far and arms the probe again (the events are created here, before the
+        caller starts its clock)."""
+        self._collect()
+        self._samples = []
+        self.__enter__()
 
     def threshold(self):
         """A launch without rows (a pass past the last slab) takes microseconds, one with rows milliseconds."""
@@ -640,6 +663,9 @@ def main():
     ap.add_argument("--slab-tokens", type=int, default=0,
                     help="c3 / c4 / c5-train-head only: slab size of the no-recompute step (0 = the package's default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--one-kernel", action="store_true",
+                    help="time only the dominant kernel of a slab-wise call, not the other two tile kernels over extra steps "
+                         "(for profiler runs, whose traces should hold the warm-up and timed steps only)")
     ap.add_argument("--no-library-gemm", action="store_true",
                     help="skip the reference points beside the measurement: the vendor bf16 GEMM of the same shape and, "
                          "for c3, the timing of the recomputing route")
@@ -767,7 +793,7 @@ def main():
         "kernel_ms": kernel_ms,
         "algorithmic_per_launch": info["alg_per_launch"],
     }
-    if isinstance(info["timer"], KernelProbe):
+    if isinstance(info["timer"], KernelProbe) and not args.one_kernel:
         # the other tile kernels of the slab-wise call, each timed over three more steps (outside the timed region)
         probe, timed_kernel = info["timer"], info["timer"].kernel
         names = {0: "lmhead_fwd_kernel<true> (forward that keeps its exponentials)", 1: "gemm_store_kernel<false, true> (d_hidden product)",

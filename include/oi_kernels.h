@@ -512,7 +512,7 @@ int oi_lmhead_dpo_fwd_bwd(const void* hidden, const void* weight, const int64_t*
  * oi_lmhead_probe_arm(kernel) and oi_lmhead_probe_read the slab-wise calls of this process record a
  * pair of HIP events, on the stream of the call, around every launch of the chosen tile kernel:
  * 0 = the forward that keeps its exponentials, 1 = the d_hidden product, 2 = the d_weight product
- * (at most 256 launches; later ones are not recorded).  oi_lmhead_probe_read waits for the recorded
+ * (at most 1024 launches; later ones are not recorded).  oi_lmhead_probe_read waits for the recorded
  * events, writes the duration of each recorded launch in milliseconds to ms[0 .. min(n, capacity)),
  * the number of recorded launches to *n_launches, and disarms the probe.  Launches whose slab is
  * empty are recorded too (they take a few microseconds).  Not thread-safe; do not arm it around a

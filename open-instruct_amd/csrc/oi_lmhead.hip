@@ -1320,7 +1320,7 @@ __global__ void __launch_bounds__(256)
 struct Probe {
     int kernel = -1;  // 0 forward with kept exponentials, 1 d_hidden product, 2 d_weight product; -1 = off
     int used = 0;
-    static constexpr int MAX_LAUNCHES = 256;
+    static constexpr int MAX_LAUNCHES = 1024;
     hipEvent_t ev[2 * MAX_LAUNCHES];
 };
 Probe g_probe;
