@@ -767,7 +767,7 @@ def test_entry_points_replay_from_a_hip_graph(slabs, t):
     """The C entry points enqueue kernels only (no allocation, no synchronisation, no memset nodes), so a
     caller may capture them in a HIP graph.  Two launch-bound cases: logprob + entropy + masked means on
     small logits, and the whole GRPO step on hidden states in one call (recomputing, and in two token slabs
-    whose d_weight accumulates through the L2's atomics).  Every replay is compared with the eager result on
+    whose d_weight accumulates in fp32 from one slab to the next).  Every replay is compared with the eager result on
     inputs that eager work changed between the replays."""
     torch.manual_seed(51)
     logits = (torch.randn(4, 128, 8000, device=DEV) * 2.0)
@@ -819,6 +819,55 @@ def test_entry_points_replay_from_a_hip_graph(slabs, t):
         torch.cuda.synchronize()
         assert torch.equal(got[0], e_small), i
         assert torch.equal(got[1], e_loss) and torch.equal(got[2], e_dh) and torch.equal(got[3], e_dw), i
+
+
+@pytest.mark.parametrize("slabs", [True, 512])
+def test_dpo_step_replays_from_a_hip_graph(slabs):
+    """The one-call DPO step (open_instruct/olmo_core_train_modules.py:190-207 as one C call: head, per-sequence
+    sums, pair loss, both gradients) enqueues kernels only, so it can be captured: a packed batch with every pair
+    in one slab, and in slabs of one or two pairs whose d_weight accumulates from slab to slab.  Every replay is
+    compared with the eager result on inputs that eager work changed between the replays."""
+    torch.manual_seed(52)
+    h, v, pairs = 128, 3000, 4
+    lens = torch.randint(60, 240, (2 * pairs,))
+    cu = torch.tensor([0] + lens.cumsum(0).tolist(), dtype=torch.int32, device=DEV)
+    total = int(cu[-1])
+    labels = torch.randint(0, v, (1, total), device=DEV)
+    for i in range(2 * pairs):
+        labels[0, int(cu[i]) : int(cu[i]) + 4 + i] = -100
+    hidden = torch.randn(1, total, h, device=DEV).bfloat16().requires_grad_(True)
+    weight = (torch.randn(v, h, device=DEV) * 0.2).bfloat16().requires_grad_(True)
+    ref_c, ref_r = -torch.rand(pairs, device=DEV) * 300, -torch.rand(pairs, device=DEV) * 300
+
+    def step():
+        hidden.grad = None
+        weight.grad = None
+        res = dpo_utils.dpo_loss_on_hidden(
+            hidden, weight, labels, ref_c, ref_r, 0.1, cu_seq_lens=cu, label_smoothing=0.05, token_slabs=slabs
+        )
+        res.loss.backward()
+        return res.loss.detach(), res.chosen_logps, res.rejected_rewards, hidden.grad, weight.grad
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    for i in range(4):
+        with torch.no_grad():  # eager work between the replays changes the inputs in place
+            hidden.mul_(0.97)
+            ref_c.add_(1.5)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [x.clone() for x in captured]
+        eager = step()
+        torch.cuda.synchronize()
+        for a, b in zip(got, eager):
+            assert torch.equal(a, b), i
 
 
 class _TinyCausalLM(torch.nn.Module):
