@@ -165,6 +165,46 @@ def test_c3_llama8b_head_grpo_in_token_slabs_full_shape():
     _check_fused_head(hidden, weight, labels, mask, lp_leaf.grad, lp, ent, hidden.grad, weight.grad, seed=5)
 
 
+def test_qwen25_7b_head_grpo_in_token_slabs_full_shape():
+    """A head shape outside the benchmark list, from a model family the reference trains
+    (Qwen2.5-7B: H = 3584, V = 152064 with 151665 used ids; here V = 151665, which is not a multiple of
+    the 256-row vocabulary tile, so the last tile of every slab's exponentials is partly padding) at
+    temperature 0.7, through grpo_loss_on_hidden in three slabs of 4096 selected rows."""
+    print("case qwen2.5-7b head, token slabs, N=16384 H=3584 V=151665 T=0.7", flush=True)
+    torch.manual_seed(4)
+    n, h, v, temperature = 16384, 3584, 151665, 0.7
+    hidden = torch.randn(n, h, device=DEV).bfloat16().requires_grad_(True)
+    weight = (torch.randn(v, h, device=DEV) * 0.02).bfloat16().requires_grad_(True)
+    labels = torch.randint(0, v, (n,), device=DEV)
+    labels[:64] = v - 1 - torch.arange(64, device=DEV)  # labels inside the partly filled last tile
+    mask = torch.rand(n, device=DEV) < 0.7
+    adv = torch.randn(n, device=DEV)
+    cfg = _cfg()
+    with torch.no_grad():
+        lp0, _ = lm_head.fused_lm_head_logprobs(hidden, weight, labels, temperature=temperature, mask=mask)
+    old = lp0 + 0.05 * torch.randn(n, device=DEV)
+    ref = lp0 + 0.1 * torch.randn(n, device=DEV)
+    loss, stats, lp, ent = grpo_utils.grpo_loss_on_hidden(
+        hidden[None], weight, labels[None], old[None], ref[None], adv[None], mask[None], cfg,
+        temperature=temperature, token_slabs=4096,
+    )  # fmt: skip
+    loss.backward()
+    torch.cuda.synchronize()
+    lp, ent = lp[0], ent[0]
+    assert (lp - lp0).abs().max().item() <= 1e-5
+    lp_leaf = lp.detach().cpu().requires_grad_(True)
+    loss_o, *_ = o_grpo.grpo_token_loss(
+        lp_leaf[None], old.cpu()[None], ref.cpu()[None], adv.cpu()[None], mask.cpu()[None].float(), cfg
+    )
+    loss_o.backward()
+    assert abs(loss.item() - loss_o.item()) <= 1e-5 + 1e-5 * abs(loss_o.item())
+    assert int(stats["num_response_tokens"].item()) == int(mask.sum().item())
+    # the oracle at temperature T is the oracle at temperature 1 on weights W / T
+    # (d_weight by the chain rule through the scaled weights: d/dW = (d/d(W/T)) / T)
+    scaled = weight.detach().float() / temperature
+    _check_fused_head(hidden, scaled, labels, mask, lp_leaf.grad, lp, ent, hidden.grad, weight.grad.float() * temperature, seed=9)
+
+
 def test_c3_llama8b_head_grpo_full_shape():
     """hidden bf16 [32768, 4096], W bf16 [128256, 4096], 70 % response rows: fused lm_head + logprob +
     entropy + GRPO loss, forward and backward to dHidden and dW, through the three differentiable
