@@ -327,7 +327,7 @@ class FusedDPOResult:
     rejected_logps: torch.Tensor
     chosen_rewards: torch.Tensor
     rejected_rewards: torch.Tensor
-    per_token_logps: torch.Tensor
+    per_token_logps: torch.Tensor | None
 
 
 # slab size of the no-recompute DPO step when the caller names none (scored tokens per slab); a slab holds
@@ -462,15 +462,25 @@ def fused_loss_olmo(
     the model, the head receives the final hidden states and, because a loss specification is set on it for
     the duration of this call, computes the loss and both gradients right there (see
     :func:`dpo_loss_on_hidden`).  ``args`` is duck-typed like the reference's (``loss_type``, ``beta``,
-    ``label_smoothing``, ``gamma_beta_ratio``); ``loss_type`` ``dpo``, ``dpo_norm`` and ``simpo`` are
-    served, ``wpo`` (whose weight needs the finished sequence means inside the gradient) is not.
+    ``label_smoothing``, ``gamma_beta_ratio``); ``loss_type`` ``dpo``, ``dpo_norm`` and ``simpo`` take the
+    one-call form.  ``wpo`` (whose weight puts the finished sequence sums of a pair inside the gradient)
+    takes the reference's own sequence here, :func:`concatenated_forward_olmo` -> :func:`compute_loss` ->
+    ``losses.mean()`` on the differentiable fused head (its backward recomputes the logits), and comes
+    back in the same result type with ``per_token_logps=None``.
     ``result.loss.backward()`` continues into the trunk through the hidden states.
     """
     loss_type = str(getattr(args.loss_type, "value", args.loss_type))
-    if loss_type not in ("dpo", "dpo_norm", "simpo"):
-        raise ValueError(f"loss type {loss_type!r} has no fused form; use concatenated_forward_olmo and compute_loss")
+    if loss_type not in ("dpo", "dpo_norm", "simpo", "wpo"):
+        raise ValueError(f"Unknown loss type: {args.loss_type}")
     if average_log_prob is None:
         average_log_prob = loss_type in ("dpo_norm", "simpo")
+    if loss_type == "wpo":
+        chosen, rejected, _ = concatenated_forward_olmo(model, batch, average_log_prob=average_log_prob, packing=packing)
+        losses, chosen_rewards, rejected_rewards = compute_loss(args, batch, chosen, rejected, reference_cache)
+        return FusedDPOResult(
+            loss=losses.mean(), losses=losses.detach(), chosen_logps=chosen.detach(), rejected_logps=rejected.detach(),
+            chosen_rewards=chosen_rewards, rejected_rewards=rejected_rewards, per_token_logps=None,
+        )  # fmt: skip
     if packing:
         concat, _ = padding_free_collator.concatenated_inputs(batch)
     else:
