@@ -592,8 +592,8 @@ def grpo_loss_on_hidden(
     buffer, the slab's tokens get their upstream gradient at once, and both backward products read
     that buffer before the next slab overwrites it (``d_weight`` accumulates in fp32 over the
     slabs).  6·N·H·V of matrix work instead of 8·N·H·V; the scratch is ``[slab, vocab]`` bf16 plus an
-    fp32 ``[vocab, hidden]``, never ``[tokens, vocab]``.  Larger slabs are faster (fewer passes over the
-    fp32 ``d_weight``, fewer launch ends).  The route has no limit on the size of the logits or on the
+    fp32 ``[vocab, hidden]``, never ``[tokens, vocab]``.  The slab size hardly matters for the time of the step
+    (8192 to 32768 tokens measured within 1 %); smaller slabs need less scratch.  The route has no limit on the size of the logits or on the
     temperature: a token whose label is extremely unlikely (largest logit more than 44 nats above the
     label's) or whose logits hold a NaN is flagged on the device and served by a recomputing backward
     over the flagged rows inside the same call.  ``token_slabs=False`` is the recomputing step: one
