@@ -1,6 +1,6 @@
 """Benchmark of the policy-loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c1|c4|c5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c1|c4|c5|...] [--slab-tokens N]
 
 Prints ONE JSON line.  A "step" is one pass of the hot path (forward + backward) over one batch of
 synthetic inputs that already live in HBM.  Workloads are the BASELINE configs:
@@ -18,10 +18,13 @@ synthetic inputs that already live in HBM.  Workloads are the BASELINE configs:
   c5: DPO at Llama-3.1-70B head shape: hidden [32768, 8192], W [128256, 8192], bwd to dHidden only.
       c5-train-head: the same batch with a trainable head (what the reference's DPO trains), loss and
       both gradients from one no-recompute call (dpo_loss_on_hidden); c5-train-head-recompute: the same
-      through the differentiable calls.
+      through the differentiable calls; c5-one-call: the frozen-head batch through dpo_loss_on_hidden.
+  pack: pack_sequences + advantage broadcast for 512 prompt / response pairs (about 1.09 M tokens).
 
 `roofline` describes the dominant kernel of the workload, timed with HIP events on the stream it
-runs on inside the timed region; `cpu_baseline` is the oracle's restatement of the reference's
+runs on inside the timed region (for the slab-wise workloads through the library's own event probe, with
+the other two tile kernels of the call timed over three more steps and reported beside it; --one-kernel
+leaves those extra steps out); `cpu_baseline` is the oracle's restatement of the reference's
 PyTorch path on a bounded sample of the same workload, on this machine's host cores.
 """
 
