@@ -1799,16 +1799,30 @@ SlabPlan plan_slabs(int64_t n, int64_t stats_rows, int64_t stats_cols, int64_t h
     return p;
 }
 
-// Equal slabs: the selected rows split into the fewest slabs of at most `cap` rows, all of the same
-// size (a multiple of 256 rows, the last one takes what is left); passes past the last slab are empty.
-__global__ void plan_equal_slabs_kernel(const int32_t* __restrict__ count, int cap, int n_passes,
-                                        SlabMeta* __restrict__ meta) {
+// The selected rows split into the fewest slabs of at most `cap` rows: all of the same size (a multiple of
+// 256 rows, the last one takes what is left), or, when that takes fewer rounds of tiles, full slabs of
+// `cap` rows and a last one with the remainder.  What is counted is the slab's d_hidden product, the one
+// tile kernel whose work items are long (a tile runs over the whole vocabulary): it has
+// ceil(rows / 256) * h_tiles tiles for `grid` resident workgroups, and a round of tiles takes the same
+// time whether it is full or not.  Passes past the last slab are empty.
+__global__ void plan_slabs_kernel(const int32_t* __restrict__ count, int cap, int n_passes, int h_tiles, int grid,
+                                  SlabMeta* __restrict__ meta) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n_passes) return;
     const int n = *count;
     const int k = n > 0 ? (n + cap - 1) / cap : 1;
-    int size = ((n + k - 1) / k + 255) / 256 * 256;
-    size = size > cap ? cap : size;
+    int equal = ((n + k - 1) / k + 255) / 256 * 256;
+    equal = equal > cap ? cap : equal;
+    auto rounds = [&](int size) {
+        int total = 0;
+        for (int j = 0; j < k; ++j) {
+            const int left = n - j * size;
+            const int rows = left < 0 ? 0 : (left > size ? size : left);
+            total += ((rows + 255) / 256 * h_tiles + grid - 1) / grid;
+        }
+        return total;
+    };
+    const int size = rounds(cap) < rounds(equal) ? cap : equal;
     const int left = n - i * size;
     meta[i].offset = i * size;
     meta[i].count = left < 0 ? 0 : (left > size ? size : left);
@@ -2133,8 +2147,9 @@ int grpo_step_in_slabs(const void* hidden, const void* weight, const int64_t* la
             hipLaunchKernelGGL(select_rows_kernel, dim3(1), dim3(SELECT_THREADS), 0, s, mask,
                                static_cast<const float*>(nullptr), n_tokens, order, count,
                                static_cast<uint32_t*>(nullptr), 0);
-            hipLaunchKernelGGL(plan_equal_slabs_kernel, dim3((unsigned)((p.n_passes + 63) / 64)), dim3(64), 0, s, count,
-                               (int)p.cap, (int)p.n_passes, meta);
+            const int64_t h_tiles = (hidden_dim + BN - 1) / BN;
+            hipLaunchKernelGGL(plan_slabs_kernel, dim3((unsigned)((p.n_passes + 63) / 64)), dim3(64), 0, s, count,
+                               (int)p.cap, (int)p.n_passes, (int)h_tiles, (int)resident_grid(p.cap / BM, h_tiles), meta);
         },
         [&](bool) {
             // every token's d loss / d logprob from its own logprob; tokens of later slabs hold numbers

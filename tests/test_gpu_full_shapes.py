@@ -205,6 +205,51 @@ def test_qwen25_7b_head_grpo_in_token_slabs_full_shape():
     _check_fused_head(hidden, scaled, labels, mask, lp_leaf.grad, lp, ent, hidden.grad, weight.grad.float() * temperature, seed=9)
 
 
+def test_token_slabs_with_a_small_remainder_slab():
+    """8500 selected rows at H = 4096 with slabs of at most 8192: two equal slabs of 4250 rows would take
+    four rounds of tiles in their d_hidden products, 8192 + 308 takes three, so the device-side plan picks
+    a full slab and a small remainder (whose d_weight product adds 308 rows' worth to the fp32 sum and
+    rounds it).  Sampled oracle check like the benchmark shapes, on a small vocabulary."""
+    print("case 8500 selected rows, H=4096 V=5000, slabs 8192 + 308", flush=True)
+    torch.manual_seed(6)
+    n, h, v = 9000, 4096, 5000
+    hidden = torch.randn(n, h, device=DEV).bfloat16().requires_grad_(True)
+    weight = (torch.randn(v, h, device=DEV) * 0.02).bfloat16().requires_grad_(True)
+    labels = torch.randint(0, v, (n,), device=DEV)
+    mask = torch.zeros(n, dtype=torch.bool, device=DEV)
+    mask[torch.randperm(n, device=DEV)[:8500]] = True
+    adv = torch.randn(n, device=DEV)
+    cfg = _cfg()
+    with torch.no_grad():
+        lp0, _ = lm_head.fused_lm_head_logprobs(hidden, weight, labels, mask=mask)
+    old = lp0 + 0.05 * torch.randn(n, device=DEV)
+    ref = lp0 + 0.1 * torch.randn(n, device=DEV)
+    loss, stats, lp, ent = grpo_utils.grpo_loss_on_hidden(
+        hidden[None], weight, labels[None], old[None], ref[None], adv[None], mask[None], cfg, token_slabs=8192
+    )
+    loss.backward()
+    torch.cuda.synchronize()
+    lp, ent = lp[0], ent[0]
+    assert (lp - lp0).abs().max().item() <= 1e-5
+    lp_leaf = lp.detach().cpu().requires_grad_(True)
+    loss_o, *_ = o_grpo.grpo_token_loss(
+        lp_leaf[None], old.cpu()[None], ref.cpu()[None], adv.cpu()[None], mask.cpu()[None].float(), cfg
+    )
+    loss_o.backward()
+    assert abs(loss.item() - loss_o.item()) <= 1e-5 + 1e-5 * abs(loss_o.item())
+    assert int(stats["num_response_tokens"].item()) == 8500
+    _check_fused_head(hidden, weight, labels, mask, lp_leaf.grad, lp, ent, hidden.grad, weight.grad, seed=11)
+    # the recomputing form of the same step agrees (different summation order: bf16 rounding of the results)
+    h2 = hidden.detach().clone().requires_grad_(True)
+    w2 = weight.detach().clone().requires_grad_(True)
+    loss2, _, lp2, _ = grpo_utils.grpo_loss_on_hidden(
+        h2[None], w2, labels[None], old[None], ref[None], adv[None], mask[None], cfg, token_slabs=False
+    )
+    loss2.backward()
+    assert (lp2[0] - lp).abs().max().item() <= 1e-5
+    assert _rel(hidden.grad.float(), h2.grad.float()) <= REL and _rel(weight.grad.float(), w2.grad.float()) <= REL
+
+
 def test_c3_llama8b_head_grpo_full_shape():
     """hidden bf16 [32768, 4096], W bf16 [128256, 4096], 70 % response rows: fused lm_head + logprob +
     entropy + GRPO loss, forward and backward to dHidden and dW, through the three differentiable
