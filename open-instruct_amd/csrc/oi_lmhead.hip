@@ -503,31 +503,37 @@ __device__ __forceinline__ void stats_update(AccTile& acc, int j, int wm, int la
     st_t = t;
 }
 
-// A finished tile as a bf16 image [256 tokens][256 vocabulary columns] in the LDS (rows of
+// A finished tile leaves as a bf16 image [256 tokens][256 vocabulary columns] through the LDS (rows of
 // STAGE_STRIDE entries; the two 8-byte halves of every 16-byte piece swapped in rows 8..15 of each
 // 16, which keeps the 8-byte stores of a wave off each other's banks), and from there to global
 // memory in 16-byte pieces of whole 512-byte rows.  Rows at or past rows_valid are written as zeros.
-__device__ __forceinline__ void stage_tile_bf16(const AccTile& acc, uint16_t* stage, int wm, int wn, int lane) {
+// It leaves one column group at a time: group j holds the 64 tokens wn*128 + j*32 + (0..31) of both
+// wn halves with all 256 vocabulary columns (every m-wave contributes its 64), i.e. 64 whole rows of
+// the image, and goes to global memory while the next group's statistics are still being computed
+// (forward per slab at the Llama-3.1-8B shape: 6.32 -> 6.28 ms against the whole image at the end, and
+// fewer live registers).
+__device__ __forceinline__ void stage_group_bf16(const AccTile& acc, uint16_t* stage, int wm, int wn, int lane, int j) {
+    asm volatile("" : "+v"(lane));
+    const int nl = acc_col(wn, j, lane);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int nl = acc_col(wn, j, lane);
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int vl = acc_row(wm, i, q * 4, lane) ^ (((nl >> 3) & 1) << 2);
-                const uint2 pk = make_uint2(oi_pack_bf16x2(acc[i][j][q * 4], acc[i][j][q * 4 + 1]),
-                                            oi_pack_bf16x2(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]));
-                *reinterpret_cast<uint2*>(stage + nl * STAGE_STRIDE + vl) = pk;
-            }
-    }
+        for (int q = 0; q < 4; ++q) {
+            const int vl = acc_row(wm, i, q * 4, lane) ^ (((nl >> 3) & 1) << 2);
+            const uint2 pk = make_uint2(oi_pack_bf16x2(acc[i][j][q * 4], acc[i][j][q * 4 + 1]),
+                                        oi_pack_bf16x2(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]));
+            *reinterpret_cast<uint2*>(stage + nl * STAGE_STRIDE + vl) = pk;
+        }
 }
-__device__ __forceinline__ void copy_staged_tile(const uint16_t* stage, uint16_t* __restrict__ dst, int64_t ld, int tid,
-                                                 int rows_valid) {
-#pragma unroll 4
-    for (int it = 0; it < 16; ++it) {
+__device__ __forceinline__ void copy_staged_group(const uint16_t* stage, uint16_t* __restrict__ dst, int64_t ld, int tid,
+                                                  int rows_valid, int j) {
+    // the lane's addresses are formed here, where they are used, not ahead of the tile's main loop
+    asm volatile("" : "+v"(tid));
+#pragma unroll 1
+    for (int it = 0; it < 4; ++it) {
         const int cidx = tid + it * NTHREADS;
-        const int row = cidx >> 5, ch = cidx & 31;
+        const int r = cidx >> 5, ch = cidx & 31;                 // r: 0..63 within the group
+        const int row = (r >> 5) * 128 + j * 32 + (r & 31);      // row of the image = token of the tile
         oi_u32x4 v = *reinterpret_cast<const oi_u32x4*>(stage + row * STAGE_STRIDE + ch * 8);
         if (row & 8) v = oi_u32x4{v.z, v.w, v.x, v.y};
         if (row >= rows_valid) v = oi_u32x4{0u, 0u, 0u, 0u};
@@ -589,6 +595,7 @@ __device__ __forceinline__ void lmhead_fwd_item(const uint16_t* __restrict__ W, 
         const int64_t m0 = vt * BM;
         gemm_tile(acc, W, hdim, m0, vocab, hidden, hdim, n0, n_tokens, hdim, lds);
         const bool partial_tile = m0 + BM > vocab;
+        const bool keep_tile = CACHE && vt >= fl.cache_tile0 && vt < fl.cache_tile0 + fl.cache_tiles;
         const int wave_row0 = (int)m0 + wm * 64;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -621,17 +628,20 @@ __device__ __forceinline__ void lmhead_fwd_item(const uint16_t* __restrict__ W, 
                     for (int r = 0; r < 16; ++r)
                         if (i * 16 + r == label_reg) acc[i][j][r] = 0.f;
             }
+            if (CACHE && keep_tile) {
+                // the operand ring is free (the product ended with a barrier); the groups use disjoint rows
+                // of the image, so one barrier per group (written -> read out) is all they need
+                __builtin_amdgcn_sched_barrier(0);
+                stage_group_bf16(acc, lds, wm, wn, lane, j);
+                __syncthreads();
+                const int64_t left = n_tokens - n0;
+                copy_staged_group(lds, fl.ecache + n0 * fl.cache_ld + (vt - fl.cache_tile0) * BM, fl.cache_ld, tid,
+                                  (int)(left < BN ? left : BN), j);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        if (CACHE && vt >= fl.cache_tile0 && vt < fl.cache_tile0 + fl.cache_tiles) {
-            // the operand ring is free (the product ended with a barrier); the next tile's first loads
-            // must wait until the image has been read out again
-            stage_tile_bf16(acc, lds, wm, wn, lane);
-            __syncthreads();
-            const int64_t left = n_tokens - n0;
-            copy_staged_tile(lds, fl.ecache + n0 * fl.cache_ld + (vt - fl.cache_tile0) * BM, fl.cache_ld, tid,
-                             (int)(left < BN ? left : BN));
-            __syncthreads();
-        }
+        // the next tile's first loads must wait until the image has been read out again
+        if (CACHE && keep_tile) __syncthreads();
     }
 
     // merge the two lane halves (same token, other rows), then the four m-waves through LDS
