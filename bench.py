@@ -18,7 +18,8 @@ synthetic inputs that already live in HBM.  Workloads are the BASELINE configs:
   c5: DPO at Llama-3.1-70B head shape: hidden [32768, 8192], W [128256, 8192], bwd to dHidden only.
       c5-train-head: the same batch with a trainable head (what the reference's DPO trains), loss and
       both gradients from one no-recompute call (dpo_loss_on_hidden); c5-train-head-recompute: the same
-      through the differentiable calls; c5-one-call: the frozen-head batch through dpo_loss_on_hidden.
+      through the differentiable calls; c5-one-call: the frozen-head batch through dpo_loss_on_hidden;
+      ref-cache: the forward-only pass over that batch that fills the reference-logprob cache of a DPO run.
   pack: pack_sequences + advantage broadcast for 512 prompt / response pairs (about 1.09 M tokens).
 
 `roofline` describes the dominant kernel of the workload, timed with HIP events on the stream it
@@ -195,6 +196,13 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, route="slabs"
     def step():
         hidden.grad = None
         weight.grad = None
+        if dpo and route == "forward":
+            # the pass that fills the reference-logprob cache: no gradient, per-sequence sums of the logprobs
+            with torch.no_grad():
+                with fwd_timer:
+                    lp, _ = oi.fused_lm_head_logprobs(hidden, weight, shifted.view(-1), mask=mask)
+                logps = oi.padding_free_collator.get_batch_logps(lp.view(1, -1), labels, cu)
+            return logps.sum()
         if dpo and route == "slabs" and (train_head or one_call):
             with probe:
                 res = oi.dpo_utils.dpo_loss_on_hidden(
@@ -240,7 +248,9 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, route="slabs"
         "bound": "mfma",
         "timer": fwd_timer,
     }
-    if dpo and (train_head or one_call):
+    if dpo and route == "forward":
+        info["flops_step"] = flops_fwd
+    elif dpo and (train_head or one_call):
         info["flops_step"] = (3.0 if train_head else 2.0) * flops_fwd
         if route == "slabs" and one_call and not train_head:
             info["kernel"] = (
@@ -256,7 +266,7 @@ def make_fused(torch, oi, n_tokens, hdim, vocab, w_std, dpo=False, route="slabs"
             )
             info["alg_per_launch"] = None  # filled in from the number of launches that had rows
             info["timer"] = probe
-    elif dpo:
+    elif dpo and route != "forward":
         # the weight takes no gradient: the forward call also accumulates the weighted sum of weight rows that
         # the backward to hidden needs (per vocabulary chunk: statistics + exponentials, then E_chunk @ W_chunk)
         info["kernel"] = (
@@ -514,7 +524,8 @@ def cpu_baseline(torch, workload):
     workload = {"c3-recompute": "c3", "c3-one-call-recompute": "c3", "c4-recompute": "c4", "c5-one-call": "c5", "c5-train-head": "c5t",
                 "c5-train-head-recompute": "c5t"}.get(workload, workload)
     train_head = workload == "c5t"
-    workload = "c5" if train_head else workload
+    forward_only = workload == "ref-cache"
+    workload = "c5" if train_head or forward_only else workload
     if workload == "c5":
         # one chosen / rejected pair of 2 x 1024 tokens (of the 8 pairs of 2 x 2048), prompts masked out
         from oracle import dpo as o_dpo
@@ -533,15 +544,22 @@ def cpu_baseline(torch, workload):
             weight.grad = None
             # reference order: bf16 lm_head GEMM, fp32 log_softmax + gather of the shifted labels, per-sequence
             # sums, sigmoid DPO loss, backward to the hidden states
-            z = torch.nn.functional.linear(hidden, weight).view(2, per, vocab)
-            per_token = o_lp.calculate_per_token_logps(z, labels)
-            logps = o_red.get_batch_logps_padded(per_token, labels)
+            with torch.set_grad_enabled(not forward_only):
+                z = torch.nn.functional.linear(hidden, weight).view(2, per, vocab)
+                per_token = o_lp.calculate_per_token_logps(z, labels)
+                logps = o_red.get_batch_logps_padded(per_token, labels)
+            if forward_only:
+                return
             losses, _, _ = o_dpo.dpo_loss(logps[:1], logps[1:], ref_c, ref_r, 0.1)
             losses.mean().backward()
 
-        sample = (f"one pair of 2 x {per} tokens (of 8 pairs of 2 x 2048) at full H={hdim}, V={vocab}, W ~ N(0, 0.01); "
-                  f"fwd + bwd to the hidden states{' and the head' if train_head else ''}; bf16 GEMM + fp32 log_softmax + "
-                  "sigmoid DPO loss")
+        if forward_only:
+            sample = (f"one pair of 2 x {per} tokens (of 8 pairs of 2 x 2048) at full H={hdim}, V={vocab}, W ~ N(0, 0.01); "
+                      "forward only, no gradient; bf16 GEMM + fp32 log_softmax + per-sequence sums")
+        else:
+            sample = (f"one pair of 2 x {per} tokens (of 8 pairs of 2 x 2048) at full H={hdim}, V={vocab}, W ~ N(0, 0.01); "
+                      f"fwd + bwd to the hidden states{' and the head' if train_head else ''}; bf16 GEMM + fp32 log_softmax + "
+                      "sigmoid DPO loss")
     elif workload in ("c3", "c4"):
         hdim = 4096
         vocab, n = (100352 if workload == "c4" else 128256), 2048
@@ -662,7 +680,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="c3",
                     choices=["c1", "c2", "c2-two-pass", "c3", "c3-recompute", "c3-one-call-recompute", "c4",
-                             "c4-recompute", "c5", "c5-one-call", "c5-train-head", "c5-train-head-recompute", "pack"])
+                             "c4-recompute", "c5", "c5-one-call", "c5-train-head", "c5-train-head-recompute", "ref-cache",
+                             "pack"])
     ap.add_argument("--slab-tokens", type=int, default=0,
                     help="c3 / c4 / c5-train-head only: slab size of the no-recompute step (0 = the package's default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -720,6 +739,12 @@ def main():
     elif args.workload == "c5":
         step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True)
         name = "c5: fused lm_head+per-sequence logprob sums+sigmoid DPO loss, hidden bf16 [32768,8192], W bf16 [128256,8192], bwd to dHidden only"
+        dtype = "bf16"
+    elif args.workload == "ref-cache":
+        step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True, route="forward")
+        name = ("ref-cache: the forward-only pass that fills the reference-logprob cache of a DPO run at the c5 shape "
+                "(hidden bf16 [32768,8192], W bf16 [128256,8192], 16 sequences): fused lm_head logprobs of the scored "
+                "positions + per-sequence sums, no gradient")
         dtype = "bf16"
     elif args.workload == "c5-one-call":
         step, info = make_fused(torch, oi, 32768, 8192, 128256, 0.01, dpo=True, one_call=True)
@@ -821,7 +846,7 @@ def main():
         roofline["whole_step_tflops"] = info["flops_step"] / (ms_per_step * 1e-3) / 1e12
         roofline["whole_step_frac"] = roofline["whole_step_tflops"] / PEAK_BF16_TFLOPS
         if not args.no_library_gemm:
-            hdim = 8192 if args.workload.startswith("c5") else 4096
+            hdim = 8192 if args.workload.startswith("c5") or args.workload == "ref-cache" else 4096
             vocab = 100352 if args.workload in ("c4", "c4-recompute") else 128256
             roofline["library_bf16_gemm_tflops"] = library_gemm_tflops(torch, 32768, hdim, vocab)
     if "bytes_step" in info:

@@ -159,6 +159,11 @@ def fused_lm_head_logprobs(
         raise ValueError(f"temperature must be positive, got {temperature}")
     if mask is not None and tuple(mask.shape) != tuple(lead):
         raise ValueError(f"mask {tuple(mask.shape)} does not match the rows of hidden {tuple(lead)}")
+    if dhidden_in_forward == "auto":
+        dhidden_in_forward = not compact_backward
+    # without a backward pass to come (torch.no_grad(): scoring passes, the reference-logprob cache) there is
+    # nothing to prepare; inside an autograd Function the grad mode is off, so it is read here
+    dhidden_in_forward = bool(dhidden_in_forward) and torch.is_grad_enabled()
     lp, ent = _FusedLMHead.apply(hid2, weight, lab1, mask, inv_t, return_entropy, compact_backward, dhidden_in_forward)
     return lp.reshape(lead), (ent.reshape(lead) if ent is not None else None)
 

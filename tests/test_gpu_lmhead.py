@@ -183,6 +183,24 @@ def test_d_hidden_in_forward_is_the_default_without_d_weight():
         )
 
 
+def test_no_grad_forward_prepares_nothing_for_a_backward():
+    """Under torch.no_grad() (scoring passes, the reference-logprob cache build: open_instruct/dpo_utils.py:405-520)
+    the forward is the plain one even when ``hidden`` is a tensor that requires a gradient and the weight is
+    frozen: the weighted sum for a backward that never comes would double the matrix work.  Seen through the
+    scratch it would allocate (a [tokens, 65536] bf16 chunk and an fp32 [tokens, hidden] sum)."""
+    hidden, weight, labels = _case(2048, 256, 70000, seed=14)
+    dh, w, lab = hidden.to(DEV).requires_grad_(True), weight.to(DEV), labels.to(DEV)
+    out_grad, _ = lm_head.fused_lm_head_logprobs(dh, w, lab)
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    with torch.no_grad():
+        out, _ = lm_head.fused_lm_head_logprobs(dh, w, lab)
+    torch.cuda.synchronize()
+    assert torch.cuda.max_memory_allocated() - before < 64 << 20  # the chunk alone would be 268 MB
+    assert not out.requires_grad and (out - out_grad.detach()).abs().max().item() <= 1e-5
+
+
 def test_dpo_lm_head_matches_calculate_per_token_logps():
     """open_instruct/test_padding_free_collator.py:366-399 with the fused head."""
     torch.manual_seed(42)
