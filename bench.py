@@ -20,6 +20,7 @@ synthetic inputs that already live in HBM.  Workloads are the BASELINE configs:
       both gradients from one no-recompute call (dpo_loss_on_hidden); c5-train-head-recompute: the same
       through the differentiable calls; c5-one-call: the frozen-head batch through dpo_loss_on_hidden;
       ref-cache: the forward-only pass over that batch that fills the reference-logprob cache of a DPO run.
+  sft: causal-LM cross-entropy (the supervised fine-tuning loss) at the c3 head shape, fwd + bwd, slab-wise.
   pack: pack_sequences + advantage broadcast for 512 prompt / response pairs (about 1.09 M tokens).
 
 `roofline` describes the dominant kernel of the workload, timed with HIP events on the stream it
@@ -465,6 +466,44 @@ def make_c4(torch, oi, hdim=4096, vocab=100352, n_seqs=16, budget=32768, route="
     return step, info
 
 
+def make_sft(torch, oi, batch=8, seq=4096, hdim=4096, vocab=128256):
+    """Supervised fine-tuning loss (open_instruct/finetune.py:818-824) at the Llama-3.1-8B head shape: causal-LM
+    cross-entropy of 8 sequences of 4096 tokens whose prompts (256..2048 tokens) carry ignored labels, forward and
+    backward to the hidden states and the head through fused_linear_cross_entropy(token_slabs=True)."""
+    dev = "cuda:0"
+    torch.manual_seed(0)
+    hidden = torch.randn(batch, seq, hdim, device=dev).bfloat16().requires_grad_(True)
+    weight = (torch.randn(vocab, hdim, device=dev) * 0.02).bfloat16().requires_grad_(True)
+    labels = torch.randint(0, vocab, (batch, seq), device=dev)
+    prompt = torch.randint(256, 2049, (batch,), device=dev)
+    labels[torch.arange(seq, device=dev).unsqueeze(0) < prompt.unsqueeze(1)] = -100
+    n_eff = int((labels[:, 1:] != -100).sum().item())
+    probe = KernelProbe(oi, 2)
+
+    def step():
+        hidden.grad = None
+        weight.grad = None
+        with probe:
+            loss = oi.fused_linear_cross_entropy(hidden, weight, labels, token_slabs=True)
+        loss.backward()
+        return loss
+
+    flops_fwd = 2.0 * n_eff * hdim * vocab
+    info = {
+        "tokens": batch * seq,
+        "rows_multiplied": n_eff,
+        "hdim": hdim,
+        "vocab": vocab,
+        "flops_step": 3.0 * flops_fwd,
+        "kernel": ("gemm_store_kernel<true, true> (d_weight product of a slab of selected tokens, added to the fp32 d_weight; "
+                   "timed launch by launch through the library's event probe)"),
+        "alg_per_launch": None,
+        "bound": "mfma",
+        "timer": probe,
+    }
+    return step, info
+
+
 def _pack_case(n=512, max_q=512, max_r=3584, pad=0, seed=0):
     import random
 
@@ -521,7 +560,7 @@ def cpu_baseline(torch, workload):
     threads = torch.get_num_threads()
     cfg = _cfg()
     torch.manual_seed(0)
-    workload = {"c3-recompute": "c3", "c3-one-call-recompute": "c3", "c4-recompute": "c4", "c5-one-call": "c5", "c5-train-head": "c5t",
+    workload = {"c3-recompute": "c3", "c3-one-call-recompute": "c3", "sft": "sft", "c4-recompute": "c4", "c5-one-call": "c5", "c5-train-head": "c5t",
                 "c5-train-head-recompute": "c5t"}.get(workload, workload)
     train_head = workload == "c5t"
     forward_only = workload == "ref-cache"
@@ -582,6 +621,23 @@ def cpu_baseline(torch, workload):
             loss.backward()
 
         sample = f"{n} of 32768 token rows at full H={hdim}, V={vocab}; fwd+bwd; bf16 GEMM + fp32 log_softmax"
+    elif workload == "sft":
+        hdim, vocab, n = 4096, 128256, 2048
+        hidden = torch.randn(1, n, hdim).bfloat16().requires_grad_(True)
+        weight = (torch.randn(vocab, hdim) * 0.02).bfloat16().requires_grad_(True)
+        labels = torch.randint(0, vocab, (1, n))
+        labels[:, : n // 4] = -100
+
+        def run():
+            hidden.grad = None
+            weight.grad = None
+            # the model forward's order: bf16 lm_head GEMM, fp32 upcast, shifted labels, mean cross-entropy
+            z = torch.nn.functional.linear(hidden, weight).float()
+            shifted = o_lp.shift_labels(labels).reshape(-1)
+            torch.nn.functional.cross_entropy(z.view(-1, vocab), shifted, ignore_index=-100).backward()
+
+        sample = (f"one sequence of {n} tokens (of 8 x 4096) at full H={hdim}, V={vocab}, a quarter of it prompt; fwd+bwd; the "
+                  "causal-LM loss as the reference's model forward computes it")
     elif workload in ("c2", "c2-two-pass"):
         n, vocab = 8192, 128256
         logits = (torch.randn(n, vocab) * 3.0).bfloat16().requires_grad_(True)
@@ -621,7 +677,7 @@ def cpu_baseline(torch, workload):
             o_red.masked_mean(lp, mask) + o_red.masked_mean(ent, mask)
 
         sample = "the full config-1 batch (2048 rows, V=32000, fp32)"
-    scaled = {"c3": 32768, "c4": 32768, "c5": 32768, "c2": 65536, "c2-two-pass": 65536}.get(workload)
+    scaled = {"c3": 32768, "c4": 32768, "c5": 32768, "sft": 32768, "c2": 65536, "c2-two-pass": 65536}.get(workload)
     run()  # warm-up
     times = []
     t_end = time.time() + 20.0
@@ -681,7 +737,7 @@ def main():
     ap.add_argument("--workload", default="c3",
                     choices=["c1", "c2", "c2-two-pass", "c3", "c3-recompute", "c3-one-call-recompute", "c4",
                              "c4-recompute", "c5", "c5-one-call", "c5-train-head", "c5-train-head-recompute", "ref-cache",
-                             "pack"])
+                             "sft", "pack"])
     ap.add_argument("--slab-tokens", type=int, default=0,
                     help="c3 / c4 / c5-train-head only: slab size of the no-recompute step (0 = the package's default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -770,6 +826,11 @@ def main():
     elif args.workload == "c2-two-pass":
         step, info = make_c2(torch, oi, single_pass=False)
         name = "c2: GRPO loss on materialised bf16 logits [64,1024,128256], fwd+bwd, reference order (logits read twice)"
+        dtype = "bf16"
+    elif args.workload == "sft":
+        step, info = make_sft(torch, oi)
+        name = ("sft: causal-LM cross-entropy through the fused head, hidden bf16 [8,4096,4096], W bf16 [128256,4096], "
+                f"prompts ignored, fwd+bwd to dHidden and dW through fused_linear_cross_entropy(token_slabs=True): {slab_note}")
         dtype = "bf16"
     elif args.workload == "pack":
         step, info = make_pack(torch, oi)
