@@ -315,6 +315,26 @@ def concatenated_forward_olmo(
     return chosen, rejected, None
 
 
+def separate_forward_olmo(model, batch: dict, average_log_prob: bool = False, output_router_logits: bool = False):
+    """Chosen and rejected sequences in two forwards of a model with the olmo-core interface;
+    open_instruct/dpo_utils.py:1022-1054.
+
+    As in :func:`concatenated_forward_olmo` the labels go into the model and its
+    :class:`~open_instruct_amd.olmo_core_train_modules.DPOLMHead` returns the per-token logps as
+    ``output.loss``; only one side's activations are alive at a time.  ``output_router_logits`` is accepted
+    and unused, ``aux_loss`` is always None, as in the reference.  (The reference empties the allocator's
+    cache after each side; the fused head leaves no ``[tokens, vocab]`` block behind to give back.)
+    """
+    del output_router_logits
+    sides = []
+    for side in ("chosen", "rejected"):
+        part = process_batch(batch, side)
+        output = model(part["input_ids"], labels=part["labels"])
+        sides.append(_get_batch_logps(output.loss, part["labels"], average_log_prob=average_log_prob))
+        del output, part
+    return sides[0], sides[1], None
+
+
 @dataclasses.dataclass
 class FusedDPOResult:
     """What :func:`dpo_loss_on_hidden` returns.  ``loss`` (``losses.mean()``) carries the graph: its

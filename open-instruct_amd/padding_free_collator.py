@@ -117,3 +117,42 @@ def concatenated_inputs(batch: dict, tag: str = "concatenated_") -> tuple[dict, 
         n_chosen = len(chosen["cu_seq_lens_k"]) - 1
         ret[f"{tag}seq_idx"] = torch.cat([chosen["seq_idx"], rejected["seq_idx"] + n_chosen], dim=-1)
     return ret, len(chosen["cu_seq_lens_k"]) - 1
+
+
+def _cu_seq_lens_of(batch: dict) -> list[torch.Tensor]:
+    """The key-side boundary tensors of a packed batch: ``cu_seq_lens_k`` (GRPO) or the chosen and rejected
+    ones (DPO)."""
+    return [v for k, v in batch.items() if k.endswith("cu_seq_lens_k")]
+
+
+def get_num_tokens(batch: dict) -> int:
+    """Real (non-padding) tokens of a training batch; open_instruct/padding_free_collator.py:232-249.
+
+    Packed: the last boundary of every ``*cu_seq_lens_k``; padded: the sum of every ``*attention_mask``;
+    otherwise the element count of the ``input_ids`` tensors.  Returns a Python number (one host read),
+    as the reference does.
+    """
+    cu = _cu_seq_lens_of(batch)
+    if cu:
+        return sum(c[-1].item() for c in cu)
+    masks = [v for k, v in batch.items() if k.endswith("attention_mask")]
+    if masks:
+        return sum(m.sum().item() for m in masks)
+    return sum(v.numel() for k, v in batch.items() if "input_ids" in k and isinstance(v, torch.Tensor))
+
+
+def get_num_padded_tokens(batch: dict) -> int:
+    """All token positions of a batch, padding included; open_instruct/padding_free_collator.py:252-257."""
+    return sum(v.numel() for k, v in batch.items() if k.endswith("input_ids") and isinstance(v, torch.Tensor))
+
+
+def get_num_sequences(batch: dict) -> torch.Tensor:
+    """Sequences of a batch as a scalar tensor (no host read); open_instruct/padding_free_collator.py:260-273.
+
+    Packed: the strictly increasing steps of every ``*cu_seq_lens_k`` (repeated boundaries are padding);
+    padded: the rows of every ``*input_ids``.
+    """
+    cu = _cu_seq_lens_of(batch)
+    if cu:
+        return sum((c[..., 1:] > c[..., :-1]).sum() for c in cu)
+    return torch.tensor(sum(v.shape[0] for k, v in batch.items() if k.endswith("input_ids")))

@@ -574,6 +574,19 @@ def test_concatenated_forward_olmo_through_dpo_lm_head(packing, average_log_prob
         got = got.float().cpu()
         assert (got - exp).abs().max().item() <= _bf16_tol(exp)
         assert ((got - exp).norm() / exp.norm()).item() <= 2e-2
+    if packing:
+        return
+    # the two-forward variant of the same stack (open_instruct/dpo_utils.py:1022-1054): same sums, same gradients
+    model.zero_grad()
+    chosen2, rejected2, aux2 = dpo_utils.separate_forward_olmo(model, batch, average_log_prob=average_log_prob)
+    assert aux2 is None and chosen2.shape == (pairs,) and rejected2.shape == (pairs,)
+    assert (chosen2 - chosen).abs().max().item() <= 1e-4 and (rejected2 - rejected).abs().max().item() <= 1e-4
+    losses2, _, _ = dpo_utils.dpo_loss(chosen2, rejected2, ref_c.to(DEV), ref_r.to(DEV), beta)
+    losses2.mean().backward()
+    for got, exp in ((model.lm_head.w_out.weight.grad, w.grad), (model.embed.weight.grad, emb.grad)):
+        got = got.float().cpu()
+        assert (got - exp).abs().max().item() <= _bf16_tol(exp)
+        assert ((got - exp).norm() / exp.norm()).item() <= 2e-2
 
 
 @pytest.mark.parametrize("b,t,h,v,axis,want_dw,slabs", [

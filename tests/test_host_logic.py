@@ -281,6 +281,35 @@ def test_doc_lens_from_attention_mask_reference_vectors(golden):
         assert got[: len(runs)] == runs and not any(got[len(runs) :]) and longest == max(runs)
 
 
+def test_batch_counters_reference_vectors(golden):
+    """open_instruct/test_padding_free_collator.py:399-419: sequences of a packed batch are the strictly
+    increasing boundary steps of every *cu_seq_lens_k, of a padded one the rows of every *input_ids; padded
+    token positions are the elements of every *input_ids."""
+    from open_instruct_amd import padding_free_collator as pfc
+
+    vec = golden["batch_counters"]
+    for case in vec["num_sequences"]:
+        batch = {k: torch.tensor(v) for k, v in case.get("batch", {}).items()}
+        batch.update({k: torch.zeros(*shape) for k, shape in case.get("batch_shapes", {}).items()})
+        got = pfc.get_num_sequences(batch)
+        assert isinstance(got, torch.Tensor) and got.ndim == 0, case["name"]
+        assert int(got) == case["expected"], case["name"]
+    for case in vec["num_padded_tokens"]:
+        batch = {k: torch.zeros(*shape) for k, shape in case["batch_shapes"].items()}
+        assert pfc.get_num_padded_tokens(batch) == case["expected"]
+    # repeated boundaries (a packed row padded to a fixed number of sequences) do not count
+    assert int(pfc.get_num_sequences({"cu_seq_lens_k": torch.tensor([0, 3, 7, 7, 7])})) == 2
+    # real tokens (open_instruct/padding_free_collator.py:232-249): the last boundaries of a packed batch, the
+    # attention-mask sums of a padded one, else every input id; non-tensor entries are skipped
+    packed = {"chosen_cu_seq_lens_k": torch.tensor([0, 3, 7]), "rejected_cu_seq_lens_k": torch.tensor([0, 4]),
+              "chosen_input_ids": torch.zeros(1, 9), "rejected_input_ids": torch.zeros(1, 6)}  # fmt: skip
+    assert pfc.get_num_tokens(packed) == 11 and pfc.get_num_padded_tokens(packed) == 15
+    padded = {"chosen_attention_mask": torch.tensor([[1, 1, 0], [1, 0, 0]]), "rejected_attention_mask": torch.tensor([[1, 1, 1]]),
+              "chosen_input_ids": torch.zeros(2, 3), "rejected_input_ids": torch.zeros(1, 3), "index": [4, 5]}  # fmt: skip
+    assert pfc.get_num_tokens(padded) == 6 and pfc.get_num_padded_tokens(padded) == 9
+    assert pfc.get_num_tokens({"input_ids": torch.zeros(2, 7), "note": "x"}) == 14
+
+
 def test_doc_lens_from_cu_seq_lens():
     """open_instruct/olmo_core_utils.py:650-665: differences of the offsets; a padded tail becomes a
     segment of its own so the lengths cover the whole row (the reference holds no vector for it;
