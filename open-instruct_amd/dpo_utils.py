@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import contextlib
 import dataclasses
+import enum
 import pathlib
 from collections.abc import Callable, Iterable
 
@@ -19,6 +20,33 @@ import torch.distributed as dist
 
 from . import _lib, lm_head, model_utils, olmo_core_utils, padding_free_collator
 from .padding_free_collator import get_batch_logps_padded
+
+
+class DPOLossType(str, enum.Enum):
+    """The preference losses of the reference and what each one needs; open_instruct/dpo_utils.py:76-92.
+    A string enum: members compare equal to their names, which is also what :func:`compute_loss` and
+    :func:`fused_loss_olmo` accept in ``args.loss_type``."""
+
+    dpo = "dpo"
+    dpo_norm = "dpo_norm"
+    simpo = "simpo"
+    wpo = "wpo"
+
+    def __str__(self) -> str:
+        return self.value
+
+    @property
+    def is_average_loss(self) -> bool:
+        """Per-sequence logprobs are token means rather than sums."""
+        return self.value in ("simpo", "dpo_norm")
+
+    @property
+    def needs_reference_model(self) -> bool:
+        return self.value in ("dpo", "dpo_norm", "wpo")
+
+    @property
+    def computes_reward_metrics(self) -> bool:
+        return self.value in ("dpo", "dpo_norm")
 
 
 class _SigmoidPairLoss(torch.autograd.Function):

@@ -13,12 +13,24 @@ open_instruct/data_loader.py:1472-1484 in one or two kernel launches each.
 
 from __future__ import annotations
 
+import enum
 from dataclasses import dataclass, field
 
 import torch
 
 from . import _lib, model_utils, olmo_core_utils
 from .rl_utils import masked_mean
+
+
+class GRPOLossType(str, enum.Enum):
+    """The policy-gradient terms of the reference; open_instruct/grpo_utils.py:69-71.  A string enum: members
+    compare equal to their names, which is also what ``config.loss_fn`` may hold."""
+
+    dapo = "dapo"
+    cispo = "cispo"
+
+    def __str__(self) -> str:
+        return self.value
 
 INVALID_LOGPROB = 1.0  # open_instruct/utils.py:83
 

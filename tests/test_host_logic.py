@@ -281,6 +281,28 @@ def test_doc_lens_from_attention_mask_reference_vectors(golden):
         assert got[: len(runs)] == runs and not any(got[len(runs) :]) and longest == max(runs)
 
 
+def test_loss_type_enums():
+    """open_instruct/dpo_utils.py:76-92, open_instruct/grpo_utils.py:69-71: string enums whose members equal
+    their names; which DPO losses average the sequence logprobs, need a reference model, report rewards."""
+    import types
+
+    from open_instruct_amd import dpo_utils, grpo_utils
+
+    T = dpo_utils.DPOLossType
+    assert [m.value for m in T] == ["dpo", "dpo_norm", "simpo", "wpo"]
+    assert T.dpo_norm == "dpo_norm" and T("wpo") is T.wpo and str(T.simpo) == "simpo"
+    table = {"dpo": (False, True, True), "dpo_norm": (True, True, True), "simpo": (True, False, False), "wpo": (False, True, False)}
+    for name, (avg, needs_ref, rewards) in table.items():
+        assert (T(name).is_average_loss, T(name).needs_reference_model, T(name).computes_reward_metrics) == (avg, needs_ref, rewards)
+    G = grpo_utils.GRPOLossType
+    assert [m.value for m in G] == ["dapo", "cispo"] and G.cispo == "cispo"
+    # a config may hold the member or its name
+    for loss_fn in (G.dapo, "dapo"):
+        assert grpo_utils._loss_fn_tag(types.SimpleNamespace(loss_fn=loss_fn)) == grpo_utils._loss_fn_tag(types.SimpleNamespace(loss_fn="dapo"))
+    with pytest.raises(ValueError):
+        grpo_utils._loss_fn_tag(types.SimpleNamespace(loss_fn="ppo"))
+
+
 def test_batch_counters_reference_vectors(golden):
     """open_instruct/test_padding_free_collator.py:399-419: sequences of a packed batch are the strictly
     increasing boundary steps of every *cu_seq_lens_k, of a padded one the rows of every *input_ids; padded
